@@ -1,0 +1,127 @@
+// Host-side error plumbing and device helpers shared by every kernel file.
+// gfx950 only: 64-lane wavefronts, DPP lane exchange, hardware OCP-FP8 and
+// BF16 pack conversions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace deepep {
+
+// ---------------------------------------------------------------------
+// Host errors.  Message format follows the reference's EPException
+// (csrc/kernels/exception.cuh:12-22): "Failed: <kind> error <file>:<line> '<what>'".
+// ---------------------------------------------------------------------
+void set_error(const char* kind, const char* file, int line, const char* what);
+void clear_error();
+
+#define EP_HOST_ASSERT(cond)                                                      \
+    do {                                                                          \
+        if (!(cond)) {                                                            \
+            ::deepep::set_error("Assertion", __FILE_NAME__, __LINE__, #cond);     \
+            return 1;                                                             \
+        }                                                                         \
+    } while (0)
+
+#define EP_HIP_CHECK(cmd)                                                                   \
+    do {                                                                                    \
+        hipError_t e_ = (cmd);                                                              \
+        if (e_ != hipSuccess) {                                                             \
+            ::deepep::set_error("HIP", __FILE_NAME__, __LINE__, hipGetErrorString(e_));     \
+            return 2;                                                                       \
+        }                                                                                   \
+    } while (0)
+
+#define EP_LAUNCH_CHECK() EP_HIP_CHECK(hipGetLastError())
+
+// Row formats; values are part of the C ABI.
+enum RowFormat : int { kRowBF16 = 0, kRowFP8 = 1, kRowFP8Pow2 = 2, kRowFP8UE8M0 = 3 };
+
+constexpr int kWave = 64;
+constexpr int kGroup = 128;        // channels per FP8 scale group
+constexpr int kRowTailBytes = 16;  // {src_token, topk_slot, src_rank, 0}
+
+__host__ __device__ inline int64_t align16(int64_t v) { return (v + 15) & ~int64_t(15); }
+
+__host__ __device__ inline int64_t row_data_bytes(int hidden, int fmt) {
+    return fmt == kRowBF16 ? int64_t(hidden) * 2 : int64_t(hidden);
+}
+__host__ __device__ inline int64_t row_scale_bytes(int hidden, int fmt) {
+    if (fmt == kRowBF16) return 0;
+    const int g = hidden / kGroup;
+    return fmt == kRowFP8UE8M0 ? g : int64_t(g) * 4;
+}
+__host__ __device__ inline int64_t row_stride_bytes(int hidden, int fmt) {
+    return align16(row_data_bytes(hidden, fmt)) + align16(row_scale_bytes(hidden, fmt)) + kRowTailBytes;
+}
+
+// ---------------------------------------------------------------------
+// Device helpers
+// ---------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
+// Wave index inside the workgroup as a scalar, so everything derived from it
+// stays in SGPRs and row addresses become scalar loads.
+__device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6); }
+
+__device__ __forceinline__ uint64_t lanes_below(int lane) { return (uint64_t(1) << lane) - 1; }
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+__device__ __forceinline__ float bf16_lo(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+
+// float32 -> bf16 bits, round to nearest even (NaN kept quiet).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+// max over the 8 lanes that share one 128-channel group (lanes 8i..8i+7):
+// two quad permutes and a half-row mirror, all DPP — no LDS traffic.
+__device__ __forceinline__ float max_over_8_lanes(float v) {
+    int t;
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
+    v = fmaxf(v, __int_as_float(t));
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false);   // quad_perm [2,3,0,1]
+    v = fmaxf(v, __int_as_float(t));
+    t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false);  // row_half_mirror
+    v = fmaxf(v, __int_as_float(t));
+    return v;
+}
+
+// Inclusive sum over the wave (lane i gets sum of lanes 0..i).
+__device__ __forceinline__ int wave_inclusive_sum(int v) {
+    const int lane = lane_id();
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        int o = __shfl_up(v, d, kWave);
+        if (lane >= d) v += o;
+    }
+    return v;
+}
+
+__device__ __forceinline__ int wave_sum(int v) {
+#pragma unroll
+    for (int d = kWave / 2; d >= 1; d >>= 1) v += __shfl_xor(v, d, kWave);
+    return v;
+}
+
+// 32-bit integer mixer used by the seeded synthesiser (lowbias32 constants).
+__host__ __device__ inline uint32_t mix32(uint32_t x) {
+    x ^= x >> 16;
+    x *= 0x7feb352du;
+    x ^= x >> 15;
+    x *= 0x846ca68bu;
+    x ^= x >> 16;
+    return x;
+}
+
+}  // namespace deepep

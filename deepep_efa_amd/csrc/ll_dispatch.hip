@@ -1,0 +1,468 @@
+// Low-latency dispatch: route ranking, fused quantise + pack (send side) and
+// segment compaction (receive side).
+//
+// Data layout in HBM (row stride S = row_stride_bytes(H, format)):
+//   recv_staging  [E_l][R][M] rows — slot j of segment (e_l, s) is the j-th
+//                 row rank s sent to local expert e_l, in ascending (t,k)
+//                 order of the sender.
+//   recv_count    [E_l][R] int32 — rows present in each segment.
+//   send_slots    [E][M] rows — this rank's rows for remote experts.
+// A staged row is [data | pad16][scales | pad16][src_token, k, src_rank, 0].
+//
+// Work is cut per wavefront, never per thread block: one wave owns one 1 KiB
+// piece of one row, so a 64-lane 16-byte access is one contiguous KiB and no
+// LDS or barrier is needed on the copy paths.
+#include "common.hpp"
+#include "quant.hpp"
+#include "segments.hpp"
+#include "../../include/deepep_hip.h"
+
+namespace deepep {
+
+constexpr int kRouteChunk = 1024;  // (token,k) entries ranked by one workgroup
+constexpr int kRouteWaves = kRouteChunk / kWave;
+
+__host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
+
+struct RouteScratch {
+    int32_t* pair_rank;   // [n] rank of the pair inside its chunk, -1 = no selection
+    int32_t* chunk_base;  // [C][E] pairs of expert e in earlier chunks
+    int num_chunks;
+    int64_t bytes;
+};
+
+static RouteScratch carve_route_scratch(void* base, int num_tokens, int num_topk, int num_experts) {
+    RouteScratch s;
+    const int64_t n = int64_t(num_tokens) * num_topk;
+    s.num_chunks = int((n + kRouteChunk - 1) / kRouteChunk);
+    if (s.num_chunks < 1) s.num_chunks = 1;
+    const int64_t rank_bytes = align256(n * 4 + 4);
+    const int64_t base_bytes = align256(int64_t(s.num_chunks) * num_experts * 4);
+    s.pair_rank = reinterpret_cast<int32_t*>(base);
+    s.chunk_base = reinterpret_cast<int32_t*>(reinterpret_cast<uint8_t*>(base) + rank_bytes);
+    s.bytes = rank_bytes + base_bytes;
+    return s;
+}
+
+// Writes the per-expert totals where the receivers look for them.
+__device__ __forceinline__ void emit_expert_count(int e, int total, int num_experts, int num_ranks, int rank,
+                                                  int src_rank, int max_tokens, int32_t* recv_count,
+                                                  int32_t* send_count) {
+    const int cnt = total < max_tokens ? total : max_tokens;
+    const int experts_per_rank = num_experts / num_ranks;
+    if (send_count != nullptr) send_count[e] = cnt;
+    if (e / experts_per_rank == rank) recv_count[(e % experts_per_rank) * num_ranks + src_rank] = cnt;
+}
+
+// ---------------------------------------------------------------------
+// Route ranking.  Entry i = t*K + k.  pair_rank[i] = number of entries i' < i
+// of the same chunk naming the same expert; chunk totals go to chunk_base for
+// the cross-chunk scan.  In-wave ranks come from ballots over the 64 lanes
+// (one ballot per distinct expert present in the wave), cross-wave offsets
+// from a 16 x E table in LDS.  Deterministic: no atomics anywhere.
+// Reference semantics: the serial (token,k) scan of
+// csrc/kernels/efa_kernels.cu:617-637 and coop_dispatch_send.cuh's token_offset.
+// ---------------------------------------------------------------------
+template <bool kSingleChunk>
+__global__ __launch_bounds__(kRouteChunk) void ll_route_rank_kernel(
+    const int64_t* __restrict__ topk_idx, int n, int num_experts, int num_ranks, int rank,
+    const int32_t* __restrict__ src_ranks, int max_tokens, int64_t scratch_stride,
+    uint8_t* __restrict__ scratch_base, int32_t* __restrict__ recv_count, int32_t* __restrict__ send_count) {
+    extern __shared__ int32_t wave_hist[];  // [kRouteWaves][E]
+    const int b = blockIdx.y, c = blockIdx.x;
+    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
+    const int num_chunks = gridDim.x;
+
+    uint8_t* my_scratch = scratch_base + int64_t(b) * scratch_stride;
+    int32_t* pair_rank = reinterpret_cast<int32_t*>(my_scratch);
+    int32_t* chunk_base = reinterpret_cast<int32_t*>(my_scratch + align256(int64_t(n) * 4 + 4));
+
+    const int i = c * kRouteChunk + tid;
+    int e = -1;
+    if (i < n) {
+        const int64_t v = topk_idx[int64_t(b) * n + i];
+        if (v >= 0 && v < num_experts) e = int(v);
+    }
+    for (int j = tid; j < kRouteWaves * num_experts; j += kRouteChunk) wave_hist[j] = 0;
+
+    uint64_t pending = __ballot(e >= 0);
+    int my_rank = 0, my_count = 0;
+    while (pending != 0) {
+        const int leader = __builtin_ctzll(pending);
+        const int e0 = __builtin_amdgcn_readlane(e, leader);
+        const uint64_t same = __ballot(e == e0);
+        if (e == e0) {
+            my_rank = __popcll(same & lanes_below(lane));
+            my_count = __popcll(same);
+        }
+        pending &= ~same;
+    }
+    __syncthreads();
+    if (e >= 0 && my_rank == 0) wave_hist[w * num_experts + e] = my_count;
+    __syncthreads();
+    for (int x = tid; x < num_experts; x += kRouteChunk) {
+        int run = 0;
+#pragma unroll
+        for (int w2 = 0; w2 < kRouteWaves; ++w2) {
+            const int cnt = wave_hist[w2 * num_experts + x];
+            wave_hist[w2 * num_experts + x] = run;
+            run += cnt;
+        }
+        if constexpr (kSingleChunk) {
+            chunk_base[x] = 0;
+            const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
+            emit_expert_count(x, run, num_experts, num_ranks, rank, src_rank, max_tokens, recv_count,
+                              send_count);
+        } else {
+            chunk_base[int64_t(c) * num_experts + x] = run;
+        }
+    }
+    __syncthreads();
+    if (i < n) pair_rank[i] = e >= 0 ? wave_hist[w * num_experts + e] + my_rank : -1;
+    (void)num_chunks;
+}
+
+// Cross-chunk exclusive scan per expert (only launched when T*K > kRouteChunk).
+__global__ __launch_bounds__(256) void ll_route_scan_kernel(int n, int num_experts, int num_ranks, int rank,
+                                                            const int32_t* __restrict__ src_ranks,
+                                                            int max_tokens, int num_chunks,
+                                                            int64_t scratch_stride,
+                                                            uint8_t* __restrict__ scratch_base,
+                                                            int32_t* __restrict__ recv_count,
+                                                            int32_t* __restrict__ send_count) {
+    const int b = blockIdx.y;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= num_experts) return;
+    uint8_t* my_scratch = scratch_base + int64_t(b) * scratch_stride;
+    int32_t* chunk_base = reinterpret_cast<int32_t*>(my_scratch + align256(int64_t(n) * 4 + 4));
+    int run = 0;
+    for (int c = 0; c < num_chunks; ++c) {
+        const int cnt = chunk_base[int64_t(c) * num_experts + e];
+        chunk_base[int64_t(c) * num_experts + e] = run;
+        run += cnt;
+    }
+    const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
+    emit_expert_count(e, run, num_experts, num_ranks, rank, src_rank, max_tokens, recv_count, send_count);
+}
+
+// ---------------------------------------------------------------------
+// Fused quantise + pack.  One wave = one (source, token, 1 KiB output piece).
+// FP8 formats: the piece is 8 scale groups (1024 channels, 2 KiB of bf16 in);
+// each 8-lane cluster owns a group, each lane 16 channels.  The quantised
+// 16 bytes stay in registers and are stored once per selection — the row is
+// read and quantised once however many experts it goes to
+// (reference idea: csrc/kernels/coop_dispatch_send.cuh:572-607).
+// ---------------------------------------------------------------------
+template <int kFmt>
+__global__ __launch_bounds__(256) void ll_send_kernel(
+    const uint8_t* __restrict__ x, const int64_t* __restrict__ topk_idx,
+    const int32_t* __restrict__ src_ranks, int num_src, int num_tokens, int hidden, int num_topk,
+    int num_experts, int num_ranks, int rank, int max_tokens, int pieces_per_row,
+    int64_t scratch_stride, const uint8_t* __restrict__ scratch_base,
+    uint8_t* __restrict__ recv_staging, uint8_t* __restrict__ send_slots, int32_t* __restrict__ pair_slot) {
+    const int lane = lane_id();
+    const int64_t item = int64_t(blockIdx.x) * (blockDim.x / kWave) + wave_in_block();
+    const int64_t num_items = int64_t(num_src) * num_tokens * pieces_per_row;
+    if (item >= num_items) return;
+    const int piece = int(item % pieces_per_row);
+    const int64_t row_id = item / pieces_per_row;  // b * T + t
+    const int b = int(row_id / num_tokens);
+    const int t = int(row_id - int64_t(b) * num_tokens);
+    const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
+    const int experts_per_rank = num_experts / num_ranks;
+
+    const int64_t data_bytes = row_data_bytes(hidden, kFmt);
+    const int64_t data_pad = align16(data_bytes);
+    const int64_t scale_pad = align16(row_scale_bytes(hidden, kFmt));
+    const int64_t stride = data_pad + scale_pad + kRowTailBytes;
+
+    // ---- load + quantise this wave's piece ------------------------------
+    u32x4 payload = {0u, 0u, 0u, 0u};
+    uint32_t scale_bits = 0;
+    bool lane_live;
+    int group = 0;
+    if constexpr (kFmt == kRowBF16) {
+        const int64_t off = int64_t(piece) * 1024 + lane * 16;
+        lane_live = off < data_bytes;
+        if (lane_live) payload = *reinterpret_cast<const u32x4*>(x + row_id * data_bytes + off);
+    } else {
+        group = piece * 8 + (lane >> 3);
+        lane_live = group < hidden / kGroup;
+        u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
+        if (lane_live) {
+            const uint8_t* src = x + (row_id * hidden + int64_t(group) * kGroup + (lane & 7) * 16) * 2;
+            lo = *reinterpret_cast<const u32x4*>(src);
+            hi = *reinterpret_cast<const u32x4*>(src + 16);
+        }
+        payload = quantise_16<kFmt>(lo, hi, scale_bits);
+    }
+
+    // ---- one store per selection ----------------------------------------
+    const int n = num_tokens * num_topk;
+    const int32_t* pair_rank = reinterpret_cast<const int32_t*>(scratch_base + int64_t(b) * scratch_stride);
+    const int32_t* chunk_base =
+        reinterpret_cast<const int32_t*>(scratch_base + int64_t(b) * scratch_stride + align256(int64_t(n) * 4 + 4));
+    const int64_t entry0 = int64_t(t) * num_topk;
+#pragma unroll 8
+    for (int k = 0; k < num_topk; ++k) {
+        const int in_chunk = pair_rank[entry0 + k];
+        int slot = -1;
+        uint8_t* row = nullptr;
+        if (in_chunk >= 0) {
+            const int e = int(topk_idx[int64_t(b) * n + entry0 + k]);
+            slot = in_chunk + chunk_base[((entry0 + k) / kRouteChunk) * num_experts + e];
+            if (slot >= max_tokens) {
+                slot = -1;
+            } else {
+                const int dst_rank = e / experts_per_rank;
+                const int local = e - dst_rank * experts_per_rank;
+                if (dst_rank == rank)
+                    row = recv_staging + ((int64_t(local) * num_ranks + src_rank) * max_tokens + slot) * stride;
+                else if (send_slots != nullptr)
+                    row = send_slots + (int64_t(e) * max_tokens + slot) * stride;
+            }
+        }
+        if (pair_slot != nullptr && piece == 0 && lane == 0) pair_slot[entry0 + k] = slot;
+        if (row == nullptr) continue;
+        if (lane_live) *reinterpret_cast<u32x4*>(row + int64_t(piece) * 1024 + lane * 16) = payload;
+        if constexpr (kFmt == kRowFP8 || kFmt == kRowFP8Pow2) {
+            if (lane_live && (lane & 7) == 0)
+                *reinterpret_cast<uint32_t*>(row + data_pad + int64_t(group) * 4) = scale_bits;
+        } else if constexpr (kFmt == kRowFP8UE8M0) {
+            if (lane_live && (lane & 7) == 0) row[data_pad + group] = uint8_t(scale_bits >> 23);
+        }
+        if (piece == 0 && lane == 0) {
+            u32x4 tail = {uint32_t(t), uint32_t(k), uint32_t(src_rank), 0u};
+            *reinterpret_cast<u32x4*>(row + data_pad + scale_pad) = tail;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------
+// Receive side.  Every workgroup rebuilds the segment prefix from the E
+// counts (a few hundred ints) in LDS, then its waves walk the flat row index
+// space: row -> (segment, j) by binary search, one wave per row.
+// Slot order is fixed by the staging order, not by atomics
+// (reference: csrc/kernels/efa_kernels.cu:1017-1052 for the ranges,
+// :1059-1213 for the deterministic scatter).
+// ---------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ll_recv_kernel(
+    const uint8_t* __restrict__ recv_staging, const int32_t* __restrict__ recv_count, int hidden,
+    int num_local_experts, int num_ranks, int max_tokens, int fmt, uint8_t* __restrict__ packed_x,
+    uint8_t* __restrict__ packed_scales, int32_t* __restrict__ src_info, int64_t* __restrict__ layout_range,
+    int32_t* __restrict__ packed_count, int32_t* __restrict__ stats) {
+    extern __shared__ int32_t flat[];  // [num_segments + 1]
+    __shared__ int32_t wave_totals[4];
+    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
+    const int num_segments = num_local_experts * num_ranks;
+
+    for (int s = tid; s < num_segments; s += 256) {
+        int c = recv_count[s];
+        c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+        flat[s] = c;
+    }
+    __syncthreads();
+    block_exclusive_scan_256(flat, num_segments, wave_totals);
+    const int total_rows = flat[num_segments];
+
+    if (blockIdx.x == 0) {
+        for (int s = tid; s < num_segments; s += 256) {
+            const int le = s / num_ranks;
+            const int64_t cnt = flat[s + 1] - flat[s];
+            const int64_t begin = flat[s] - flat[le * num_ranks];
+            layout_range[s] = cnt > 0 ? ((begin << 32) | cnt) : 0;
+        }
+        for (int le = tid; le < num_local_experts; le += 256) {
+            const int c = flat[(le + 1) * num_ranks] - flat[le * num_ranks];
+            packed_count[le] = c;
+            if (stats != nullptr) stats[le] += c;
+        }
+    }
+
+    const int64_t data_bytes = row_data_bytes(hidden, fmt);
+    const int64_t data_pad = align16(data_bytes);
+    const int64_t scale_bytes = row_scale_bytes(hidden, fmt);
+    const int64_t stride = data_pad + align16(scale_bytes) + kRowTailBytes;
+    const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
+    const int waves_total = gridDim.x * 4;
+
+    for (int row = blockIdx.x * 4 + w; row < total_rows; row += waves_total) {
+        const int seg = __builtin_amdgcn_readfirstlane(find_segment(flat, num_segments, row));
+        const int j = row - __builtin_amdgcn_readfirstlane(flat[seg]);
+        const int le = seg / num_ranks;
+        const int64_t slot = int64_t(row) - __builtin_amdgcn_readfirstlane(flat[le * num_ranks]);
+        const uint8_t* src = recv_staging + (int64_t(seg) * max_tokens + j) * stride;
+        const int64_t out_row = int64_t(le) * slots_per_expert + slot;
+        wave_copy_vec16(src, packed_x + out_row * data_bytes, int(data_bytes / 16), lane);
+        if (packed_scales != nullptr && scale_bytes > 0) {
+            const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src + data_pad);
+            uint32_t* d32 = reinterpret_cast<uint32_t*>(packed_scales + out_row * scale_bytes);
+            for (int v = lane; v < int(scale_bytes / 4); v += kWave) d32[v] = s32[v];
+        }
+        if (lane == 0)
+            src_info[out_row] = *reinterpret_cast<const int32_t*>(src + data_pad + align16(scale_bytes));
+    }
+}
+
+// ---------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------
+static int check_ll_shape(int num_tokens, int hidden, int num_topk, int num_experts, int num_ranks, int rank,
+                          int max_tokens, int row_format) {
+    EP_HOST_ASSERT(num_tokens >= 0 && hidden > 0 && num_topk > 0);
+    EP_HOST_ASSERT(hidden % 128 == 0);
+    EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
+    EP_HOST_ASSERT(rank >= 0 && rank < num_ranks);
+    EP_HOST_ASSERT(max_tokens > 0 && num_tokens <= max_tokens);
+    EP_HOST_ASSERT(row_format >= kRowBF16 && row_format <= kRowFP8UE8M0);
+    EP_HOST_ASSERT(row_format != kRowFP8UE8M0 || (hidden / 128) % 4 == 0);
+    EP_HOST_ASSERT(int64_t(num_tokens) * num_topk < (int64_t(1) << 30));
+    EP_HOST_ASSERT(num_experts <= 4096);
+    return 0;
+}
+
+static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_t* src_ranks, int num_src,
+                            int num_tokens, int hidden, int num_topk, int num_experts, int num_ranks, int rank,
+                            int max_tokens, int row_format, void* recv_staging, int32_t* recv_count,
+                            void* send_slots, int32_t* send_count, int32_t* pair_slot, void* workspace,
+                            size_t workspace_bytes, hipStream_t stream) {
+    const RouteScratch rs = carve_route_scratch(workspace, num_tokens, num_topk, num_experts);
+    EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(rs.bytes) * size_t(num_src));
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
+    const int n = num_tokens * num_topk;
+    uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
+    const size_t lds = size_t(kRouteWaves) * num_experts * sizeof(int32_t);
+    EP_HOST_ASSERT(lds <= 64 * 1024);
+
+    // Route.  Counts must be published even for an empty batch of tokens.
+    dim3 rgrid(rs.num_chunks, num_src);
+    if (rs.num_chunks == 1) {
+        ll_route_rank_kernel<true><<<rgrid, kRouteChunk, lds, stream>>>(
+            topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count,
+            send_count);
+        EP_LAUNCH_CHECK();
+    } else {
+        ll_route_rank_kernel<false><<<rgrid, kRouteChunk, lds, stream>>>(
+            topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count,
+            send_count);
+        EP_LAUNCH_CHECK();
+        dim3 sgrid((num_experts + 255) / 256, num_src);
+        ll_route_scan_kernel<<<sgrid, 256, 0, stream>>>(n, num_experts, num_ranks, rank, src_ranks, max_tokens,
+                                                        rs.num_chunks, rs.bytes, ws, recv_count, send_count);
+        EP_LAUNCH_CHECK();
+    }
+    if (n == 0) return 0;
+
+    const int pieces = row_format == kRowBF16 ? (hidden * 2 + 1023) / 1024 : (hidden / kGroup + 7) / 8;
+    const int64_t items = int64_t(num_src) * num_tokens * pieces;
+    const int64_t blocks = (items + 3) / 4;
+    EP_HOST_ASSERT(blocks < (int64_t(1) << 31));
+    const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
+    uint8_t* stg = reinterpret_cast<uint8_t*>(recv_staging);
+    uint8_t* snd = reinterpret_cast<uint8_t*>(send_slots);
+#define DEEPEP_LAUNCH_SEND(FMT)                                                                              \
+    ll_send_kernel<FMT><<<dim3(unsigned(blocks)), 256, 0, stream>>>(                                         \
+        xb, topk_idx, src_ranks, num_src, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,        \
+        max_tokens, pieces, rs.bytes, ws, stg, snd, pair_slot)
+    switch (row_format) {
+        case kRowBF16: DEEPEP_LAUNCH_SEND(kRowBF16); break;
+        case kRowFP8: DEEPEP_LAUNCH_SEND(kRowFP8); break;
+        case kRowFP8Pow2: DEEPEP_LAUNCH_SEND(kRowFP8Pow2); break;
+        default: DEEPEP_LAUNCH_SEND(kRowFP8UE8M0); break;
+    }
+#undef DEEPEP_LAUNCH_SEND
+    EP_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace deepep
+
+using namespace deepep;
+
+extern "C" {
+
+size_t deepep_ll_row_data_bytes(int hidden, int row_format) { return size_t(row_data_bytes(hidden, row_format)); }
+size_t deepep_ll_row_scale_bytes(int hidden, int row_format) { return size_t(row_scale_bytes(hidden, row_format)); }
+size_t deepep_ll_row_stride(int hidden, int row_format) { return size_t(row_stride_bytes(hidden, row_format)); }
+
+size_t deepep_ll_dispatch_workspace_bytes(int num_tokens, int num_topk, int num_experts) {
+    return size_t(carve_route_scratch(nullptr, num_tokens, num_topk, num_experts).bytes);
+}
+
+int deepep_ll_dispatch_send(const void* x, const int64_t* topk_idx, int num_tokens, int hidden, int num_topk,
+                            int num_experts, int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                            int row_format, void* recv_staging, int32_t* recv_count, void* send_slots,
+                            int32_t* send_count, int32_t* pair_slot, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+    clear_error();
+    if (int rc = check_ll_shape(num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                                num_max_dispatch_tokens_per_rank, row_format))
+        return rc;
+    EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
+    EP_HOST_ASSERT(recv_staging != nullptr && recv_count != nullptr);
+    EP_HOST_ASSERT(send_count != nullptr && pair_slot != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_staging) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(send_slots) & 15) == 0);
+    return launch_send_side(x, topk_idx, nullptr, 1, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                            num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count, send_slots,
+                            send_count, pair_slot, workspace, workspace_bytes,
+                            reinterpret_cast<hipStream_t>(stream));
+}
+
+int deepep_loopback_dispatch_from_peers(const void* x, const int64_t* topk_idx, const int32_t* src_ranks,
+                                        int num_src, int num_tokens, int hidden, int num_topk, int num_experts,
+                                        int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                                        int row_format, void* recv_staging, int32_t* recv_count, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
+    clear_error();
+    if (int rc = check_ll_shape(num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                                num_max_dispatch_tokens_per_rank, row_format))
+        return rc;
+    EP_HOST_ASSERT(num_src >= 0 && num_src <= 65535);
+    if (num_src == 0) return 0;
+    EP_HOST_ASSERT(src_ranks != nullptr && recv_staging != nullptr && recv_count != nullptr);
+    EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_staging) & 15) == 0);
+    return launch_send_side(x, topk_idx, src_ranks, num_src, num_tokens, hidden, num_topk, num_experts, num_ranks,
+                            rank, num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count, nullptr,
+                            nullptr, nullptr, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
+                            int num_ranks, int num_max_dispatch_tokens_per_rank, int row_format,
+                            void* packed_recv_x, void* packed_recv_scales, int32_t* packed_recv_src_info,
+                            int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
+                            int32_t* cumulative_local_expert_recv_stats, void* stream) {
+    clear_error();
+    EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
+    EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
+    EP_HOST_ASSERT(num_max_dispatch_tokens_per_rank > 0);
+    EP_HOST_ASSERT(row_format >= kRowBF16 && row_format <= kRowFP8UE8M0);
+    EP_HOST_ASSERT(row_format != kRowFP8UE8M0 || (hidden / 128) % 4 == 0);
+    EP_HOST_ASSERT(num_experts <= 1024);
+    EP_HOST_ASSERT(recv_staging != nullptr && recv_count != nullptr && packed_recv_x != nullptr);
+    EP_HOST_ASSERT(row_format == kRowBF16 || packed_recv_scales != nullptr);
+    EP_HOST_ASSERT(packed_recv_src_info != nullptr && packed_recv_layout_range != nullptr &&
+                   packed_recv_count != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_staging) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_scales) & 3) == 0);
+    const int num_local_experts = num_experts / num_ranks;
+    const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
+    EP_HOST_ASSERT(max_rows < (int64_t(1) << 31));
+    int64_t blocks = (max_rows + 3) / 4;
+    const int64_t cap = max_rows > (int64_t(1) << 18) ? 4096 : 512;
+    if (blocks > cap) blocks = cap;
+    const size_t lds = size_t(num_experts + 1) * sizeof(int32_t);
+    ll_recv_kernel<<<dim3(unsigned(blocks)), 256, lds, reinterpret_cast<hipStream_t>(stream)>>>(
+        reinterpret_cast<const uint8_t*>(recv_staging), recv_count, hidden, num_local_experts, num_ranks,
+        num_max_dispatch_tokens_per_rank, row_format, reinterpret_cast<uint8_t*>(packed_recv_x),
+        reinterpret_cast<uint8_t*>(packed_recv_scales), packed_recv_src_info, packed_recv_layout_range,
+        packed_recv_count, cumulative_local_expert_recv_stats);
+    EP_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,122 @@
+"""Device buffers and C-ABI calls of the low-latency path for one rank.
+
+``LowLatencyState`` plays the part of the reference's ``_ll_get_cache``
+(deep_ep/buffer.py:1623-1813): every tensor the path needs is allocated once
+per shape and reused by later calls, so a dispatch/combine pair launches
+kernels and nothing else.  Nothing is ever zero-filled per call (the
+reference clears ~240 MB per dispatch, deep_ep/buffer.py:2370-2378); rows at
+or beyond ``packed_recv_count`` are simply not defined.
+"""
+from dataclasses import dataclass
+
+import torch
+
+from . import _capi
+
+ROW_BF16, ROW_FP8, ROW_FP8_POW2, ROW_FP8_UE8M0 = 0, 1, 2, 3
+
+
+def row_format(use_fp8: bool, round_scale: bool, use_ue8m0: bool) -> int:
+    if not use_fp8:
+        return ROW_BF16
+    if use_ue8m0:
+        assert round_scale, "use_ue8m0 requires round_scale"
+        return ROW_FP8_UE8M0
+    return ROW_FP8_POW2 if round_scale else ROW_FP8
+
+
+def current_stream_ptr():
+    return torch.cuda.current_stream().cuda_stream
+
+
+@dataclass(frozen=True)
+class LLShape:
+    num_ranks: int
+    rank: int
+    num_experts: int
+    max_tokens: int  # num_max_dispatch_tokens_per_rank
+    hidden: int
+    num_topk: int
+    fmt: int
+
+    @property
+    def num_local_experts(self) -> int:
+        return self.num_experts // self.num_ranks
+
+    @property
+    def slots_per_expert(self) -> int:
+        return self.max_tokens * self.num_ranks
+
+
+class LowLatencyState:
+    """All device memory of one rank's low-latency dispatch + combine for one shape."""
+
+    def __init__(self, shape: LLShape, device="cuda", keep_remote_rows: bool = True):
+        lib = _capi.load()
+        self.lib = lib
+        self.shape = s = shape
+        assert s.num_experts % s.num_ranks == 0 and 0 <= s.rank < s.num_ranks
+        assert s.hidden % 128 == 0
+        self.stride = lib.deepep_ll_row_stride(s.hidden, s.fmt)
+        self.data_bytes = lib.deepep_ll_row_data_bytes(s.hidden, s.fmt)
+        self.scale_bytes = lib.deepep_ll_row_scale_bytes(s.hidden, s.fmt)
+        el, r, m, e, h = s.num_local_experts, s.num_ranks, s.max_tokens, s.num_experts, s.hidden
+        u8 = dict(dtype=torch.uint8, device=device)
+        i32 = dict(dtype=torch.int32, device=device)
+        # dispatch
+        self.recv_staging = torch.empty(el * r * m * self.stride, **u8)
+        self.recv_count = torch.zeros(el * r, **i32)
+        self.send_slots = torch.empty(e * m * self.stride, **u8) if keep_remote_rows else None
+        self.send_count = torch.zeros(e, **i32)
+        self.pair_slot = torch.full((m, s.num_topk), -1, **i32)
+        self.workspace = torch.empty(max(256, lib.deepep_ll_dispatch_workspace_bytes(m, s.num_topk, e)), **u8)
+        if s.fmt == ROW_BF16:
+            self.packed_recv_x = torch.empty((el, r * m, h), dtype=torch.bfloat16, device=device)
+            self.packed_recv_scales = None
+        else:
+            self.packed_recv_x = torch.empty((el, r * m, h), dtype=torch.float8_e4m3fn, device=device)
+            if s.fmt == ROW_FP8_UE8M0:
+                self.packed_recv_scales = torch.empty((el, r * m, h // 512), **i32)
+            else:
+                self.packed_recv_scales = torch.empty((el, r * m, h // 128), dtype=torch.float32, device=device)
+        self.packed_recv_count = torch.zeros(el, **i32)
+        self.packed_recv_src_info = torch.empty((el, r * m), **i32)
+        self.packed_recv_layout_range = torch.zeros((el, r), dtype=torch.int64, device=device)
+        # combine
+        self.combine_staging = torch.empty((e, m, h), dtype=torch.bfloat16, device=device)
+        self.combine_send_slots = (torch.empty((el, r, m, h), dtype=torch.bfloat16, device=device)
+                                   if keep_remote_rows else None)
+        self.combined_x = torch.empty((m, h), dtype=torch.bfloat16, device=device)
+
+    # -- dispatch ---------------------------------------------------------
+    def dispatch_send(self, x: torch.Tensor, topk_idx: torch.Tensor) -> None:
+        s = self.shape
+        t = x.shape[0]
+        _capi.check(self.lib.deepep_ll_dispatch_send(
+            _capi.ptr(x), _capi.ptr(topk_idx), t, s.hidden, s.num_topk, s.num_experts, s.num_ranks, s.rank,
+            s.max_tokens, s.fmt, _capi.ptr(self.recv_staging), _capi.ptr(self.recv_count),
+            _capi.ptr(self.send_slots), _capi.ptr(self.send_count), _capi.ptr(self.pair_slot),
+            _capi.ptr(self.workspace), self.workspace.numel(), current_stream_ptr()))
+
+    def dispatch_recv(self, stats: torch.Tensor = None) -> None:
+        s = self.shape
+        _capi.check(self.lib.deepep_ll_dispatch_recv(
+            _capi.ptr(self.recv_staging), _capi.ptr(self.recv_count), s.hidden, s.num_experts, s.num_ranks,
+            s.max_tokens, s.fmt, _capi.ptr(self.packed_recv_x), _capi.ptr(self.packed_recv_scales),
+            _capi.ptr(self.packed_recv_src_info), _capi.ptr(self.packed_recv_layout_range),
+            _capi.ptr(self.packed_recv_count), _capi.ptr(stats), current_stream_ptr()))
+
+    # -- combine ----------------------------------------------------------
+    def combine_send(self, x: torch.Tensor, layout_range: torch.Tensor = None) -> None:
+        s = self.shape
+        lr = self.packed_recv_layout_range if layout_range is None else layout_range
+        _capi.check(self.lib.deepep_ll_combine_send(
+            _capi.ptr(x), _capi.ptr(lr), s.hidden, s.num_experts, s.num_ranks, s.rank, s.max_tokens,
+            _capi.ptr(self.combine_staging), _capi.ptr(self.combine_send_slots), current_stream_ptr()))
+
+    def combine_recv(self, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor) -> None:
+        s = self.shape
+        t = topk_idx.shape[0]
+        _capi.check(self.lib.deepep_ll_combine_recv(
+            _capi.ptr(self.combine_staging), _capi.ptr(topk_idx), _capi.ptr(topk_weights), _capi.ptr(self.pair_slot),
+            t, s.hidden, s.num_topk, s.num_experts, s.max_tokens, _capi.ptr(out), current_stream_ptr()))

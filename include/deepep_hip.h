@@ -1,0 +1,290 @@
+/*
+ * deepep_hip.h — C ABI of the MI355X (gfx950) MoE token dispatch/combine hot path.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (`hipStream_t` passed as `void*`; NULL = the null stream).  Nothing here
+ * allocates device memory: outputs, staging buffers and workspaces are
+ * owned by the caller.  All work is enqueued on `stream` and is complete in
+ * stream order when the call returns; no entry point synchronises the host.
+ *
+ * Return value: 0 on success.  Non-zero = failure; `deepep_last_error()`
+ * then returns a thread-local message shaped like the reference's
+ * EPException text, "Failed: Assertion error <file>:<line> '<cond>'"
+ * (reference: csrc/kernels/exception.cuh:12-22,46-53).
+ *
+ * Vocabulary (reference: deep_ep/buffer.py:1836-1842):
+ *   T  tokens on this rank            H  hidden size (multiple of 128)
+ *   K  top-k                          E  experts in the EP world
+ *   R  ranks in the EP world          E_l = E / R local experts per rank
+ *   M  num_max_dispatch_tokens_per_rank            N = M * R
+ *   G  = H / 128 scale groups per token
+ *
+ * Expert e lives on rank e / E_l with local id e % E_l
+ * (reference: csrc/kernels/efa_kernels.cu:526,628).  topk_idx < 0 means
+ * "no selection" (reference: csrc/kernels/layout.cu:36,83).
+ */
+#ifndef DEEPEP_HIP_H
+#define DEEPEP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ */
+/* Library                                                            */
+/* ------------------------------------------------------------------ */
+
+/* Message of the last failure on the calling thread ("" if none). */
+const char* deepep_last_error(void);
+
+/* ABI revision of this header; bumped on any signature change. */
+int deepep_abi_version(void);
+
+/* ------------------------------------------------------------------ */
+/* Row formats of the low-latency path                                */
+/* ------------------------------------------------------------------ */
+
+/* Payload encodings of a dispatched token row.
+ * Reference: deep_ep/buffer.py:1647-1667 (data_bpt / scale_bpt / packed_bpt)
+ * and csrc/kernels/efa_kernels.cu:155-185 (scale encodings). */
+enum {
+    DEEPEP_ROW_BF16 = 0,       /* 2H bytes of bf16, no scales                    */
+    DEEPEP_ROW_FP8 = 1,        /* H bytes e4m3fn + G float32 scales (amax/448)   */
+    DEEPEP_ROW_FP8_POW2 = 2,   /* as FP8, scales rounded up to a power of two    */
+    DEEPEP_ROW_FP8_UE8M0 = 3   /* as POW2, scales stored as G exponent bytes     */
+};
+
+/* Bytes of the payload part of a row (data only). */
+size_t deepep_ll_row_data_bytes(int hidden, int row_format);
+/* Bytes of the scale part of a row (0 for bf16). */
+size_t deepep_ll_row_scale_bytes(int hidden, int row_format);
+/* Stride of one staged row: data and scales each padded to 16 B, plus a
+ * 16 B tail {int32 src_token, int32 topk_slot, int32 src_rank, int32 0}.
+ * 7408 for fp8 at H = 7168 — the value the reference's cooperative send
+ * uses (csrc/kernels/coop_dispatch_send.cu:73-75). */
+size_t deepep_ll_row_stride(int hidden, int row_format);
+
+/* Arithmetic of the reference's buffer sizing, kept for API parity.
+ * Replaces get_low_latency_rdma_size_hint (csrc/config.hpp:127-193). */
+size_t deepep_get_low_latency_rdma_size_hint(int num_max_dispatch_tokens_per_rank, int hidden,
+                                             int num_ranks, int num_experts);
+
+/* ------------------------------------------------------------------ */
+/* Route counting and layout                                          */
+/* ------------------------------------------------------------------ */
+
+/* Bytes of scratch `deepep_get_dispatch_layout` needs for this shape. */
+size_t deepep_layout_workspace_bytes(int num_tokens, int num_ranks, int num_experts);
+
+/* Per-expert pair counts, per-rank distinct-token counts, per-node counts
+ * and the token×rank membership matrix, in one pass over topk_idx.
+ *   topk_idx                  [T, K] int64
+ *   num_tokens_per_rank       [R] int32 (out)
+ *   num_tokens_per_rdma_rank  [R / 8] int32 (out) or NULL
+ *   num_tokens_per_expert     [E] int32 (out)
+ *   is_token_in_rank          [T, R] bool bytes (out)
+ * Replaces layout::get_dispatch_layout (csrc/kernels/layout.cu:9-149) as
+ * called by Buffer::get_dispatch_layout (csrc/deep_ep.cpp:517-581). */
+int deepep_get_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_topk,
+                               int num_ranks, int num_experts,
+                               int32_t* num_tokens_per_rank, int32_t* num_tokens_per_rdma_rank,
+                               int32_t* num_tokens_per_expert, uint8_t* is_token_in_rank,
+                               void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of scratch `deepep_moe_routing_sort` needs. */
+size_t deepep_routing_sort_workspace_bytes(int num_tokens, int num_ranks);
+
+/* Token ids grouped by destination rank, ascending inside each rank.
+ *   is_token_in_rank  [T, R] bool bytes
+ *   sorted_token_ids  [T * R] int64 (out; first send_cumsum[R] entries valid)
+ *   send_counts       [R] int32 (out)
+ *   send_cumsum       [R + 1] int64 (out, exclusive prefix; [R] = total)
+ * Replaces moe_routing_sort (csrc/kernels/efa_kernels.cu:220-318,1591-1651);
+ * the total stays on the device — the caller reads send_cumsum[R]. */
+int deepep_moe_routing_sort(const uint8_t* is_token_in_rank, int num_tokens, int num_ranks,
+                            int64_t* sorted_token_ids, int32_t* send_counts, int64_t* send_cumsum,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* channel_prefix_matrix[d, c] = number of tokens bound for rank d in
+ * channels 0..c, channel c owning tokens [min(c*ceil(T/C),T), min(+ceil(T/C),T)).
+ *   is_token_in_rank       [T, R] bool bytes
+ *   channel_prefix_matrix  [R, C] int32 (out)
+ * Replaces blocks >= 1 of intranode::notify_dispatch
+ * (csrc/kernels/intranode.cu:90-112, csrc/kernels/utils.cuh:434-438). */
+int deepep_channel_prefix_matrix(const uint8_t* is_token_in_rank, int num_tokens, int num_ranks,
+                                 int num_channels, int32_t* channel_prefix_matrix, void* stream);
+
+/* Normal-mode pack: dst_row[i] = src_row[sorted_token_ids[i]] for
+ * i < *num_rows_dev, rows of `row_bytes` (multiple of 16) bytes.  A second
+ * (scale) plane is gathered in the same launch when scale_src != NULL.
+ *   max_rows bounds the grid; rows >= *num_rows_dev are not touched.
+ * Replaces the torch index gathers x_data[flat_sorted_token_ids] and
+ * x_scales[flat_sorted_token_ids] (deep_ep/buffer.py:877,917). */
+int deepep_pack_rows(const void* src, const void* scale_src, const int64_t* sorted_token_ids,
+                     const int64_t* num_rows_dev, int64_t max_rows, int num_src_rows,
+                     int row_bytes, int scale_row_bytes,
+                     void* dst, void* scale_dst, void* stream);
+
+/* ------------------------------------------------------------------ */
+/* FP8 cast                                                           */
+/* ------------------------------------------------------------------ */
+
+/* Per token, per 128 channels: amax = max(max|x|, 1e-4), scale = amax/448,
+ * q = e4m3fn_rne(clamp(x * (448/amax), ±448)).
+ *   x        [M, N] bf16          x_fp8   [M, N] e4m3fn bytes (out)
+ *   scales   [M, N/128] float32, or [M, N/512] int32 for UE8M0 (out)
+ *   row_format: DEEPEP_ROW_FP8 | _POW2 | _UE8M0
+ * Replaces per_token_cast_to_fp8 (csrc/kernels/efa_kernels.cu:104-187,2281-2327;
+ * torch form deep_ep/buffer.py:1590-1621). */
+int deepep_per_token_cast_to_fp8(const void* x, int num_rows, int num_cols, int row_format,
+                                 void* x_fp8, void* scales, void* stream);
+
+/* ------------------------------------------------------------------ */
+/* Low-latency dispatch                                               */
+/* ------------------------------------------------------------------ */
+
+/* Bytes of scratch `deepep_ll_dispatch_send` needs. */
+size_t deepep_ll_dispatch_workspace_bytes(int num_tokens, int num_topk, int num_experts);
+
+/* Send side of the low-latency dispatch, one launch sequence:
+ *   route   — send_count[e] = pairs (t,k) with topk_idx[t,k] == e;
+ *             pair_slot[t,k] = rank of the pair among this rank's pairs for
+ *             that expert in ascending (t,k) order (-1 if no selection);
+ *   quantise + pack — each token row is quantised once (row_format) and
+ *             written once per selection into slot pair_slot[t,k] of its
+ *             expert: rows for this rank's own experts go straight into
+ *             recv_staging[(e_l * R + rank) * M + slot] (the self-copy the
+ *             reference does on the host side, csrc/transport/ll_pipeline.cpp:1542),
+ *             rows for remote experts into send_slots[e * M + slot];
+ *   counts  — recv_count[e_l * R + rank] and send_count[e].
+ *   x             [T, H] bf16        topk_idx   [T, K] int64
+ *   recv_staging  [E_l, R, M] rows of deepep_ll_row_stride bytes (in/out)
+ *   recv_count    [E_l, R] int32 (in/out; only column `rank` is written)
+ *   send_slots    [E, M] rows (out) or NULL to drop remote rows
+ *   send_count    [E] int32 (out)     pair_slot  [T, K] int32 (out)
+ * A pair whose slot would reach M (only possible when one token names the
+ * same expert twice) is dropped and its pair_slot is -1.
+ * Replaces per_token_cast_to_fp8 + ll_dispatch_route_and_pack_v3
+ * (csrc/kernels/efa_kernels.cu:2281,2332; kernels :512-845) and the
+ * cooperative a2a_dispatch_send (csrc/deep_ep.cpp:3641,
+ * csrc/kernels/coop_dispatch_send.cuh:304-790). */
+int deepep_ll_dispatch_send(const void* x, const int64_t* topk_idx,
+                            int num_tokens, int hidden, int num_topk,
+                            int num_experts, int num_ranks, int rank,
+                            int num_max_dispatch_tokens_per_rank, int row_format,
+                            void* recv_staging, int32_t* recv_count,
+                            void* send_slots, int32_t* send_count, int32_t* pair_slot,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
+/* Receive side: compacts the staged rows of every (local expert, source
+ * rank) segment into the packed layout.
+ *   begin(e,s) = sum_{s' < s} recv_count[e,s'];  rows [begin, begin+cnt)
+ *   of expert e hold source rank s's rows in staging order.
+ *   packed_recv_x            [E_l, N, H] e4m3fn bytes (or bf16) (out)
+ *   packed_recv_scales       [E_l, N, G] float32 / [E_l, N, G/4] int32 (out) or NULL
+ *   packed_recv_src_info     [E_l, N] int32 source token index (out)
+ *   packed_recv_layout_range [E_l, R] int64 = (begin << 32) | cnt, 0 if cnt == 0 (out)
+ *   packed_recv_count        [E_l] int32 (out)
+ *   cumulative_local_expert_recv_stats [E_l] int32, += count, or NULL
+ * Rows at or beyond packed_recv_count[e] are left untouched.
+ * Replaces ll_recv_unpack_v2 (csrc/kernels/efa_kernels.cu:2121-2231;
+ * kernels :877-1389) and a2a_dispatch_recv (csrc/deep_ep.cpp:3709,
+ * csrc/kernels/coop_dispatch_recv.cuh:39-304). */
+int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
+                            int hidden, int num_experts, int num_ranks,
+                            int num_max_dispatch_tokens_per_rank, int row_format,
+                            void* packed_recv_x, void* packed_recv_scales,
+                            int32_t* packed_recv_src_info, int64_t* packed_recv_layout_range,
+                            int32_t* packed_recv_count,
+                            int32_t* cumulative_local_expert_recv_stats, void* stream);
+
+/* ------------------------------------------------------------------ */
+/* Low-latency combine                                                */
+/* ------------------------------------------------------------------ */
+
+/* Send side: returns every live expert-output row to the rank it came from,
+ * in arrival order.  Row j of segment (e_l, s) — x[e_l, begin(e_l,s) + j] —
+ * goes to slot j of expert rank*E_l + e_l on rank s: this rank's own rows
+ * into combine_staging[(rank * E_l + e_l) * M + j], other ranks' rows into
+ * combine_send_slots[(e_l * R + s) * M + j] (NULL drops them).
+ *   x                   [E_l, N, H] bf16
+ *   layout_range        [E_l, R] int64 from the dispatch
+ *   combine_staging     [E, M, H] bf16 (in/out)
+ *   combine_send_slots  [E_l, R, M, H] bf16 (out) or NULL
+ * Replaces the two torch gathers of deep_ep/buffer.py:2601-2608 and
+ * a2a_combine_send (csrc/deep_ep.cpp:3804, csrc/kernels/coop_combine_send.cuh:34-275). */
+int deepep_ll_combine_send(const void* x, const int64_t* layout_range,
+                           int hidden, int num_experts, int num_ranks, int rank,
+                           int num_max_dispatch_tokens_per_rank,
+                           void* combine_staging, void* combine_send_slots, void* stream);
+
+/* Receive side: out[t,:] = bf16( sum_k [pair_slot[t,k] >= 0] * w[t,k] *
+ * f32(combine_staging[topk_idx[t,k], pair_slot[t,k], :]) ), accumulated in
+ * float32 as acc = fma(row_k, w_k, acc) for k = 0..K-1; tokens with no live
+ * selection give zeros.
+ *   combine_staging [E, M, H] bf16     topk_idx [T, K] int64
+ *   topk_weights    [T, K] float32     pair_slot [T, K] int32 from the dispatch
+ *   out             [T, H] bf16 (out)
+ * Replaces ll_combine_weighted_reduce_v2 (csrc/kernels/efa_kernels.cu:1413-1486,1982-2031)
+ * and a2a_combine_recv (csrc/deep_ep.cpp:3850, csrc/kernels/coop_combine_recv.cuh:69-283). */
+int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
+                           const float* topk_weights, const int32_t* pair_slot,
+                           int num_tokens, int hidden, int num_topk, int num_experts,
+                           int num_max_dispatch_tokens_per_rank, void* out, void* stream);
+
+/* ------------------------------------------------------------------ */
+/* Single-GPU loopback: peers synthesised in HBM                      */
+/* These stand where the reference has its transport                  */
+/* (csrc/transport/, dist.all_to_all_single at deep_ep/buffer.py:2268,2297,2735). */
+/* ------------------------------------------------------------------ */
+
+/* Seeded routing for `num_src` ranks: for each (rank, token) draws K distinct
+ * experts by repeated inverse-CDF sampling of 32-bit hashes against
+ * `expert_cdf` (E uint32 inclusive upper bounds), rejecting repeats.
+ *   src_ranks  [num_src] int32 world rank of each batch entry
+ *   topk_idx   [num_src, T, K] int64 (out) */
+int deepep_synth_topk_idx(const uint32_t* expert_cdf, const int32_t* src_ranks, int num_src,
+                          int num_tokens, int num_topk, int num_experts, uint32_t seed,
+                          int64_t* topk_idx, void* stream);
+
+/* Seeded bf16 rows, approximately N(0,1): value(seed, row_key, column) is the
+ * centred sum of the four bytes of a 32-bit hash times 1/147.8 in float32,
+ * rounded to bf16; rows whose key hash is 0 mod `outlier_period` are scaled
+ * by 100 first (outlier_period 0 = never).
+ *   row_keys  [num_rows] uint32 or NULL (key = first_key + row index)
+ *   dst       num_rows rows of `row_stride_bytes`, first 2*hidden bytes written */
+int deepep_synth_bf16_rows(void* dst, int64_t num_rows, int hidden, int64_t row_stride_bytes,
+                           const uint32_t* row_keys, uint32_t first_key, uint32_t seed,
+                           int outlier_period, void* stream);
+
+/* Runs the send side for `num_src` peer ranks and keeps only the rows bound
+ * for `rank`: they land in recv_staging[(e_l * R + src) * M + slot] with
+ * recv_count[e_l * R + src], exactly where the peers' own sends would put them.
+ *   x [num_src, T, H] bf16   topk_idx [num_src, T, K] int64   src_ranks [num_src] int32 (device)
+ *   workspace of num_src * deepep_ll_dispatch_workspace_bytes(T, K, E) bytes */
+int deepep_loopback_dispatch_from_peers(const void* x, const int64_t* topk_idx,
+                                        const int32_t* src_ranks, int num_src,
+                                        int num_tokens, int hidden, int num_topk,
+                                        int num_experts, int num_ranks, int rank,
+                                        int num_max_dispatch_tokens_per_rank, int row_format,
+                                        void* recv_staging, int32_t* recv_count,
+                                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Plays the remote experts for this rank's own pairs: for every remote
+ * expert e and slot j < send_count[e] writes combine_staging[e, j, :].
+ *   mode 0: the dequantised send_slots row (f32(q) * scale -> bf16), i.e. an
+ *           identity expert, the recipe of tests/test_low_latency.py:111;
+ *   mode 1: a seeded row with key e * M + j (see deepep_synth_bf16_rows). */
+int deepep_loopback_combine_from_peers(const void* send_slots, const int32_t* send_count,
+                                       int hidden, int num_experts, int num_ranks, int rank,
+                                       int num_max_dispatch_tokens_per_rank, int row_format,
+                                       int mode, uint32_t seed,
+                                       void* combine_staging, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEEPEP_HIP_H */

@@ -1,0 +1,465 @@
+"""CPU oracle of the MoE token dispatch/combine hot path.
+
+TEST INFRASTRUCTURE ONLY.  This module restates, on the CPU with torch and
+numpy, what the reference computes on this path; it is the checker for the
+HIP kernels and the timed CPU baseline of ``bench.py``.  Nothing in the
+product package imports it, and the product never falls back to it.
+
+Every function names the reference lines it follows.  What pins each one
+(the reference stores no golden vectors for this path; its tests are
+generative on CUDA RNG streams that cannot be replayed here):
+
+* layout counts, ``is_token_in_rank``  — brute force over tiny inputs written as
+  literal Python loops, and the closed forms of ``tests/test_intranode.py:35-66``.
+* FP8 cast — follows the live CUDA kernel (``csrc/kernels/efa_kernels.cu:156-169``:
+  ``scale = amax / 448.0f``, ``inv = 448.0f / amax``, IEEE float32 division; nvcc
+  flags in ``setup.py:12-13`` carry no fast-math).  The reference's torch helpers
+  (``deep_ep/buffer.py:1602``, ``tests/utils.py:57``) write ``448.0 / amax``, which
+  torch evaluates as ``amax.reciprocal() * 448.0`` — one ulp off for ~27 % of amax
+  values, and therefore a different FP8 byte for the rare element that lands on
+  a rounding tie.  ``per_token_cast_to_fp8_torch_helper`` keeps that form so the
+  difference stays measured (``tests/test_oracle.py``).  Pinned by torch's own
+  ``float8_e4m3fn`` CPU cast (a library routine), an
+  independent bit-level encoder in ``oracle_kernels.c`` run over every float32
+  that a bf16 x scale product can produce in the tests, and special cases
+  (all-zero group, exact powers of two, ±448 saturation, -0).
+* dispatch outputs — the invariants ``tests/test_low_latency.py:119-147``
+  checks, plus a literal serial restatement of the reference's deterministic
+  kernels (``_serial_dispatch``) compared against the vectorised form.
+* combine — the closed form ``x * sum(w)`` of ``tests/test_low_latency.py:181``
+  and a float64 sum.
+* ``get_low_latency_rdma_size_hint`` — hand-computed values.
+* ``round_scale`` scales: **parity unpinned at ulp boundaries** — the reference
+  computes ``exp2(ceil(log2(s)))`` in float32 (``deep_ep/buffer.py:1601``,
+  ``csrc/kernels/efa_kernels.cu:158``), whose result for s within one ulp above
+  a power of two depends on the libm in use; this oracle (and the kernel) take
+  the mathematical value, the smallest power of two >= s.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+FP8_MAX = 448.0
+GROUP = 128
+
+ROW_BF16, ROW_FP8, ROW_FP8_POW2, ROW_FP8_UE8M0 = 0, 1, 2, 3
+
+
+# ----------------------------------------------------------------------------
+# Sizes
+# ----------------------------------------------------------------------------
+def align_up(a: int, b: int) -> int:
+    return (a + b - 1) // b * b
+
+
+def get_low_latency_rdma_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
+                                   num_experts: int) -> int:
+    """csrc/config.hpp:127-193 (LowLatencyLayout + get_low_latency_rdma_size_hint)."""
+    num_scales = hidden // 128
+    dispatch_msg = 16 + max(hidden * 2, hidden + num_scales * 4)
+    combine_msg = num_scales * 4 + hidden * 2
+    m, e = num_max_dispatch_tokens_per_rank, num_experts
+    send = max(m * dispatch_msg, e * m * combine_msg)
+    recv = max(e * m * dispatch_msg, e * m * combine_msg)
+    sig = align_up(e * 4, 128)
+    total = send * 2 + recv * 2 + sig * 2
+    return (total + 128) // 128 * 128
+
+
+def row_data_bytes(hidden: int, fmt: int) -> int:
+    return hidden * 2 if fmt == ROW_BF16 else hidden
+
+
+def row_scale_bytes(hidden: int, fmt: int) -> int:
+    if fmt == ROW_BF16:
+        return 0
+    g = hidden // GROUP
+    return g if fmt == ROW_FP8_UE8M0 else 4 * g
+
+
+def row_stride(hidden: int, fmt: int) -> int:
+    """data and scales padded to 16 B + 16 B tail (csrc/kernels/coop_dispatch_send.cu:73-75)."""
+    return align_up(row_data_bytes(hidden, fmt), 16) + align_up(row_scale_bytes(hidden, fmt), 16) + 16
+
+
+# ----------------------------------------------------------------------------
+# Layout
+# ----------------------------------------------------------------------------
+def get_dispatch_layout(topk_idx: torch.Tensor, num_experts: int, num_ranks: int):
+    """csrc/kernels/layout.cu:9-121; recipe of tests/test_intranode.py:35-66.
+
+    Returns (num_tokens_per_rank i32 [R], num_tokens_per_rdma_rank i32 [R/8] or None,
+    num_tokens_per_expert i32 [E], is_token_in_rank bool [T, R]).
+    """
+    t = topk_idx.shape[0]
+    epr = num_experts // num_ranks
+    valid = (topk_idx >= 0) & (topk_idx < num_experts)
+    flat = topk_idx[valid]
+    per_expert = torch.bincount(flat, minlength=num_experts).to(torch.int32)
+    is_in = torch.zeros((t, num_ranks), dtype=torch.bool)
+    tok = torch.arange(t).view(-1, 1).expand_as(topk_idx)[valid]
+    is_in[tok, flat // epr] = True
+    per_rank = is_in.sum(0).to(torch.int32)
+    per_rdma = None
+    if num_ranks > 8 and num_ranks % 8 == 0:
+        per_rdma = is_in.view(t, num_ranks // 8, 8).any(-1).sum(0).to(torch.int32)
+    return per_rank, per_rdma, per_expert, is_in
+
+
+def moe_routing_sort(is_token_in_rank: torch.Tensor):
+    """csrc/kernels/efa_kernels.cu:220-318,1591-1651: ids ascending inside each rank."""
+    t, r = is_token_in_rank.shape
+    rank_of, tok_of = torch.nonzero(is_token_in_rank.t().contiguous(), as_tuple=True)
+    counts = is_token_in_rank.sum(0).to(torch.int32)
+    cumsum = torch.zeros(r + 1, dtype=torch.int64)
+    cumsum[1:] = torch.cumsum(counts.to(torch.int64), 0)
+    return tok_of.to(torch.int64), counts, cumsum, int(cumsum[-1])
+
+
+def channel_prefix_matrix(is_token_in_rank: torch.Tensor, num_channels: int) -> torch.Tensor:
+    """csrc/kernels/intranode.cu:90-112 with the ranges of csrc/kernels/utils.cuh:434-438."""
+    t, r = is_token_in_rank.shape
+    per = (t + num_channels - 1) // num_channels
+    out = torch.zeros((r, num_channels), dtype=torch.int32)
+    for c in range(num_channels):
+        b = min(per * c, t)
+        e = min(b + per, t)
+        out[:, c] = is_token_in_rank[b:e].sum(0).to(torch.int32)
+    return torch.cumsum(out, 1).to(torch.int32)
+
+
+# ----------------------------------------------------------------------------
+# FP8
+# ----------------------------------------------------------------------------
+def pow2_ceil(s: torch.Tensor) -> torch.Tensor:
+    """Smallest power of two >= s for positive normal float32 (bit arithmetic)."""
+    bits = s.contiguous().view(torch.int32)
+    ex = (bits >> 23) & 0xFF
+    ex = ex + ((bits & 0x7FFFFF) != 0).to(torch.int32)
+    return (ex << 23).view(torch.float32)
+
+
+def per_token_cast_to_fp8(x: torch.Tensor, round_scale: bool = False, use_ue8m0: bool = False):
+    """deep_ep/buffer.py:1590-1621 and csrc/kernels/efa_kernels.cu:143-185.
+
+    x [M, N] bf16 -> (x_fp8 [M, N] float8_e4m3fn, scales [M, N/128] f32 | [M, N/512] i32).
+    """
+    assert x.dim() == 2 and x.shape[1] % GROUP == 0
+    m, n = x.shape
+    xg = x.view(m, -1, GROUP).float()
+    amax = xg.abs().amax(dim=2).clamp(min=1e-4)
+    scales = amax / FP8_MAX
+    if round_scale:
+        scales = pow2_ceil(scales)
+        inv = torch.ones_like(scales) / scales  # exact: scales are powers of two
+    else:
+        inv = torch.full_like(amax, FP8_MAX) / amax  # tensor / tensor: IEEE division, as 448.0f / amax
+    q = (xg * inv.unsqueeze(2)).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn).view(m, n)
+    if use_ue8m0:
+        assert round_scale and (n // GROUP) % 4 == 0
+        ex = ((scales.contiguous().view(torch.int32) >> 23) & 0xFF).to(torch.uint8)
+        return q, ex.view(m, -1, 4).contiguous().view(torch.int32).view(m, -1)
+    return q, scales
+
+
+def per_token_cast_to_fp8_torch_helper(x: torch.Tensor):
+    """tests/utils.py:50-58 verbatim in meaning: ``448.0 / amax`` is reciprocal-then-multiply in torch."""
+    m, n = x.shape
+    xv = x.view(m, -1, GROUP)
+    amax = xv.abs().float().amax(dim=2).view(m, -1).clamp(1e-4)
+    return (xv * (448.0 / amax.unsqueeze(2))).to(torch.float8_e4m3fn).view(m, n), (amax / 448.0).view(m, -1)
+
+
+def per_token_cast_back(x_fp8: torch.Tensor, scales: torch.Tensor) -> torch.Tensor:
+    """tests/utils.py:61-74."""
+    if x_fp8.numel() == 0:
+        return x_fp8.to(torch.bfloat16)
+    m, n = x_fp8.shape
+    if scales.dtype == torch.int32:
+        scales = (scales.contiguous().view(torch.uint8).to(torch.int32) << 23).view(torch.float32)
+    xf = x_fp8.to(torch.float32).view(m, -1, GROUP)
+    return (xf * scales.reshape(m, -1, 1)).view(m, n).to(torch.bfloat16)
+
+
+def quantise_rows(x: torch.Tensor, fmt: int):
+    """Payload bytes [T, data_bytes] u8 and scale bytes [T, scale_bytes] u8 of each token row."""
+    t = x.shape[0]
+    if fmt == ROW_BF16:
+        return x.contiguous().view(torch.uint8).view(t, -1), torch.zeros((t, 0), dtype=torch.uint8)
+    q, s = per_token_cast_to_fp8(x, round_scale=fmt != ROW_FP8, use_ue8m0=fmt == ROW_FP8_UE8M0)
+    return q.view(torch.uint8).view(t, -1), s.contiguous().view(torch.uint8).view(t, -1)
+
+
+# ----------------------------------------------------------------------------
+# Low-latency dispatch
+# ----------------------------------------------------------------------------
+def route(topk_idx: torch.Tensor, num_experts: int, max_tokens: int):
+    """Send-side routing of one rank.
+
+    send_count[e] = pairs (t,k) naming expert e (csrc/kernels/coop_dispatch_send.cuh:360-395
+    num_routed); pair_slot[t,k] = rank of the pair among this rank's pairs for
+    that expert in ascending (t,k) order — the order of the reference's serial
+    scan (csrc/kernels/efa_kernels.cu:617-637).  Pairs beyond max_tokens are dropped.
+    """
+    t, k = topk_idx.shape
+    flat = topk_idx.reshape(-1)
+    valid = (flat >= 0) & (flat < num_experts)
+    idx = torch.nonzero(valid).view(-1)
+    e = flat[idx]
+    order = torch.sort(e, stable=True).indices
+    e_sorted = e[order]
+    counts = torch.bincount(e_sorted, minlength=num_experts)
+    starts = torch.cumsum(counts, 0) - counts
+    slot_sorted = torch.arange(e_sorted.numel()) - starts[e_sorted]
+    pair_slot = torch.full((t * k,), -1, dtype=torch.int32)
+    pair_slot[idx[order]] = slot_sorted.to(torch.int32)
+    pair_slot[pair_slot >= max_tokens] = -1
+    send_count = counts.clamp(max=max_tokens).to(torch.int32)
+    return send_count, pair_slot.view(t, k)
+
+
+def ll_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_tokens: int, fmt: int = ROW_FP8):
+    """What rank `rank` receives when every rank of the world dispatches.
+
+    all_x: list of R tensors [T_s, H] bf16; all_topk_idx: list of R tensors [T_s, K] int64.
+    Follows deep_ep/buffer.py:1816-1887,2266-2457 (nccl-fallback branch) with
+    ll_recv_build_positions (csrc/kernels/efa_kernels.cu:1017-1052) for the
+    ranges and the deterministic scatter (:1059-1213) for the slot order.
+
+    Returns dict with packed_recv_x u8 [E_l, N, data_bytes], packed_recv_scales u8
+    [E_l, N, scale_bytes], packed_recv_count i32 [E_l], packed_recv_src_info i32
+    [E_l, N], packed_recv_layout_range i64 [E_l, R]; rows past the count are zero.
+    """
+    r = len(all_x)
+    epr = num_experts // r
+    n = max_tokens * r
+    hidden = all_x[0].shape[1]
+    db, sb = row_data_bytes(hidden, fmt), row_scale_bytes(hidden, fmt)
+    px = torch.zeros((epr, n, db), dtype=torch.uint8)
+    ps = torch.zeros((epr, n, sb), dtype=torch.uint8)
+    src_info = torch.zeros((epr, n), dtype=torch.int32)
+    layout = torch.zeros((epr, r), dtype=torch.int64)
+    count = torch.zeros(epr, dtype=torch.int32)
+    cursor = [0] * epr
+    per_src = []
+    for s in range(r):
+        _, pair_slot = route(all_topk_idx[s], num_experts, max_tokens)
+        data, scales = quantise_rows(all_x[s], fmt)
+        per_src.append((pair_slot, data, scales))
+    for le in range(epr):
+        e = rank * epr + le
+        for s in range(r):
+            pair_slot, data, scales = per_src[s]
+            sel = (all_topk_idx[s] == e) & (pair_slot >= 0)
+            tok, kk = torch.nonzero(sel, as_tuple=True)
+            slots = pair_slot[tok, kk].to(torch.int64)
+            c = int(tok.numel())
+            if c:
+                b = cursor[le]
+                px[le, b + slots] = data[tok]
+                if sb:
+                    ps[le, b + slots] = scales[tok]
+                src_info[le, b + slots] = tok.to(torch.int32)
+                layout[le, s] = (b << 32) | c
+                cursor[le] += c
+        count[le] = cursor[le]
+    return dict(packed_recv_x=px, packed_recv_scales=ps, packed_recv_count=count,
+                packed_recv_src_info=src_info, packed_recv_layout_range=layout)
+
+
+def _serial_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_tokens: int, fmt: int = ROW_FP8):
+    """Literal restatement, in Python loops, of the reference's deterministic kernels:
+    sender scan csrc/kernels/efa_kernels.cu:617-637 (per destination rank, (t,k) order),
+    receiver count/build :877-923,1017-1052 and scatter :1112-1141 (arrival order per
+    source, position = pair_cumsum + running pair counter).  Small inputs only."""
+    r = len(all_x)
+    epr = num_experts // r
+    n = max_tokens * r
+    hidden = all_x[0].shape[1]
+    db, sb = row_data_bytes(hidden, fmt), row_scale_bytes(hidden, fmt)
+    arrivals = []  # per source: list of (token, local_eid) in send order
+    for s in range(r):
+        rows = []
+        tk = all_topk_idx[s].tolist()
+        for t, row in enumerate(tk):
+            for e in row:
+                if e >= 0 and e // epr == rank:
+                    rows.append((t, e % epr))
+        arrivals.append(rows)
+    pair_counts = [[0] * r for _ in range(epr)]
+    for s in range(r):
+        for _, le in arrivals[s]:
+            pair_counts[le][s] += 1
+    px = torch.zeros((epr, n, db), dtype=torch.uint8)
+    ps = torch.zeros((epr, n, sb), dtype=torch.uint8)
+    src_info = torch.zeros((epr, n), dtype=torch.int32)
+    layout = torch.zeros((epr, r), dtype=torch.int64)
+    count = torch.zeros(epr, dtype=torch.int32)
+    pair_cumsum = [[0] * r for _ in range(epr)]
+    for le in range(epr):
+        pos = 0
+        for s in range(r):
+            c = pair_counts[le][s]
+            pair_cumsum[le][s] = pos
+            layout[le, s] = ((pos << 32) | c) if c > 0 else 0
+            pos += c
+        count[le] = pos
+    for s in range(r):
+        data, scales = quantise_rows(all_x[s], fmt)
+        written = [0] * epr
+        for t, le in arrivals[s]:
+            p = pair_cumsum[le][s] + written[le]
+            written[le] += 1
+            px[le, p] = data[t]
+            if sb:
+                ps[le, p] = scales[t]
+            src_info[le, p] = t
+    return dict(packed_recv_x=px, packed_recv_scales=ps, packed_recv_count=count,
+                packed_recv_src_info=src_info, packed_recv_layout_range=layout)
+
+
+def staged_rows(x: torch.Tensor, topk_idx: torch.Tensor, src_rank: int, num_experts: int, max_tokens: int,
+                fmt: int):
+    """Rows one rank emits, keyed (expert, slot) -> stride-sized row bytes, as the
+    send side stages them: [data|pad][scales|pad][token, k, src_rank, 0]."""
+    hidden = x.shape[1]
+    db, sb = row_data_bytes(hidden, fmt), row_scale_bytes(hidden, fmt)
+    dp, sp = align_up(db, 16), align_up(sb, 16)
+    stride = dp + sp + 16
+    send_count, pair_slot = route(topk_idx, num_experts, max_tokens)
+    data, scales = quantise_rows(x, fmt)
+    tok, kk = torch.nonzero(pair_slot >= 0, as_tuple=True)
+    rows = torch.zeros((tok.numel(), stride), dtype=torch.uint8)
+    rows[:, :db] = data[tok]
+    if sb:
+        rows[:, dp:dp + sb] = scales[tok]
+    tail = torch.stack([tok.to(torch.int32), kk.to(torch.int32), torch.full_like(tok, src_rank, dtype=torch.int32),
+                        torch.zeros_like(tok, dtype=torch.int32)], 1).contiguous()
+    rows[:, dp + sp:] = tail.view(torch.uint8).view(-1, 16)
+    experts = topk_idx[tok, kk]
+    slots = pair_slot[tok, kk].to(torch.int64)
+    return send_count, pair_slot, experts, slots, rows
+
+
+# ----------------------------------------------------------------------------
+# Low-latency combine
+# ----------------------------------------------------------------------------
+def ll_combine(pair_rows: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
+               pair_live: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = sum_k [live] w[t,k] * f32(pair_rows[t,k]) in float64, rounded to bf16 by the caller's check.
+
+    pair_rows [T, K, H] bf16 — the expert output returned for each pair.
+    csrc/kernels/efa_kernels.cu:1413-1474 (weight lookup + accumulate) and
+    csrc/kernels/coop_combine_recv.cuh:222-260 (per-pair, k order).  Returns float64 [T, H].
+    """
+    live = (topk_idx >= 0) if pair_live is None else pair_live
+    w = topk_weights.double() * live.double()
+    return (pair_rows.double() * w.unsqueeze(-1)).sum(1)
+
+
+def ll_combine_f32_chain(pair_rows: torch.Tensor, topk_weights: torch.Tensor, pair_live: torch.Tensor):
+    """Bit-level definition: acc = 0; for k: acc = fma(f32(row_k), w_k, acc); bf16_rne(acc).
+
+    float32 FMA emulated exactly: the product of two float32 is exact in float64;
+    the float64 sum with a float32 addend is rounded once to float64 and once more
+    to float32 — double rounding can differ from a true FMA only when the float64
+    result sits exactly on a float32 rounding boundary, which the C checker
+    (oracle_kernels.c, fmaf) covers; this torch form is used for speed.
+    """
+    t, k, h = pair_rows.shape
+    acc = torch.zeros((t, h), dtype=torch.float32)
+    for j in range(k):
+        prod = pair_rows[:, j].double() * topk_weights[:, j].double().unsqueeze(1)
+        nxt = (prod + acc.double()).float()
+        acc = torch.where(pair_live[:, j].unsqueeze(1), nxt, acc)
+    return acc.to(torch.bfloat16)
+
+
+def calc_diff(x: torch.Tensor, y: torch.Tensor) -> float:
+    """tests/utils.py:39-43."""
+    x, y = x.double() + 1, y.double() + 1
+    den = (x * x + y * y).sum()
+    return float(1 - 2 * (x * y).sum() / den)
+
+
+# ----------------------------------------------------------------------------
+# Seeded world (mirrors the synthesiser kernels; integer hashing + exact float32 steps)
+# ----------------------------------------------------------------------------
+_M32 = np.uint64(0xFFFFFFFF)
+
+
+def mix32(x):
+    x = np.asarray(x, dtype=np.uint64) & _M32
+    x ^= x >> np.uint64(16)
+    x = (x * np.uint64(0x7FEB352D)) & _M32
+    x ^= x >> np.uint64(15)
+    x = (x * np.uint64(0x846CA68B)) & _M32
+    x ^= x >> np.uint64(16)
+    return x
+
+
+def row_hash(seed: int, key):
+    key = np.asarray(key, dtype=np.uint64)
+    return mix32(np.uint64(seed & 0xFFFFFFFF) ^ mix32((key + np.uint64(0x9E3779B9)) & _M32))
+
+
+def synth_bf16_rows(keys, hidden: int, seed: int, outlier_period: int = 0) -> torch.Tensor:
+    """bf16 rows [len(keys), hidden]; value(seed, key, col) as the synthesiser defines it."""
+    keys = np.asarray(keys, dtype=np.uint64)
+    rh = row_hash(seed, keys)[:, None]
+    col = np.arange(hidden, dtype=np.uint64)[None, :]
+    h = mix32(rh ^ ((col * np.uint64(0x9E3779B1) + np.uint64(0x85EBCA6B)) & _M32))
+    s = (h & np.uint64(255)) + ((h >> np.uint64(8)) & np.uint64(255)) + ((h >> np.uint64(16)) & np.uint64(255)) + (
+        h >> np.uint64(24))
+    f = (s.astype(np.int64) - 510).astype(np.float32) * np.array([0x3BDDB47B], dtype=np.uint32).view(np.float32)[0]
+    if outlier_period > 0:
+        hot = (mix32(rh ^ np.uint64(0x5BD1E995)) % np.uint64(outlier_period)) == 0
+        f = np.where(hot, f * np.float32(100.0), f).astype(np.float32)
+    return torch.from_numpy(f).to(torch.bfloat16)
+
+
+def uniform_cdf(num_experts: int) -> np.ndarray:
+    """Inclusive 32-bit upper bounds of E equal cells."""
+    return (((np.arange(1, num_experts + 1, dtype=np.uint64) << np.uint64(32)) // np.uint64(num_experts)) -
+            np.uint64(1)).astype(np.uint32)
+
+
+def zipf_cdf(num_experts: int, s: float = 1.2) -> np.ndarray:
+    """p(e) proportional to (e+1)^-s, as inclusive 32-bit upper bounds; last cell closes at 2^32-1."""
+    p = (np.arange(1, num_experts + 1, dtype=np.float64)) ** (-s)
+    c = np.cumsum(p / p.sum())
+    out = np.minimum(np.floor(c * 4294967296.0), 4294967295.0).astype(np.uint64)
+    out[-1] = 0xFFFFFFFF
+    return out.astype(np.uint32)
+
+
+def synth_topk_idx(cdf: np.ndarray, ranks, num_tokens: int, num_topk: int, seed: int) -> torch.Tensor:
+    """int64 [len(ranks), T, K]: K distinct experts per token by repeated inverse-CDF draws."""
+    num_experts = len(cdf)
+    ranks = np.asarray(ranks, dtype=np.uint64)
+    keys = (ranks[:, None] * np.uint64(num_tokens) + np.arange(num_tokens, dtype=np.uint64)[None, :]) & _M32
+    th = row_hash((seed ^ 0x7F4A7C15) & 0xFFFFFFFF, keys).reshape(-1)
+    n = th.shape[0]
+    chosen = np.full((n, num_topk), -1, dtype=np.int64)
+    have = np.zeros(n, dtype=np.int64)
+    cdf64 = cdf.astype(np.uint64)
+    for c in range(64 * num_topk):
+        todo = have < num_topk
+        if not todo.any():
+            break
+        u = mix32((th + np.uint64((c * 0x9E3779B9) & 0xFFFFFFFF)) & _M32)
+        e = np.searchsorted(cdf64, u, side='left').astype(np.int64)
+        seen = (chosen == e[:, None]).any(1)
+        take = todo & ~seen
+        rows = np.nonzero(take)[0]
+        chosen[rows, have[rows]] = e[rows]
+        have[rows] += 1
+    for row in np.nonzero(have < num_topk)[0]:
+        for e in range(num_experts):
+            if have[row] >= num_topk:
+                break
+            if e not in chosen[row, :have[row]]:
+                chosen[row, have[row]] = e
+                have[row] += 1
+    return torch.from_numpy(chosen.reshape(len(ranks), num_tokens, num_topk))

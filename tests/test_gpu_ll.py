@@ -1,0 +1,335 @@
+"""GPU parity of the low-latency dispatch + combine path, through the C ABI.
+
+One GPU plays rank `rank` of an R-rank world; the other ranks' rows are put
+in HBM by the loopback entry points.  Expected values come from the CPU
+oracle restated from the reference.  Integer outputs, FP8 bytes and scales
+must be bit-exact; the combine must match the float32 FMA-chain definition
+bit for bit and the float64 sum within 1e-2 relative.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import deepep_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def rt():
+    from deepep_efa_amd import _capi, ll_runtime, loopback
+    _capi.load()
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+
+    class NS:
+        pass
+
+    ns = NS()
+    ns.capi, ns.ll, ns.lb = _capi, ll_runtime, loopback
+    return ns
+
+
+def make_world(r, t, h, k, e, seed, drop=10, recipe="randn"):
+    g = torch.Generator().manual_seed(seed)
+    if recipe == "rank_const":  # tests/test_low_latency.py:59-60
+        xs = []
+        for rank in range(r):
+            x = torch.ones((t, h), dtype=torch.bfloat16) * (rank - 128)
+            x[:, -128:] = torch.arange(t).to(torch.bfloat16).view(-1, 1)
+            xs.append(x)
+        x_all = torch.stack(xs)
+    else:
+        x_all = torch.randn((r, t, h), generator=g).to(torch.bfloat16)
+        x_all[:, ::9] *= 30
+    scores = torch.rand((r, t, e), generator=g)
+    topk = torch.topk(scores, k, dim=-1)[1].contiguous()
+    for _ in range(drop):
+        s, i, j = [int(torch.randint(0, n, (1,), generator=g)) for n in (r, t, k)]
+        topk[s, i, j] = -1
+    w = torch.randn((r, t, k), generator=g).abs()
+    return x_all, topk, w
+
+
+def dispatch_on_gpu(rt, x_all, topk_all, rank, e, m, fmt, stats=None):
+    r, t, h = x_all.shape
+    k = topk_all.shape[2]
+    shape = rt.ll.LLShape(num_ranks=r, rank=rank, num_experts=e, max_tokens=m, hidden=h, num_topk=k, fmt=fmt)
+    st = rt.ll.LowLatencyState(shape)
+    world = rt.lb.LoopbackWorld(r, rank, seed=0)
+    world.set_inputs(x_all.cuda(), topk_all.cuda())
+    x, topk = world.own_inputs()
+    st.dispatch_send(x, topk)
+    world.dispatch_from_peers(st)
+    st.dispatch_recv(stats)
+    torch.cuda.synchronize()
+    return st, world
+
+
+def check_dispatch(st, want, fmt):
+    count = st.packed_recv_count.cpu()
+    assert torch.equal(count, want["packed_recv_count"])
+    assert torch.equal(st.packed_recv_layout_range.cpu(), want["packed_recv_layout_range"])
+    px = st.packed_recv_x.view(torch.uint8).view(want["packed_recv_x"].shape).cpu()
+    src = st.packed_recv_src_info.cpu()
+    ps = None if st.packed_recv_scales is None else \
+        st.packed_recv_scales.view(torch.uint8).view(want["packed_recv_scales"].shape).cpu()
+    for le in range(count.numel()):
+        n = int(count[le])
+        assert torch.equal(src[le, :n], want["packed_recv_src_info"][le, :n]), f"src_info expert {le}"
+        assert torch.equal(px[le, :n], want["packed_recv_x"][le, :n]), f"payload bytes expert {le}"
+        if ps is not None:
+            assert torch.equal(ps[le, :n], want["packed_recv_scales"][le, :n]), f"scale bytes expert {le}"
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16, O.ROW_FP8_POW2, O.ROW_FP8_UE8M0])
+@pytest.mark.parametrize("r,rank,t,h,k,e", [(4, 1, 8, 512, 3, 16), (8, 7, 33, 1024, 4, 64), (2, 0, 1, 512, 1, 2)])
+def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e):
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=r * 100 + t, drop=min(5, t))
+    st, _ = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
+    check_dispatch(st, want, fmt)
+
+
+def test_dispatch_send_staging_and_send_slots(rt):
+    """The send side alone: own rows for own experts land in recv_staging, the rest in send_slots."""
+    r, rank, t, h, k, e, m = 4, 2, 20, 512, 4, 32, 24
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=5, drop=6)
+    shape = rt.ll.LLShape(r, rank, e, m, h, k, O.ROW_FP8)
+    st = rt.ll.LowLatencyState(shape)
+    st.recv_staging.fill_(0xAB)
+    st.send_slots.fill_(0xCD)
+    st.dispatch_send(x_all[rank].cuda(), topk_all[rank].cuda())
+    torch.cuda.synchronize()
+    send_count, pair_slot, experts, slots, rows = O.staged_rows(x_all[rank], topk_all[rank], rank, e, m, O.ROW_FP8)
+    assert torch.equal(st.send_count.cpu(), send_count)
+    assert torch.equal(st.pair_slot[:t].cpu(), pair_slot)
+    stride = st.stride
+    staging = st.recv_staging.cpu().view(e // r, r, m, stride)
+    sendbuf = st.send_slots.cpu().view(e, m, stride)
+    epr = e // r
+    touched_stage = torch.zeros((epr, r, m), dtype=torch.bool)
+    touched_send = torch.zeros((e, m), dtype=torch.bool)
+    for i in range(rows.shape[0]):
+        ex, sl = int(experts[i]), int(slots[i])
+        if ex // epr == rank:
+            assert torch.equal(staging[ex % epr, rank, sl], rows[i])
+            touched_stage[ex % epr, rank, sl] = True
+        else:
+            assert torch.equal(sendbuf[ex, sl], rows[i])
+            touched_send[ex, sl] = True
+    assert (staging[~touched_stage] == 0xAB).all() and (sendbuf[~touched_send] == 0xCD).all()
+    rc = st.recv_count.cpu().view(epr, r)
+    assert torch.equal(rc[:, rank], send_count[rank * epr:(rank + 1) * epr])
+    assert (rc[:, [s for s in range(r) if s != rank]] == 0).all()
+
+
+@pytest.mark.parametrize("use_fp8", [True, False])
+def test_reference_recipe_roundtrip(rt, use_fp8):
+    """tests/test_low_latency.py:59-60,113-147,181-184 on one rank of an 8-rank world."""
+    r, rank, t, h, k, e = 8, 3, 64, 2048, 6, 64
+    fmt = O.ROW_FP8 if use_fp8 else O.ROW_BF16
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=77, drop=10, recipe="rank_const")
+    stats = torch.zeros(e // r, dtype=torch.int32, device="cuda")
+    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt, stats)
+    epr = e // r
+    count = st.packed_recv_count.cpu()
+    lr_all = st.packed_recv_layout_range.cpu()
+    assert torch.equal(stats.cpu(), count)
+    for i in range(epr):
+        expert = rank * epr + i
+        n = int(count[i])
+        lr = lr_all[i]
+        assert n == int((lr & 0xFFFFFFFF).sum()) == int((topk_all == expert).sum())
+        if n == 0:
+            continue
+        if use_fp8:
+            recv = O.per_token_cast_back(st.packed_recv_x[i, :n].cpu(), st.packed_recv_scales[i, :n].cpu()).float()
+        else:
+            recv = st.packed_recv_x[i, :n].cpu().float()
+        src = st.packed_recv_src_info[i, :n].cpu()
+        assert torch.equal(recv[:, :-128].amin(-1), recv[:, :-128].amax(-1))
+        assert (recv[:, -128:] - src.view(-1, 1) % t).sum().item() == 0
+        for j in range(r):
+            begin, cnt = int(lr[j] >> 32), int(lr[j] & 0xFFFFFFFF)
+            assert int((recv[:, :-128].amin(-1) == j - 128).sum()) == int((topk_all[j] == expert).sum())
+            assert (recv[begin:begin + cnt, :-128] - j + 128).sum().item() == 0
+    # combine with an identity expert (simulated_gemm_x = dequantised recv)
+    if use_fp8:
+        el, n_slots = st.packed_recv_x.shape[:2]
+        q = st.packed_recv_x.view(-1, h).cpu()
+        sc = st.packed_recv_scales.view(-1, h // 128).cpu()
+        live = torch.zeros((el, n_slots), dtype=torch.bool)
+        for i in range(el):
+            live[i, :int(count[i])] = True
+        y = torch.zeros((el * n_slots, h), dtype=torch.bfloat16)
+        y[live.view(-1)] = O.per_token_cast_back(q[live.view(-1)], sc[live.view(-1)])
+        y = y.view(el, n_slots, h).cuda()
+    else:
+        y = st.packed_recv_x.clone()
+    world.combine_from_peers(st, mode=0)
+    st.combine_send(y)
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    topk, w = topk_all[rank].cuda(), w_all[rank].cuda()
+    st.combine_recv(topk, w, out)
+    torch.cuda.synchronize()
+    x = x_all[rank]
+    wsum = w_all[rank].masked_fill(topk_all[rank] == -1, 0).sum(1).view(-1, 1)
+    diff = O.calc_diff(x.float() * wsum, out.cpu())
+    assert torch.isnan(out.float()).sum().item() == 0
+    assert diff < (9e-4 if use_fp8 else 1e-5), diff
+
+
+@pytest.mark.parametrize("r,rank,t,h,k,e", [(32, 5, 128, 7168, 8, 256), (4, 0, 16, 512, 3, 8)])
+def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e):
+    """Seeded expert outputs along the dispatch routing; combine vs the float32 chain and the float64 sum."""
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=31 + r, drop=10)
+    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, O.ROW_FP8)
+    epr, n_slots, lib, capi = e // r, r * t, rt.capi.load(), rt.capi
+    seed_local, seed_remote = 1234, 4321
+    # local experts' outputs: row key = local_expert * N + slot
+    y = torch.zeros((epr, n_slots, h), dtype=torch.bfloat16, device="cuda")
+    capi.check(lib.deepep_synth_bf16_rows(capi.ptr(y), epr * n_slots, h, h * 2, None, 0, seed_local, 0,
+                                          torch.cuda.current_stream().cuda_stream))
+    world.combine_from_peers(st, mode=1, seed=seed_remote)
+    st.combine_send(y)
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    st.combine_recv(topk_all[rank].cuda(), w_all[rank].cuda(), out)
+    torch.cuda.synchronize()
+    # oracle: which row does each of this rank's pairs get back?
+    topk, w = topk_all[rank], w_all[rank]
+    _, pair_slot = O.route(topk, e, t)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
+    keys_local, keys_remote = [], []
+    pair_rows = torch.zeros((t, k, h), dtype=torch.bfloat16)
+    live = pair_slot >= 0
+    idx_local, idx_remote = [], []
+    for ti in range(t):
+        for ki in range(k):
+            if not live[ti, ki]:
+                continue
+            ex, sl = int(topk[ti, ki]), int(pair_slot[ti, ki])
+            if ex // epr == rank:
+                begin = int(want["packed_recv_layout_range"][ex % epr, rank] >> 32)
+                keys_local.append((ex % epr) * n_slots + begin + sl)
+                idx_local.append((ti, ki))
+            else:
+                keys_remote.append(ex * t + sl)
+                idx_remote.append((ti, ki))
+    if idx_local:
+        rows = O.synth_bf16_rows(np.array(keys_local, dtype=np.uint32), h, seed_local)
+        ii = torch.tensor(idx_local)
+        pair_rows[ii[:, 0], ii[:, 1]] = rows
+    if idx_remote:
+        rows = O.synth_bf16_rows(np.array(keys_remote, dtype=np.uint32), h, seed_remote)
+        ii = torch.tensor(idx_remote)
+        pair_rows[ii[:, 0], ii[:, 1]] = rows
+    chain = torch.empty((t, h), dtype=torch.int16)
+    live8 = live.to(torch.uint8).contiguous()
+    oracle_c.oracle_combine_chain(ctypes.c_void_p(pair_rows.view(torch.int16).data_ptr()),
+                                  ctypes.c_void_p(w.contiguous().data_ptr()), ctypes.c_void_p(live8.data_ptr()), t, k,
+                                  h, ctypes.c_void_p(chain.data_ptr()))
+    got = out.cpu()
+    assert torch.equal(got.view(torch.int16), chain), "combine differs from the float32 FMA chain"
+    ref = O.ll_combine(pair_rows, topk, w, live)
+    err = (got.double() - ref).abs()
+    assert (err <= 1e-2 * ref.abs() + 1e-2 * ref.abs().mean()).all()
+    assert O.calc_diff(got, ref) < 1e-5
+
+
+def test_ll_config_full_size(rt):
+    """One GPU's share of EP=32 at 128 tokens x 7168, top-8 of 256 experts, seeded world."""
+    r, rank, t, h, k, e = 32, 11, 128, 7168, 8, 256
+    shape = rt.ll.LLShape(r, rank, e, t, h, k, O.ROW_FP8)
+    st = rt.ll.LowLatencyState(shape)
+    world = rt.lb.LoopbackWorld(r, rank, seed=2024)
+    world.synthesise(t, h, k, e)
+    x, topk = world.own_inputs()
+    st.dispatch_send(x, topk)
+    world.dispatch_from_peers(st)
+    st.dispatch_recv()
+    torch.cuda.synchronize()
+    # the oracle regenerates the same world from the seed
+    topk_all = O.synth_topk_idx(O.uniform_cdf(e), np.arange(r), t, k, 2024)
+    assert torch.equal(world.topk_idx_all.cpu(), topk_all)
+    x_all = O.synth_bf16_rows(np.arange(r * t, dtype=np.uint32), h, 2024).view(r, t, h)
+    assert torch.equal(world.x_all.cpu().view(torch.int16), x_all.view(torch.int16))
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
+    check_dispatch(st, want, O.ROW_FP8)
+    assert int(st.packed_recv_count.sum()) == int(((topk_all // (e // r)) == rank).sum())
+
+
+def test_skewed_routing_roundtrip(rt):
+    """Zipf(1.2) popularity, 1 % outlier rows, EP=64 with 4 local experts, hot experts past half their slots."""
+    r, rank, t, h, k, e = 64, 0, 256, 1024, 8, 256
+    shape = rt.ll.LLShape(r, rank, e, t, h, k, O.ROW_FP8)
+    st = rt.ll.LowLatencyState(shape)
+    world = rt.lb.LoopbackWorld(r, rank, seed=99)
+    world.synthesise(t, h, k, e, popularity="zipf", outlier_period=100)
+    x, topk = world.own_inputs()
+    st.dispatch_send(x, topk)
+    world.dispatch_from_peers(st)
+    st.dispatch_recv()
+    torch.cuda.synchronize()
+    topk_all = O.synth_topk_idx(O.zipf_cdf(e), np.arange(r), t, k, 99)
+    x_all = O.synth_bf16_rows(np.arange(r * t, dtype=np.uint32), h, 99, outlier_period=100).view(r, t, h)
+    assert torch.equal(world.topk_idx_all.cpu(), topk_all)
+    assert torch.equal(world.x_all.cpu().view(torch.int16), x_all.view(torch.int16))
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
+    check_dispatch(st, want, O.ROW_FP8)
+    assert int(st.packed_recv_count[0]) > r * t // 2, "the hottest expert should fill over half its slots"
+    # round trip with identity experts: combined == x * sum(w) within FP8 error
+    count = st.packed_recv_count.cpu()
+    el, n_slots = st.packed_recv_x.shape[:2]
+    y = torch.zeros((el, n_slots, h), dtype=torch.bfloat16)
+    for i in range(el):
+        n = int(count[i])
+        y[i, :n] = O.per_token_cast_back(st.packed_recv_x[i, :n].cpu(), st.packed_recv_scales[i, :n].cpu())
+    world.combine_from_peers(st, mode=0)
+    st.combine_send(y.cuda())
+    g = torch.Generator().manual_seed(1)
+    w = torch.softmax(torch.randn((t, k), generator=g), dim=-1)
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    st.combine_recv(topk, w.cuda(), out)
+    torch.cuda.synchronize()
+    diff = O.calc_diff(x_all[rank].float() * w.sum(1, keepdim=True), out.cpu())
+    assert diff < 9e-4, diff
+
+
+def test_ll_argument_errors(rt):
+    lib, capi = rt.capi.load(), rt.capi
+    z = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    # tokens beyond num_max_dispatch_tokens_per_rank
+    rc = lib.deepep_ll_dispatch_send(capi.ptr(z), capi.ptr(z), 9, 128, 2, 8, 2, 0, 8, 1, capi.ptr(z), capi.ptr(z),
+                                     capi.ptr(z), capi.ptr(z), capi.ptr(z), capi.ptr(z), 4096, s)
+    assert rc != 0 and "num_tokens <= max_tokens" in lib.deepep_last_error().decode()
+    # experts not divisible by ranks
+    rc = lib.deepep_ll_dispatch_recv(capi.ptr(z), capi.ptr(z), 128, 9, 2, 8, 1, capi.ptr(z), capi.ptr(z), capi.ptr(z),
+                                     capi.ptr(z), capi.ptr(z), None, s)
+    assert rc != 0 and "num_experts % num_ranks == 0" in lib.deepep_last_error().decode()
+    # workspace too small
+    rc = lib.deepep_ll_dispatch_send(capi.ptr(z), capi.ptr(z), 8, 128, 2, 8, 2, 0, 8, 1, capi.ptr(z), capi.ptr(z),
+                                     capi.ptr(z), capi.ptr(z), capi.ptr(z), capi.ptr(z), 16, s)
+    assert rc != 0 and "workspace_bytes" in lib.deepep_last_error().decode()
+    torch.cuda.synchronize()
+
+
+def test_empty_batch(rt):
+    """No tokens on this rank: counts come from the peers alone, combine returns nothing."""
+    r, rank, t, h, k, e = 4, 2, 6, 512, 2, 8
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=8, drop=0)
+    shape = rt.ll.LLShape(r, rank, e, t, h, k, O.ROW_FP8)
+    st = rt.ll.LowLatencyState(shape)
+    world = rt.lb.LoopbackWorld(r, rank)
+    world.set_inputs(x_all.cuda(), topk_all.cuda())
+    st.dispatch_send(x_all[rank, :0].cuda(), topk_all[rank, :0].cuda())
+    world.dispatch_from_peers(st)
+    st.dispatch_recv()
+    torch.cuda.synchronize()
+    xs, tks = list(x_all), list(topk_all)
+    xs[rank], tks[rank] = xs[rank][:0], tks[rank][:0]
+    want = O.ll_dispatch(xs, tks, rank, e, t, O.ROW_FP8)
+    check_dispatch(st, want, O.ROW_FP8)
+    assert (st.send_count == 0).all()

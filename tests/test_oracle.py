@@ -1,0 +1,353 @@
+"""Pins the CPU oracle: library routines, closed forms, brute force and invariants.
+
+No GPU.  A plausible mistake in the oracle (wrong rounding, dropped clamp, wrong
+segment order, transposed index) must fail at least one test here.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import deepep_oracle as O
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+# --------------------------------------------------------------------------
+# FP8
+# --------------------------------------------------------------------------
+def test_e4m3_encoder_matches_torch_cast_on_every_bf16_input(oracle_c):
+    # All 65536 bf16 bit patterns as float32, plus values that bf16 * float32
+    # scale products reach: dense sweep around every e4m3 rounding boundary.
+    bf = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+    grid = []
+    for b in range(256):
+        v = oracle_c.oracle_e4m3_decode(b)
+        if v == v:
+            grid.append(v)
+    grid = torch.tensor(sorted(set(grid)), dtype=torch.float32)
+    mids = (grid[1:] + grid[:-1]) / 2
+    near = torch.cat([torch.nextafter(mids, torch.tensor(float("inf"))), mids,
+                      torch.nextafter(mids, torch.tensor(-float("inf")))])
+    rnd = torch.empty(200000).uniform_(-448, 448, generator=torch.Generator().manual_seed(7))
+    tiny = torch.empty(50000).uniform_(-0.05, 0.05, generator=torch.Generator().manual_seed(8))
+    x = torch.cat([bf, grid, near, rnd, tiny])
+    x = x[torch.isfinite(x)].clamp(-448, 448).contiguous()
+    want = x.to(torch.float8_e4m3fn).view(torch.uint8)
+    got = torch.empty_like(want)
+    oracle_c.oracle_e4m3_encode_many(_ptr(x), _ptr(got), x.numel())
+    assert torch.equal(got, want)
+
+
+def test_e4m3_known_answers(oracle_c):
+    # Hand-checked bytes of the OCP format: 1-4-3, bias 7.
+    cases = [(0.0, 0x00), (-0.0, 0x80), (1.0, 0x38), (-1.0, 0xB8), (448.0, 0x7E), (-448.0, 0xFE), (2.0 ** -9, 0x01),
+             (2.0 ** -6, 0x08), (0.3, 42), (447.9, 126), (17.0, 88), (1.0625, 0x38), (1.1875, 0x3A), (2.0 ** -10, 0x00),
+             (3 * 2.0 ** -10, 0x02)]
+    for v, b in cases:
+        assert oracle_c.oracle_e4m3_encode(v) == b, (v, b)
+        assert torch.tensor([v]).to(torch.float8_e4m3fn).view(torch.uint8).item() == b, (v, b)
+
+
+def test_e4m3_decode_roundtrip(oracle_c):
+    for b in range(256):
+        v = oracle_c.oracle_e4m3_decode(b)
+        if v != v:
+            assert b & 0x7F == 0x7F
+            continue
+        assert oracle_c.oracle_e4m3_encode(v) == b
+        assert torch.tensor([b], dtype=torch.uint8).view(torch.float8_e4m3fn).float().item() == v
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_FP8_POW2, O.ROW_FP8_UE8M0])
+def test_torch_cast_matches_scalar_c_cast(oracle_c, fmt):
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn((37, 512), generator=g)
+    x[3] *= 100
+    x[5] = 0
+    x[7, :128] = 1e-6
+    x[9, 5] = 448 * 3.0
+    x[11] = -x[11].abs()
+    x = x.to(torch.bfloat16)
+    q, s = O.per_token_cast_to_fp8(x, round_scale=fmt != O.ROW_FP8, use_ue8m0=fmt == O.ROW_FP8_UE8M0)
+    q2 = torch.empty((37, 512), dtype=torch.uint8)
+    sb = 1 if fmt == O.ROW_FP8_UE8M0 else 4
+    s2 = torch.empty((37, 4 * sb), dtype=torch.uint8)
+    xb = x.view(torch.int16).contiguous()
+    oracle_c.oracle_per_token_cast(_ptr(xb), 37, 512, fmt, _ptr(q2), _ptr(s2))
+    assert torch.equal(q.view(torch.uint8), q2)
+    assert torch.equal(s.contiguous().view(torch.uint8).view(37, -1), s2)
+
+
+def test_cast_special_cases():
+    x = torch.zeros((2, 256), dtype=torch.bfloat16)
+    x[1, :128] = 2.0
+    x[1, 128:] = -3.0
+    x[1, 130] = 1.5
+    q, s = O.per_token_cast_to_fp8(x)
+    assert s[0, 0].item() == np.float32(1e-4) / np.float32(448.0)
+    assert (q[0].view(torch.uint8) == 0).all()
+    assert s[1, 0].item() == np.float32(2.0) / np.float32(448.0) and (q[1, :128].view(torch.uint8) == 0x7E).all()
+    assert (q[1, 128:130].view(torch.uint8) == 0xFE).all() and q[1, 130].float().item() == 224.0
+    # dequantised amax is exact
+    back = O.per_token_cast_back(q, s)
+    assert back[1, 0].item() == 2.0 and back[1, 128].item() == -3.0 and back[1, 130].item() == 1.5
+    # round_scale: scale is the smallest power of two >= amax/448; ue8m0 carries its exponent byte
+    q2, s2 = O.per_token_cast_to_fp8(x, round_scale=True)
+    for v, raw in zip(s2[1].tolist(), (2.0 / 448, 3.0 / 448)):
+        assert np.log2(v) == np.ceil(np.log2(raw)) and v >= raw > v / 2
+    x512 = torch.randn((3, 512)).to(torch.bfloat16)
+    _, sp = O.per_token_cast_to_fp8(x512, round_scale=True)
+    _, su = O.per_token_cast_to_fp8(x512, round_scale=True, use_ue8m0=True)
+    assert su.dtype == torch.int32 and su.shape == (3, 1)
+    assert torch.equal(su.view(torch.uint8).view(3, 4).to(torch.int32), (sp.view(torch.int32) >> 23) & 0xFF)
+    assert torch.equal(O.per_token_cast_back(_, su).float(), O.per_token_cast_back(_, sp).float())
+
+
+def test_pow2_ceil_exact():
+    s = torch.tensor([1.0, 1.0000001, 0.5, 0.75, 3.0, 2.0 ** -20, 2.0 ** -20 * 1.5, 2.2e-7])
+    want = torch.tensor([1.0, 2.0, 0.5, 1.0, 4.0, 2.0 ** -20, 2.0 ** -19, 2.0 ** -22])
+    assert torch.equal(O.pow2_ceil(s), want)
+
+
+def test_cast_error_bound_and_reference_torch_helper():
+    x = (torch.randn((64, 1024), generator=torch.Generator().manual_seed(5)) * 3).to(torch.bfloat16)
+    q, s = O.per_token_cast_to_fp8(x)
+    xv = x.view(64, -1, 128)
+    amax = xv.abs().float().amax(dim=2).view(64, -1).clamp(1e-4)
+    # IEEE division written with numpy, element by element, gives the same bytes
+    inv = torch.from_numpy(np.float32(448.0) / amax.numpy())
+    q_np = (xv.float() * inv.unsqueeze(2)).clamp(-448, 448).to(torch.float8_e4m3fn).view(64, 1024)
+    assert torch.equal(q.view(torch.uint8), q_np.view(torch.uint8))
+    assert torch.equal(s, torch.from_numpy(amax.numpy() / np.float32(448.0)))
+    back = O.per_token_cast_back(q, s).float()
+    err = (back - x.float()).abs().view(64, -1, 128)
+    # half an e4m3 step at the top binade is 16 (scaled units); the bf16 round of the result adds 2^-9 relative
+    assert (err <= amax.unsqueeze(2) * (16 / 448.0 + 2.0 ** -8)).all()
+    # The reference's torch helper (reciprocal-multiply) has the same scales and differs from
+    # the kernel's division in well under 1 % of bytes, each by one e4m3 code.
+    qh, sh = O.per_token_cast_to_fp8_torch_helper(x)
+    assert torch.equal(sh, s)
+    a, b = q.view(torch.uint8).to(torch.int32), qh.view(torch.uint8).to(torch.int32)
+    diff = a != b
+    assert diff.float().mean().item() < 0.01
+    assert ((a - b).abs()[diff] == 1).all()
+
+
+# --------------------------------------------------------------------------
+# Layout
+# --------------------------------------------------------------------------
+def _brute_layout(topk, num_experts, num_ranks):
+    t, k = topk.shape
+    epr = num_experts // num_ranks
+    pe = [0] * num_experts
+    pr = [0] * num_ranks
+    pn = [0] * (num_ranks // 8)
+    is_in = [[False] * num_ranks for _ in range(t)]
+    for i in range(t):
+        for j in range(k):
+            e = int(topk[i, j])
+            if e >= 0:
+                pe[e] += 1
+                is_in[i][e // epr] = True
+        for r in range(num_ranks):
+            pr[r] += is_in[i][r]
+        for n in range(num_ranks // 8):
+            pn[n] += any(is_in[i][8 * n:8 * n + 8])
+    return pr, pn, pe, is_in
+
+
+@pytest.mark.parametrize("t,k,e,r", [(1, 1, 2, 2), (13, 3, 16, 4), (40, 8, 64, 16), (0, 4, 8, 8), (9, 6, 48, 24)])
+def test_layout_matches_brute_force(t, k, e, r):
+    g = torch.Generator().manual_seed(t * 31 + e)
+    topk = torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(t)]) if t else torch.zeros((0, k), dtype=torch.int64)
+    if t > 2:
+        topk[1, 0] = -1
+        topk[2, :] = -1
+    pr, pn, pe, is_in = O.get_dispatch_layout(topk, e, r)
+    bpr, bpn, bpe, bis = _brute_layout(topk, e, r)
+    assert pr.tolist() == bpr and pe.tolist() == bpe and is_in.tolist() == bis
+    if r > 8 and r % 8 == 0:
+        assert pn.tolist() == bpn
+    else:
+        assert pn is None
+    # closed forms of tests/test_intranode.py:41-58
+    for i in range(e):
+        assert pe[i].item() == (topk == i).sum().item()
+
+
+def test_routing_sort_and_channel_prefix():
+    g = torch.Generator().manual_seed(3)
+    is_in = torch.rand((53, 6), generator=g) < 0.4
+    ids, counts, cumsum, total = O.moe_routing_sort(is_in)
+    assert total == int(is_in.sum()) and counts.tolist() == is_in.sum(0).tolist()
+    for r in range(6):
+        seg = ids[cumsum[r]:cumsum[r + 1]].tolist()
+        assert seg == [t for t in range(53) if is_in[t, r]]
+    cpm = O.channel_prefix_matrix(is_in, 10)
+    per = -(-53 // 10)
+    for d in range(6):
+        run = 0
+        for c in range(10):
+            b = min(per * c, 53)
+            run += sum(bool(is_in[t, d]) for t in range(b, min(b + per, 53)))
+            assert cpm[d, c].item() == run
+    assert cpm[:, -1].tolist() == counts.tolist()
+
+
+# --------------------------------------------------------------------------
+# Dispatch / combine
+# --------------------------------------------------------------------------
+def _world(r, t, h, k, e, seed, drop=5):
+    g = torch.Generator().manual_seed(seed)
+    xs = [torch.randn((t, h), generator=g).to(torch.bfloat16) for _ in range(r)]
+    tk = [torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(t)]) for _ in range(r)]
+    for _ in range(drop):
+        s, i, j = [int(torch.randint(0, n, (1,), generator=g)) for n in (r, t, k)]
+        tk[s][i, j] = -1
+    return xs, tk
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16, O.ROW_FP8_UE8M0])
+def test_vectorised_dispatch_equals_serial_restatement(fmt):
+    xs, tk = _world(4, 8, 512, 3, 16, seed=2)
+    for rank in range(4):
+        a = O.ll_dispatch(xs, tk, rank, 16, 8, fmt)
+        b = O._serial_dispatch(xs, tk, rank, 16, 8, fmt)
+        for key in a:
+            assert torch.equal(a[key], b[key]), (rank, key)
+
+
+def test_dispatch_invariants_of_reference_test():
+    # tests/test_low_latency.py:59-60,119-147: x = rank-128 with the token index in the last 128 columns.
+    r, t, h, k, e = 4, 16, 256, 4, 16
+    g = torch.Generator().manual_seed(9)
+    xs = []
+    for rank in range(r):
+        x = torch.ones((t, h), dtype=torch.bfloat16) * (rank - 128)
+        x[:, -128:] = torch.arange(t).to(torch.bfloat16).view(-1, 1)
+        xs.append(x)
+    tk = [torch.topk(torch.randn((t, e), generator=g).abs() + 1, k, dim=-1)[1] for _ in range(r)]
+    for s in range(r):
+        tk[s][s, 0] = -1
+    all_tk = torch.stack(tk)
+    for rank in range(r):
+        out = O.ll_dispatch(xs, tk, rank, e, t, O.ROW_FP8)
+        epr = e // r
+        for i in range(epr):
+            expert = rank * epr + i
+            n = out["packed_recv_count"][i].item()
+            lr = out["packed_recv_layout_range"][i]
+            assert n == (lr & 0xFFFFFFFF).sum().item() == (all_tk == expert).sum().item()
+            q = out["packed_recv_x"][i, :n].view(torch.float8_e4m3fn)
+            sc = out["packed_recv_scales"][i, :n].view(torch.float32)
+            recv = O.per_token_cast_back(q, sc).float()
+            assert torch.equal(recv[:, :-128].amin(-1), recv[:, :-128].amax(-1))
+            src = out["packed_recv_src_info"][i, :n]
+            assert (recv[:, -128:] - src.view(-1, 1) % t).sum().item() == 0
+            for j in range(r):
+                begin, cnt = (lr[j] >> 32).item(), (lr[j] & 0xFFFFFFFF).item()
+                assert cnt == (all_tk[j] == expert).sum().item()
+                assert (recv[begin:begin + cnt, :-128] - j + 128).sum().item() == 0
+                assert src[begin:begin + cnt].tolist() == sorted(src[begin:begin + cnt].tolist())
+
+
+def test_route_slots_and_staged_rows():
+    xs, tk = _world(2, 10, 256, 3, 8, seed=4, drop=3)
+    send_count, pair_slot = O.route(tk[0], 8, 10)
+    seen = {}
+    for t in range(10):
+        for k in range(3):
+            e = int(tk[0][t, k])
+            if e < 0:
+                assert pair_slot[t, k] == -1
+                continue
+            assert pair_slot[t, k] == seen.get(e, 0)
+            seen[e] = seen.get(e, 0) + 1
+    assert send_count.tolist() == [seen.get(e, 0) for e in range(8)]
+    sc, ps, experts, slots, rows = O.staged_rows(xs[0], tk[0], 1, 8, 10, O.ROW_FP8)
+    assert rows.shape[1] == O.row_stride(256, O.ROW_FP8) == 256 + 16 + 16
+    tail = rows[:, -16:].contiguous().view(torch.int32)
+    assert (tail[:, 2] == 1).all() and (tail[:, 3] == 0).all()
+    q, s = O.per_token_cast_to_fp8(xs[0])
+    assert torch.equal(rows[:, :256], q.view(torch.uint8)[tail[:, 0].long()])
+    assert torch.equal(rows[:, 256:264].contiguous().view(torch.float32), s[tail[:, 0].long()])
+
+
+def test_combine_closed_form_and_chain(oracle_c):
+    t, k, h = 12, 5, 256
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn((t, h), generator=g).to(torch.bfloat16)
+    w = torch.randn((t, k), generator=g).abs()
+    topk = torch.randint(0, 32, (t, k), generator=g)
+    topk[0, 1] = -1
+    topk[3, :] = -1
+    live = topk >= 0
+    rows = x.unsqueeze(1).expand(t, k, h).contiguous()
+    ref = O.ll_combine(rows, topk, w)
+    # tests/test_low_latency.py:181: combined == x * sum of live weights
+    want = x.double() * (w.double() * live.double()).sum(1, keepdim=True)
+    assert torch.allclose(ref, want, rtol=1e-12, atol=0)
+    assert (ref[3] == 0).all()
+    chain = O.ll_combine_f32_chain(rows, w, live)
+    out = torch.empty((t, h), dtype=torch.int16)
+    live8 = live.to(torch.uint8).contiguous()
+    oracle_c.oracle_combine_chain(_ptr(rows.view(torch.int16)), _ptr(w.contiguous()), _ptr(live8), t, k, h, _ptr(out))
+    assert torch.equal(out.view(torch.bfloat16), chain)
+    rel = (chain.double() - ref).abs() / ref.abs().clamp(min=1e-2)
+    assert rel.max().item() < 1e-2
+    assert O.calc_diff(chain, ref) < 1e-5
+    # a random-output case: the chain is within bf16 rounding of the float64 sum
+    rows2 = torch.randn((t, k, h), generator=g).to(torch.bfloat16)
+    ref2 = O.ll_combine(rows2, topk, w)
+    chain2 = O.ll_combine_f32_chain(rows2, w, live)
+    assert ((chain2.double() - ref2).abs() <= ref2.abs() * 2 ** -8 + 1e-6).all()
+
+
+def test_size_hint_hand_values():
+    # SURVEY hand computation for (128, 7168, 32, 256)
+    assert O.get_low_latency_rdma_size_hint(128, 7168, 32, 256) == 1908410496
+    # tiny case by hand: M=1,H=128,E=2: dmsg=16+256=272, cmsg=4+256=260; send=max(272,520)=520; recv=max(544,520)=544
+    # sig=128 -> total = 1040+1088+256 = 2384 -> (2384+128)//128*128 = 2432
+    assert O.get_low_latency_rdma_size_hint(1, 128, 2, 2) == 2432
+    assert O.row_stride(7168, O.ROW_FP8) == 7408 and O.row_stride(7168, O.ROW_BF16) == 14352
+    assert O.row_stride(7168, O.ROW_FP8_UE8M0) == 7168 + 64 + 16
+
+
+# --------------------------------------------------------------------------
+# Seeded world: numpy restatement vs the C one, and distribution sanity
+# --------------------------------------------------------------------------
+def test_seeded_rows_numpy_equals_c(oracle_c):
+    for x in (0, 1, 0xDEADBEEF, 0xFFFFFFFF, 12345):
+        assert int(O.mix32(x)) == oracle_c.oracle_mix32(x)
+    keys = np.array([0, 1, 2, 99, 2 ** 31, 2 ** 32 - 1, 777], dtype=np.uint32)
+    for period in (0, 3):
+        a = O.synth_bf16_rows(keys, 384, seed=42, outlier_period=period)
+        b = torch.empty((len(keys), 384), dtype=torch.int16)
+        oracle_c.oracle_synth_bf16_rows(keys.ctypes.data_as(ctypes.c_void_p), len(keys), 384, 42, period, _ptr(b))
+        assert torch.equal(a.view(torch.int16), b)
+    big = O.synth_bf16_rows(np.arange(64, dtype=np.uint32), 7168, seed=1).float()
+    assert abs(big.mean().item()) < 0.01 and abs(big.std().item() - 1.0) < 0.02
+    hot = O.synth_bf16_rows(np.arange(4000, dtype=np.uint32), 8, seed=1, outlier_period=100).float()
+    frac = ((hot.abs().amax(1)) > 20).float().mean().item()
+    assert 0.004 < frac < 0.02
+
+
+@pytest.mark.parametrize("cdf_name", ["uniform", "zipf"])
+def test_seeded_topk_numpy_equals_c(oracle_c, cdf_name):
+    e, k, t = 64, 8, 50
+    cdf = O.uniform_cdf(e) if cdf_name == "uniform" else O.zipf_cdf(e)
+    assert cdf[-1] == 0xFFFFFFFF and (np.diff(cdf.astype(np.int64)) >= 0).all()
+    ranks = np.array([0, 3, 5], dtype=np.int32)
+    a = O.synth_topk_idx(cdf, ranks, t, k, seed=17)
+    b = torch.empty((3, t, k), dtype=torch.int64)
+    oracle_c.oracle_synth_topk_idx(cdf.ctypes.data_as(ctypes.c_void_p), ranks.ctypes.data_as(ctypes.c_void_p), 3, t, k,
+                                   e, 17, _ptr(b))
+    assert torch.equal(a, b)
+    srt = torch.sort(a, dim=-1).values
+    assert (srt[..., 1:] != srt[..., :-1]).all() and a.min() >= 0 and a.max() < e
+    if cdf_name == "zipf":
+        assert (a == 0).any(-1).float().mean() > 0.5  # the hottest expert is in most tokens
