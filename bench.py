@@ -108,21 +108,20 @@ def main():
     wall = time.perf_counter() - wall0
     us_per_step = ev0.elapsed_time(ev1) * 1e3 / args.steps
 
-    # per entry point, events around every call
+    # per entry point: the same call `steps` times back to back between two events.  Consecutive
+    # launches on one stream leave well under a microsecond between kernels on this GPU, so the
+    # mean is the kernel's duration (the rocprofv3 summary under profiles/ is the cross-check).
     per_call = {}
     for name, fn in calls.items():
-        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-                 for _ in range(args.steps)]
-        for a, b in pairs:
-            step_before = [f for n2, f in calls.items() if n2 != name]
-            a.record()
+        for _ in range(10):
             fn()
-            b.record()
-            for f in step_before[:1]:
-                f()  # keep the stream busy so the next start event is not an idle-queue timestamp
         torch.cuda.synchronize()
-        ts = sorted(a.elapsed_time(b) * 1e3 for a, b in pairs)
-        per_call[name] = sum(ts) / len(ts)
+        ev0.record()
+        for _ in range(args.steps):
+            fn()
+        ev1.record()
+        torch.cuda.synchronize()
+        per_call[name] = ev0.elapsed_time(ev1) * 1e3 / args.steps
 
     graph_us = None
     if not args.no_graph:

@@ -19,7 +19,7 @@ namespace deepep {
 // ---------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ll_combine_send_kernel(
     const uint8_t* __restrict__ x, const int64_t* __restrict__ layout_range, int hidden, int num_local_experts,
-    int num_ranks, int rank, int max_tokens, uint8_t* __restrict__ combine_staging,
+    int num_ranks, int rank, int max_tokens, int parts, uint8_t* __restrict__ combine_staging,
     uint8_t* __restrict__ combine_send_slots) {
     extern __shared__ int32_t flat[];  // [num_segments + 1] then begin[num_segments]
     __shared__ int32_t wave_totals[4];
@@ -41,9 +41,10 @@ __global__ __launch_bounds__(256) void ll_combine_send_kernel(
     const int64_t row_bytes = int64_t(hidden) * 2;
     const int num_vec = int(row_bytes / 16);
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
-    const int waves_total = gridDim.x * 4;
+    const int64_t waves_total = int64_t(gridDim.x) * 4;
 
-    for (int row = blockIdx.x * 4 + w; row < total_rows; row += waves_total) {
+    for (int64_t item = blockIdx.x * 4 + w; item < int64_t(total_rows) * parts; item += waves_total) {
+        const int row = int(item / parts), part = int(item - int64_t(row) * parts);
         const int seg = __builtin_amdgcn_readfirstlane(find_segment(flat, num_segments, row));
         const int j = row - __builtin_amdgcn_readfirstlane(flat[seg]);
         const int le = seg / num_ranks;
@@ -58,7 +59,9 @@ __global__ __launch_bounds__(256) void ll_combine_send_kernel(
             dst = combine_send_slots + (int64_t(seg) * max_tokens + j) * row_bytes;
         else
             continue;
-        wave_copy_vec16(src, dst, num_vec, lane);
+        int v_begin, v_end;
+        row_part_range(num_vec, parts, part, v_begin, v_end);
+        wave_copy_vec16(src, dst, v_begin, v_end, lane);
     }
 }
 
@@ -147,13 +150,14 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
     const int num_local_experts = num_experts / num_ranks;
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     EP_HOST_ASSERT(max_rows < (int64_t(1) << 31));
-    int64_t blocks = (max_rows + 3) / 4;
-    const int64_t cap = max_rows > (int64_t(1) << 18) ? 4096 : 512;
+    const int parts = choose_row_parts(max_rows, int64_t(hidden) * 2);
+    int64_t blocks = (max_rows * parts + 3) / 4;
+    const int64_t cap = max_rows > (int64_t(1) << 18) ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(2 * num_experts + 1) * sizeof(int32_t);
     ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, lds, reinterpret_cast<hipStream_t>(stream)>>>(
         reinterpret_cast<const uint8_t*>(x), layout_range, hidden, num_local_experts, num_ranks, rank,
-        num_max_dispatch_tokens_per_rank, reinterpret_cast<uint8_t*>(combine_staging),
+        num_max_dispatch_tokens_per_rank, parts, reinterpret_cast<uint8_t*>(combine_staging),
         reinterpret_cast<uint8_t*>(combine_send_slots));
     EP_LAUNCH_CHECK();
     return 0;

@@ -15,6 +15,8 @@
 #include "common.hpp"
 #include "quant.hpp"
 #include "segments.hpp"
+#include <cstdlib>
+
 #include "../../include/deepep_hip.h"
 
 namespace deepep {
@@ -146,94 +148,173 @@ __global__ __launch_bounds__(256) void ll_route_scan_kernel(int n, int num_exper
 }
 
 // ---------------------------------------------------------------------
-// Fused quantise + pack.  One wave = one (source, token, 1 KiB output piece).
+// Fused quantise + pack.  A workgroup owns one token (of one source); each of
+// its waves owns one (1 KiB output piece, share of the K selections).
 // FP8 formats: the piece is 8 scale groups (1024 channels, 2 KiB of bf16 in);
 // each 8-lane cluster owns a group, each lane 16 channels.  The quantised
 // 16 bytes stay in registers and are stored once per selection — the row is
 // read and quantised once however many experts it goes to
 // (reference idea: csrc/kernels/coop_dispatch_send.cuh:572-607).
+//
+// Per-selection bookkeeping (slot, destination row address, row tail,
+// pair_slot) is done once per token by the first K threads and handed to the
+// waves through LDS, so a wave's own work is: two loads, the DPP quantise,
+// and per selection one 8-byte LDS read and two stores.
+//
+// kFusedRoute (small batches): no route kernel runs first.  While the row
+// loads are in flight the workgroup ranks the token's selections itself: its
+// threads sweep the (token,k) entries before the token, one entry per thread
+// per step, and bump an LDS counter for every entry that names one of the
+// token's experts.  The sweep is O(T*K) per token, which at T*K <= 2048 is one
+// or two loads per thread and costs less than a dependent launch.  The
+// per-expert totals come from one extra row of workgroups (blockIdx.y == T),
+// an LDS histogram per source.
 // ---------------------------------------------------------------------
-template <int kFmt>
-__global__ __launch_bounds__(256) void ll_send_kernel(
+constexpr int kMaxTopk = 64;
+constexpr int kFusedMaxEntries = 2048;
+constexpr int kSendMaxWaves = 16;
+
+template <int kFmt, bool kFusedRoute>
+__global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(
     const uint8_t* __restrict__ x, const int64_t* __restrict__ topk_idx,
-    const int32_t* __restrict__ src_ranks, int num_src, int num_tokens, int hidden, int num_topk,
-    int num_experts, int num_ranks, int rank, int max_tokens, int pieces_per_row,
-    int64_t scratch_stride, const uint8_t* __restrict__ scratch_base,
-    uint8_t* __restrict__ recv_staging, uint8_t* __restrict__ send_slots, int32_t* __restrict__ pair_slot) {
-    const int lane = lane_id();
-    const int64_t item = int64_t(blockIdx.x) * (blockDim.x / kWave) + wave_in_block();
-    const int64_t num_items = int64_t(num_src) * num_tokens * pieces_per_row;
-    if (item >= num_items) return;
-    const int piece = int(item % pieces_per_row);
-    const int64_t row_id = item / pieces_per_row;  // b * T + t
-    const int b = int(row_id / num_tokens);
-    const int t = int(row_id - int64_t(b) * num_tokens);
+    const int32_t* __restrict__ src_ranks, int num_tokens, int hidden, int num_topk, int num_experts,
+    int num_ranks, int rank, int max_tokens, int pieces_per_row, int split_log2, uint32_t rank_of_expert_magic,
+    int64_t scratch_stride, const uint8_t* __restrict__ scratch_base, uint8_t* __restrict__ recv_staging,
+    uint8_t* __restrict__ send_slots, int32_t* __restrict__ pair_slot, int32_t* __restrict__ recv_count,
+    int32_t* __restrict__ send_count) {
+    extern __shared__ int32_t lds_hist[];  // [E], counting workgroups only
+    __shared__ int32_t sel_expert[kMaxTopk];
+    __shared__ int32_t sel_count[kMaxTopk];
+    __shared__ uint64_t sel_row[kMaxTopk];
+    const int lane = lane_id(), tid = threadIdx.x;
+    const int b = blockIdx.z, t = blockIdx.y;
+    const int n = num_tokens * num_topk;
     const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
-    const int experts_per_rank = num_experts / num_ranks;
+    const int64_t* my_topk = topk_idx + int64_t(b) * n;
+
+    if constexpr (kFusedRoute) {
+        if (t == num_tokens) {  // the counting row of the grid: one workgroup per source
+            if (blockIdx.x != 0) return;
+            for (int j = tid; j < num_experts; j += blockDim.x) lds_hist[j] = 0;
+            __syncthreads();
+            for (int i = tid; i < n; i += blockDim.x) {
+                const int64_t v = my_topk[i];
+                if (v >= 0 && v < num_experts) atomicAdd(&lds_hist[int(v)], 1);
+            }
+            __syncthreads();
+            for (int e = tid; e < num_experts; e += blockDim.x)
+                emit_expert_count(e, lds_hist[e], num_experts, num_ranks, rank, src_rank, max_tokens, recv_count,
+                                  send_count);
+            return;
+        }
+    }
+
+    const int item = int(blockIdx.x) * int(blockDim.x >> 6) + wave_in_block();
+    const int split = 1 << split_log2;
+    const bool wave_live = item < (pieces_per_row << split_log2);
+    const int part = item & (split - 1);
+    const int piece = item >> split_log2;
+    const int64_t row_id = int64_t(b) * num_tokens + t;
+    const int entry0 = t * num_topk;
 
     const int64_t data_bytes = row_data_bytes(hidden, kFmt);
     const int64_t data_pad = align16(data_bytes);
     const int64_t scale_pad = align16(row_scale_bytes(hidden, kFmt));
     const int64_t stride = data_pad + scale_pad + kRowTailBytes;
 
-    // ---- load + quantise this wave's piece ------------------------------
-    u32x4 payload = {0u, 0u, 0u, 0u};
-    uint32_t scale_bits = 0;
+    // ---- issue this wave's row loads ------------------------------------
+    u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
     bool lane_live;
     int group = 0;
     if constexpr (kFmt == kRowBF16) {
         const int64_t off = int64_t(piece) * 1024 + lane * 16;
-        lane_live = off < data_bytes;
-        if (lane_live) payload = *reinterpret_cast<const u32x4*>(x + row_id * data_bytes + off);
+        lane_live = wave_live && off < data_bytes;
+        if (lane_live) lo = *reinterpret_cast<const u32x4*>(x + row_id * data_bytes + off);
     } else {
         group = piece * 8 + (lane >> 3);
-        lane_live = group < hidden / kGroup;
-        u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
+        lane_live = wave_live && group < hidden / kGroup;
         if (lane_live) {
             const uint8_t* src = x + (row_id * hidden + int64_t(group) * kGroup + (lane & 7) * 16) * 2;
             lo = *reinterpret_cast<const u32x4*>(src);
             hi = *reinterpret_cast<const u32x4*>(src + 16);
         }
-        payload = quantise_16<kFmt>(lo, hi, scale_bits);
     }
 
-    // ---- one store per selection ----------------------------------------
-    const int n = num_tokens * num_topk;
-    const int32_t* pair_rank = reinterpret_cast<const int32_t*>(scratch_base + int64_t(b) * scratch_stride);
-    const int32_t* chunk_base =
-        reinterpret_cast<const int32_t*>(scratch_base + int64_t(b) * scratch_stride + align256(int64_t(n) * 4 + 4));
-    const int64_t entry0 = int64_t(t) * num_topk;
-#pragma unroll 8
-    for (int k = 0; k < num_topk; ++k) {
-        const int in_chunk = pair_rank[entry0 + k];
-        int slot = -1;
+    // ---- per-selection bookkeeping, once per token --------------------------
+    int my_expert = -1, my_slot = -1;  // threads 0..K-1: selection k = tid
+    if (tid < num_topk) {
+        const int64_t v = my_topk[entry0 + tid];
+        if (v >= 0 && v < num_experts) my_expert = int(v);
+        if constexpr (kFusedRoute) {
+            sel_expert[tid] = my_expert;
+            sel_count[tid] = 0;
+        } else {
+            const int32_t* pair_rank = reinterpret_cast<const int32_t*>(scratch_base + int64_t(b) * scratch_stride);
+            const int32_t* chunk_base = reinterpret_cast<const int32_t*>(
+                scratch_base + int64_t(b) * scratch_stride + align256(int64_t(n) * 4 + 4));
+            const int in_chunk = pair_rank[entry0 + tid];
+            if (in_chunk >= 0 && my_expert >= 0)
+                my_slot = in_chunk + chunk_base[((entry0 + tid) / kRouteChunk) * num_experts + my_expert];
+        }
+    }
+    if constexpr (kFusedRoute) {
+        __syncthreads();
+        for (int i = tid; i < entry0; i += blockDim.x) {
+            const int64_t v = my_topk[i];
+            if (v < 0 || v >= num_experts) continue;
+            for (int k = 0; k < num_topk; ++k)
+                if (int(v) == sel_expert[k]) atomicAdd(&sel_count[k], 1);
+        }
+        __syncthreads();
+        if (tid < num_topk && my_expert >= 0) {
+            my_slot = sel_count[tid];
+            for (int k2 = 0; k2 < tid; ++k2)  // the same expert named earlier in this token
+                if (sel_expert[k2] == my_expert) my_slot += 1;
+        }
+    }
+    if (tid < num_topk) {
+        if (my_slot >= max_tokens) my_slot = -1;
         uint8_t* row = nullptr;
-        if (in_chunk >= 0) {
-            const int e = int(topk_idx[int64_t(b) * n + entry0 + k]);
-            slot = in_chunk + chunk_base[((entry0 + k) / kRouteChunk) * num_experts + e];
-            if (slot >= max_tokens) {
-                slot = -1;
-            } else {
-                const int dst_rank = e / experts_per_rank;
-                const int local = e - dst_rank * experts_per_rank;
-                if (dst_rank == rank)
-                    row = recv_staging + ((int64_t(local) * num_ranks + src_rank) * max_tokens + slot) * stride;
-                else if (send_slots != nullptr)
-                    row = send_slots + (int64_t(e) * max_tokens + slot) * stride;
+        if (my_slot >= 0) {
+            // my_expert / E_l by multiply-high; magic 0 stands for E_l == 1
+            const int dst_rank = rank_of_expert_magic != 0
+                                     ? int(__umulhi(uint32_t(my_expert), rank_of_expert_magic))
+                                     : my_expert;
+            const int local = my_expert - dst_rank * (num_experts / num_ranks);
+            if (dst_rank == rank)
+                row = recv_staging + ((int64_t(local) * num_ranks + src_rank) * max_tokens + my_slot) * stride;
+            else if (send_slots != nullptr)
+                row = send_slots + (int64_t(my_expert) * max_tokens + my_slot) * stride;
+        }
+        sel_row[tid] = reinterpret_cast<uint64_t>(row);
+        if (blockIdx.x == 0) {
+            if (pair_slot != nullptr) pair_slot[entry0 + tid] = my_slot;
+            if (row != nullptr) {
+                u32x4 tail = {uint32_t(t), uint32_t(tid), uint32_t(src_rank), 0u};
+                *reinterpret_cast<u32x4*>(row + data_pad + scale_pad) = tail;
             }
         }
-        if (pair_slot != nullptr && piece == 0 && lane == 0) pair_slot[entry0 + k] = slot;
+    }
+    __syncthreads();
+    if (!wave_live) return;
+
+    // ---- quantise, then one store per selection ---------------------------
+    u32x4 payload = lo;
+    uint32_t scale_bits = 0;
+    if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
+    const int64_t lane_off = int64_t(piece) * 1024 + lane * 16;
+    for (int k = part; k < num_topk; k += split) {
+        const uint64_t row_bits = sel_row[k];
+        const uint32_t lo32 = __builtin_amdgcn_readfirstlane(uint32_t(row_bits));
+        const uint32_t hi32 = __builtin_amdgcn_readfirstlane(uint32_t(row_bits >> 32));
+        uint8_t* row = reinterpret_cast<uint8_t*>((uint64_t(hi32) << 32) | lo32);
         if (row == nullptr) continue;
-        if (lane_live) *reinterpret_cast<u32x4*>(row + int64_t(piece) * 1024 + lane * 16) = payload;
+        if (lane_live) *reinterpret_cast<u32x4*>(row + lane_off) = payload;
         if constexpr (kFmt == kRowFP8 || kFmt == kRowFP8Pow2) {
             if (lane_live && (lane & 7) == 0)
                 *reinterpret_cast<uint32_t*>(row + data_pad + int64_t(group) * 4) = scale_bits;
         } else if constexpr (kFmt == kRowFP8UE8M0) {
             if (lane_live && (lane & 7) == 0) row[data_pad + group] = uint8_t(scale_bits >> 23);
-        }
-        if (piece == 0 && lane == 0) {
-            u32x4 tail = {uint32_t(t), uint32_t(k), uint32_t(src_rank), 0u};
-            *reinterpret_cast<u32x4*>(row + data_pad + scale_pad) = tail;
         }
     }
 }
@@ -248,7 +329,7 @@ __global__ __launch_bounds__(256) void ll_send_kernel(
 // ---------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ll_recv_kernel(
     const uint8_t* __restrict__ recv_staging, const int32_t* __restrict__ recv_count, int hidden,
-    int num_local_experts, int num_ranks, int max_tokens, int fmt, uint8_t* __restrict__ packed_x,
+    int num_local_experts, int num_ranks, int max_tokens, int fmt, int parts, uint8_t* __restrict__ packed_x,
     uint8_t* __restrict__ packed_scales, int32_t* __restrict__ src_info, int64_t* __restrict__ layout_range,
     int32_t* __restrict__ packed_count, int32_t* __restrict__ stats) {
     extern __shared__ int32_t flat[];  // [num_segments + 1]
@@ -284,16 +365,20 @@ __global__ __launch_bounds__(256) void ll_recv_kernel(
     const int64_t scale_bytes = row_scale_bytes(hidden, fmt);
     const int64_t stride = data_pad + align16(scale_bytes) + kRowTailBytes;
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
-    const int waves_total = gridDim.x * 4;
-
-    for (int row = blockIdx.x * 4 + w; row < total_rows; row += waves_total) {
+    const int64_t waves_total = int64_t(gridDim.x) * 4;
+    const int num_vec = int(data_bytes / 16);
+    for (int64_t item = blockIdx.x * 4 + w; item < int64_t(total_rows) * parts; item += waves_total) {
+        const int row = int(item / parts), part = int(item - int64_t(row) * parts);
         const int seg = __builtin_amdgcn_readfirstlane(find_segment(flat, num_segments, row));
         const int j = row - __builtin_amdgcn_readfirstlane(flat[seg]);
         const int le = seg / num_ranks;
         const int64_t slot = int64_t(row) - __builtin_amdgcn_readfirstlane(flat[le * num_ranks]);
         const uint8_t* src = recv_staging + (int64_t(seg) * max_tokens + j) * stride;
         const int64_t out_row = int64_t(le) * slots_per_expert + slot;
-        wave_copy_vec16(src, packed_x + out_row * data_bytes, int(data_bytes / 16), lane);
+        int v_begin, v_end;
+        row_part_range(num_vec, parts, part, v_begin, v_end);
+        wave_copy_vec16(src, packed_x + out_row * data_bytes, v_begin, v_end, lane);
+        if (part != parts - 1) continue;  // the last part is the shortest: it also carries scales and source index
         if (packed_scales != nullptr && scale_bytes > 0) {
             const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src + data_pad);
             uint32_t* d32 = reinterpret_cast<uint32_t*>(packed_scales + out_row * scale_bytes);
@@ -309,7 +394,7 @@ __global__ __launch_bounds__(256) void ll_recv_kernel(
 // ---------------------------------------------------------------------
 static int check_ll_shape(int num_tokens, int hidden, int num_topk, int num_experts, int num_ranks, int rank,
                           int max_tokens, int row_format) {
-    EP_HOST_ASSERT(num_tokens >= 0 && hidden > 0 && num_topk > 0);
+    EP_HOST_ASSERT(num_tokens >= 0 && hidden > 0 && num_topk > 0 && num_topk <= kMaxTopk);
     EP_HOST_ASSERT(hidden % 128 == 0);
     EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
     EP_HOST_ASSERT(rank >= 0 && rank < num_ranks);
@@ -319,6 +404,14 @@ static int check_ll_shape(int num_tokens, int hidden, int num_topk, int num_expe
     EP_HOST_ASSERT(int64_t(num_tokens) * num_topk < (int64_t(1) << 30));
     EP_HOST_ASSERT(num_experts <= 4096);
     return 0;
+}
+
+static int send_split_override() {
+    static const int v = [] {
+        const char* s = getenv("DEEPEP_SEND_SPLIT");
+        return s != nullptr ? atoi(s) : 0;
+    }();
+    return v;
 }
 
 static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_t* src_ranks, int num_src,
@@ -331,39 +424,62 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
     const int n = num_tokens * num_topk;
     uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
-    const size_t lds = size_t(kRouteWaves) * num_experts * sizeof(int32_t);
-    EP_HOST_ASSERT(lds <= 64 * 1024);
+    const bool fused = n <= kFusedMaxEntries;
 
-    // Route.  Counts must be published even for an empty batch of tokens.
-    dim3 rgrid(rs.num_chunks, num_src);
-    if (rs.num_chunks == 1) {
-        ll_route_rank_kernel<true><<<rgrid, kRouteChunk, lds, stream>>>(
-            topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count,
-            send_count);
-        EP_LAUNCH_CHECK();
-    } else {
-        ll_route_rank_kernel<false><<<rgrid, kRouteChunk, lds, stream>>>(
-            topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count,
-            send_count);
-        EP_LAUNCH_CHECK();
-        dim3 sgrid((num_experts + 255) / 256, num_src);
-        ll_route_scan_kernel<<<sgrid, 256, 0, stream>>>(n, num_experts, num_ranks, rank, src_ranks, max_tokens,
-                                                        rs.num_chunks, rs.bytes, ws, recv_count, send_count);
-        EP_LAUNCH_CHECK();
+    if (!fused) {
+        // Route kernels.  Counts are published even for an empty batch of tokens.
+        const size_t lds = size_t(kRouteWaves) * num_experts * sizeof(int32_t);
+        EP_HOST_ASSERT(lds <= 64 * 1024);
+        dim3 rgrid(rs.num_chunks, num_src);
+        if (rs.num_chunks == 1) {
+            ll_route_rank_kernel<true><<<rgrid, kRouteChunk, lds, stream>>>(
+                topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count,
+                send_count);
+            EP_LAUNCH_CHECK();
+        } else {
+            ll_route_rank_kernel<false><<<rgrid, kRouteChunk, lds, stream>>>(
+                topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count,
+                send_count);
+            EP_LAUNCH_CHECK();
+            dim3 sgrid((num_experts + 255) / 256, num_src);
+            ll_route_scan_kernel<<<sgrid, 256, 0, stream>>>(n, num_experts, num_ranks, rank, src_ranks, max_tokens,
+                                                            rs.num_chunks, rs.bytes, ws, recv_count, send_count);
+            EP_LAUNCH_CHECK();
+        }
+        if (n == 0) return 0;
     }
-    if (n == 0) return 0;
 
     const int pieces = row_format == kRowBF16 ? (hidden * 2 + 1023) / 1024 : (hidden / kGroup + 7) / 8;
-    const int64_t items = int64_t(num_src) * num_tokens * pieces;
-    const int64_t blocks = (items + 3) / 4;
-    EP_HOST_ASSERT(blocks < (int64_t(1) << 31));
+    // A small batch cannot fill 1024 SIMDs with one wave per row piece: give a share of the
+    // K stores of each piece to a second wave.
+    int split_log2 = int64_t(num_src) * num_tokens * pieces < 4096 && num_topk > 1 ? 1 : 0;
+    if (send_split_override() == 1) split_log2 = 0;
+    if (send_split_override() == 2) split_log2 = 1;
+    if (send_split_override() == 4) split_log2 = 2;
+    const int items = pieces << split_log2;  // waves per token
+    const int waves = items < kSendMaxWaves ? items : kSendMaxWaves;
+    const int blocks_per_token = (items + waves - 1) / waves;
+    EP_HOST_ASSERT(num_tokens < 65535 && num_src <= 65535);
+    const dim3 grid(blocks_per_token, num_tokens + (fused ? 1 : 0), num_src);
+    const size_t lds = fused ? size_t(num_experts) * sizeof(int32_t) : 0;
+    // floor(e / E_l) == umulhi(e, ceil(2^32 / E_l)) for every e below 2^16.
+    const uint32_t experts_per_rank = uint32_t(num_experts / num_ranks);
+    const uint32_t magic =
+        experts_per_rank == 1 ? 0u : uint32_t(((uint64_t(1) << 32) + experts_per_rank - 1) / experts_per_rank);
+    EP_HOST_ASSERT(num_experts < 65536);
     const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
     uint8_t* stg = reinterpret_cast<uint8_t*>(recv_staging);
     uint8_t* snd = reinterpret_cast<uint8_t*>(send_slots);
-#define DEEPEP_LAUNCH_SEND(FMT)                                                                              \
-    ll_send_kernel<FMT><<<dim3(unsigned(blocks)), 256, 0, stream>>>(                                         \
-        xb, topk_idx, src_ranks, num_src, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,        \
-        max_tokens, pieces, rs.bytes, ws, stg, snd, pair_slot)
+#define DEEPEP_SEND_ARGS                                                                                       \
+    xb, topk_idx, src_ranks, num_tokens, hidden, num_topk, num_experts, num_ranks, rank, max_tokens, pieces,    \
+        split_log2, magic, rs.bytes, ws, stg, snd, pair_slot, recv_count, send_count
+#define DEEPEP_LAUNCH_SEND(FMT)                                                                     \
+    do {                                                                                             \
+        if (fused)                                                                                   \
+            ll_send_kernel<FMT, true><<<grid, waves * kWave, lds, stream>>>(DEEPEP_SEND_ARGS);       \
+        else                                                                                         \
+            ll_send_kernel<FMT, false><<<grid, waves * kWave, 0, stream>>>(DEEPEP_SEND_ARGS);        \
+    } while (0)
     switch (row_format) {
         case kRowBF16: DEEPEP_LAUNCH_SEND(kRowBF16); break;
         case kRowFP8: DEEPEP_LAUNCH_SEND(kRowFP8); break;
@@ -371,6 +487,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
         default: DEEPEP_LAUNCH_SEND(kRowFP8UE8M0); break;
     }
 #undef DEEPEP_LAUNCH_SEND
+#undef DEEPEP_SEND_ARGS
     EP_LAUNCH_CHECK();
     return 0;
 }
@@ -452,13 +569,14 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
     const int num_local_experts = num_experts / num_ranks;
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     EP_HOST_ASSERT(max_rows < (int64_t(1) << 31));
-    int64_t blocks = (max_rows + 3) / 4;
-    const int64_t cap = max_rows > (int64_t(1) << 18) ? 4096 : 512;
+    const int parts = choose_row_parts(max_rows, row_data_bytes(hidden, row_format));
+    int64_t blocks = (max_rows * parts + 3) / 4;
+    const int64_t cap = max_rows > (int64_t(1) << 18) ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(num_experts + 1) * sizeof(int32_t);
     ll_recv_kernel<<<dim3(unsigned(blocks)), 256, lds, reinterpret_cast<hipStream_t>(stream)>>>(
         reinterpret_cast<const uint8_t*>(recv_staging), recv_count, hidden, num_local_experts, num_ranks,
-        num_max_dispatch_tokens_per_rank, row_format, reinterpret_cast<uint8_t*>(packed_recv_x),
+        num_max_dispatch_tokens_per_rank, row_format, parts, reinterpret_cast<uint8_t*>(packed_recv_x),
         reinterpret_cast<uint8_t*>(packed_recv_scales), packed_recv_src_info, packed_recv_layout_range,
         packed_recv_count, cumulative_local_expert_recv_stats);
     EP_LAUNCH_CHECK();

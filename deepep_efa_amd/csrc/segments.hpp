@@ -3,6 +3,8 @@
 // segment search, and the 16-byte-per-lane row copy.
 #pragma once
 
+#include <cstdlib>
+
 #include "common.hpp"
 
 namespace deepep {
@@ -46,24 +48,43 @@ __device__ __forceinline__ int find_segment(const int32_t* flat, int num_segment
     return lo;
 }
 
-// Copies `num_vec` 16-byte vectors with one wave, eight loads in flight per lane.
+// Copies 16-byte vectors [v_begin, v_end) of a row with one wave, eight loads
+// in flight per lane.
 __device__ __forceinline__ void wave_copy_vec16(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
-                                                int num_vec, int lane) {
+                                                int v_begin, int v_end, int lane) {
     const u32x4* s = reinterpret_cast<const u32x4*>(src);
     u32x4* d = reinterpret_cast<u32x4*>(dst);
-    for (int base = 0; base < num_vec; base += kWave * 8) {
+    for (int base = v_begin; base < v_end; base += kWave * 8) {
         u32x4 r[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int v = base + u * kWave + lane;
-            if (v < num_vec) r[u] = s[v];
+            if (v < v_end) r[u] = s[v];
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int v = base + u * kWave + lane;
-            if (v < num_vec) d[v] = r[u];
+            if (v < v_end) d[v] = r[u];
         }
     }
+}
+
+// A row of num_vec vectors cut into `parts` runs of whole 64-vector (1 KiB) chunks.
+__device__ __forceinline__ void row_part_range(int num_vec, int parts, int part, int& v_begin, int& v_end) {
+    const int chunks = (num_vec + kWave - 1) / kWave;
+    const int per = (chunks + parts - 1) / parts;
+    v_begin = min(part * per * kWave, num_vec);
+    v_end = min(v_begin + per * kWave, num_vec);
+}
+
+// Host-side choice of `parts`: small problems cannot fill the chip with one wave per row.
+inline int choose_row_parts(int64_t max_rows, int64_t row_bytes) {
+    if (const char* s = getenv("DEEPEP_ROW_PARTS")) {
+        const int v = atoi(s);
+        if (v >= 1 && v <= 8) return v;
+    }
+    if (max_rows > (int64_t(1) << 18)) return 1;
+    return row_bytes > 8192 ? 4 : 2;
 }
 
 }  // namespace deepep

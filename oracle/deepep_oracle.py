@@ -147,7 +147,7 @@ def per_token_cast_to_fp8(x: torch.Tensor, round_scale: bool = False, use_ue8m0:
     """
     assert x.dim() == 2 and x.shape[1] % GROUP == 0
     m, n = x.shape
-    xg = x.view(m, -1, GROUP).float()
+    xg = x.view(m, n // GROUP, GROUP).float()
     amax = xg.abs().amax(dim=2).clamp(min=1e-4)
     scales = amax / FP8_MAX
     if round_scale:
@@ -159,7 +159,7 @@ def per_token_cast_to_fp8(x: torch.Tensor, round_scale: bool = False, use_ue8m0:
     if use_ue8m0:
         assert round_scale and (n // GROUP) % 4 == 0
         ex = ((scales.contiguous().view(torch.int32) >> 23) & 0xFF).to(torch.uint8)
-        return q, ex.view(m, -1, 4).contiguous().view(torch.int32).view(m, -1)
+        return q, ex.view(m, n // GROUP // 4, 4).contiguous().view(torch.int32).view(m, n // GROUP // 4)
     return q, scales
 
 
@@ -186,9 +186,9 @@ def quantise_rows(x: torch.Tensor, fmt: int):
     """Payload bytes [T, data_bytes] u8 and scale bytes [T, scale_bytes] u8 of each token row."""
     t = x.shape[0]
     if fmt == ROW_BF16:
-        return x.contiguous().view(torch.uint8).view(t, -1), torch.zeros((t, 0), dtype=torch.uint8)
+        return x.contiguous().view(torch.uint8).view(t, x.shape[1] * 2), torch.zeros((t, 0), dtype=torch.uint8)
     q, s = per_token_cast_to_fp8(x, round_scale=fmt != ROW_FP8, use_ue8m0=fmt == ROW_FP8_UE8M0)
-    return q.view(torch.uint8).view(t, -1), s.contiguous().view(torch.uint8).view(t, -1)
+    return q.view(torch.uint8).view(t, x.shape[1]), s.contiguous().view(torch.uint8).view(t, row_scale_bytes(x.shape[1], fmt))
 
 
 # ----------------------------------------------------------------------------

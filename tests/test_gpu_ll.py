@@ -84,7 +84,12 @@ def check_dispatch(st, want, fmt):
 
 
 @pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16, O.ROW_FP8_POW2, O.ROW_FP8_UE8M0])
-@pytest.mark.parametrize("r,rank,t,h,k,e", [(4, 1, 8, 512, 3, 16), (8, 7, 33, 1024, 4, 64), (2, 0, 1, 512, 1, 2)])
+@pytest.mark.parametrize("r,rank,t,h,k,e", [
+    (4, 1, 8, 512, 3, 16), (8, 7, 33, 1024, 4, 64), (2, 0, 1, 512, 1, 2),
+    (4, 1, 40, 512, 9, 64),    # K > 8: separate route kernel, one chunk
+    (2, 1, 600, 512, 8, 16),   # T*K > 2048: chunked route + cross-chunk scan
+    (4, 3, 300, 512, 11, 32),  # both
+])
 def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e):
     x_all, topk_all, _ = make_world(r, t, h, k, e, seed=r * 100 + t, drop=min(5, t))
     st, _ = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt)
