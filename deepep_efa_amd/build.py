@@ -29,5 +29,31 @@ def build_hip_library(verbose: bool = True) -> str:
     return LIB
 
 
+HOST_MODULE = os.path.join(HERE, "deep_ep_cpp.so")
+
+
+def build_host_module(verbose: bool = True) -> str:
+    """Builds the pybind11 host module deep_ep_cpp (C++ only, no device code) with g++
+    against the installed PyTorch-ROCm and links it to libdeepep_hip.so."""
+    import sysconfig
+
+    import torch
+    tdir = os.path.dirname(torch.__file__)
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function", "-Wno-sign-compare",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=deep_ep_cpp",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           f"-I{tdir}/include", f"-I{tdir}/include/torch/csrc/api/include", f"-I{sysconfig.get_paths()['include']}",
+           "-I/opt/rocm/include", os.path.join(CSRC, "deep_ep_cpp.cpp"), "-o", HOST_MODULE,
+           f"-L{HERE}", "-ldeepep_hip", f"-L{tdir}/lib", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-lc10", "-lc10_hip",
+           "-ltorch_python", "-lamdhip64", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tdir}/lib"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose and proc.stdout.strip():
+        print(proc.stdout, file=sys.stderr)
+    if proc.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + proc.stdout)
+    return HOST_MODULE
+
+
 if __name__ == "__main__":
     print(build_hip_library())
+    print(build_host_module())
