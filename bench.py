@@ -36,6 +36,153 @@ def algorithmic_bytes(t, h, k, p, rv, stride, e, r):
     }
 
 
+def time_calls(torch, fn, n):
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(n):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / n
+
+
+def calibrate_copy(torch, _capi, lib):
+    """A plain copy through the pack kernel with identity row ids: 32768 rows x 14336 B read and written once.
+    Under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` the counters of pack_rows_kernel divided into the
+    known 469762048 bytes give the scale of each counter on this GPU."""
+    rows, row_bytes = 32768, 14336
+    src = torch.empty((rows, row_bytes), dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty_like(src)
+    ids = torch.arange(rows, dtype=torch.int64, device="cuda")
+    n_dev = torch.tensor([rows], dtype=torch.int64, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def fn():
+        _capi.check(lib.deepep_pack_rows(_capi.ptr(src), None, _capi.ptr(ids), _capi.ptr(n_dev), rows, rows, row_bytes,
+                                         0, _capi.ptr(dst), None, stream))
+    us = time_calls(torch, fn, 10)
+    assert torch.equal(src, dst)
+    print(json.dumps({"calibrate_copy": {"kernel": "pack_rows_kernel", "bytes_read": rows * row_bytes,
+                                         "bytes_written": rows * row_bytes, "us": round(us, 2),
+                                         "GBps": round(2 * rows * row_bytes / us / 1e3, 1)}}))
+
+
+def read_traffic_summary(kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary (None if absent)."""
+    path = os.path.join(ROOT, "profiles", "ll_dispatch_combine_ep32_128tok_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        parts = line.split()
+        if len(parts) >= 4 and parts[0] == kernel and parts[1].isdigit() and parts[2].isdigit():
+            return int(parts[1]) + int(parts[2])
+    return None
+
+
+def bench_pack(torch, _capi, lib, loopback, args):
+    """Normal-mode layout + pack at 4096 tokens x 7168, top-8 of 256 experts, 8 ranks x 32 experts."""
+    t, h, k, e, r = 4096, 7168, 8, 256, 8
+    world = loopback.LoopbackWorld(r, 0, seed=args.seed)
+    world.synthesise(t, h, k, e)
+    x, topk = world.own_inputs()
+    stream = torch.cuda.current_stream().cuda_stream
+    i32 = dict(dtype=torch.int32, device="cuda")
+    per_rank, per_expert = torch.empty(r, **i32), torch.empty(e, **i32)
+    is_in = torch.empty((t, r), dtype=torch.bool, device="cuda")
+    ws = torch.empty(max(256, lib.deepep_layout_workspace_bytes(t, r, e)), dtype=torch.uint8, device="cuda")
+    ids = torch.empty(t * r, dtype=torch.int64, device="cuda")
+    counts, cumsum = torch.empty(r, **i32), torch.empty(r + 1, dtype=torch.int64, device="cuda")
+    ws2 = torch.empty(max(256, lib.deepep_routing_sort_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
+    cpm = torch.empty((r, 10), **i32)
+
+    def layout():
+        _capi.check(lib.deepep_get_dispatch_layout(_capi.ptr(topk), t, k, r, e, _capi.ptr(per_rank), None,
+                                                   _capi.ptr(per_expert), _capi.ptr(is_in), _capi.ptr(ws), ws.numel(),
+                                                   stream))
+
+    def sort():
+        _capi.check(lib.deepep_moe_routing_sort(_capi.ptr(is_in), t, r, _capi.ptr(ids), _capi.ptr(counts),
+                                                _capi.ptr(cumsum), _capi.ptr(ws2), ws2.numel(), stream))
+
+    def prefix():
+        _capi.check(lib.deepep_channel_prefix_matrix(_capi.ptr(is_in), t, r, 10, _capi.ptr(cpm), stream))
+
+    layout(), sort(), prefix()
+    torch.cuda.synchronize()
+    s = int(cumsum[r])
+    total_dev = cumsum[r:]
+    q = torch.empty((t, h), dtype=torch.uint8, device="cuda")
+    sc = torch.empty((t, h // 128), dtype=torch.float32, device="cuda")
+    _capi.check(lib.deepep_per_token_cast_to_fp8(_capi.ptr(x), t, h, 1, _capi.ptr(q), _capi.ptr(sc), stream))
+    out16 = torch.empty((s, h), dtype=torch.bfloat16, device="cuda")
+    out8 = torch.empty((s, h), dtype=torch.uint8, device="cuda")
+    outs = torch.empty((s, h // 128), dtype=torch.float32, device="cuda")
+
+    def pack_bf16():
+        _capi.check(lib.deepep_pack_rows(_capi.ptr(x), None, _capi.ptr(ids), _capi.ptr(total_dev), s, t, 2 * h, 0,
+                                         _capi.ptr(out16), None, stream))
+
+    def pack_fp8():
+        _capi.check(lib.deepep_pack_rows(_capi.ptr(q), _capi.ptr(sc), _capi.ptr(ids), _capi.ptr(total_dev), s, t, h,
+                                         h // 32, _capi.ptr(out8), _capi.ptr(outs), stream))
+
+    def cast():
+        _capi.check(lib.deepep_per_token_cast_to_fp8(_capi.ptr(x), t, h, 1, _capi.ptr(q), _capi.ptr(sc), stream))
+
+    n = max(10, args.steps // 4)
+    res = {"workload": "4096 tokens x 7168 bf16, top-8 of 256 experts, 8 ranks x 32 experts", "rows_packed": s}
+    for name, fn, nbytes in (("layout", layout, t * k * 8 + t * r + 4 * (r + e)),
+                             ("routing_sort", sort, 2 * t * r + s * 8),
+                             ("channel_prefix", prefix, t * r + r * 10 * 4),
+                             ("cast_fp8", cast, t * 2 * h + t * h + t * (h // 32)),
+                             ("pack_bf16", pack_bf16, s * 2 * h * 2 + s * 8),
+                             ("pack_fp8", pack_fp8, s * (h + h // 32) * 2 + s * 8)):
+        us = time_calls(torch, fn, n)
+        res[name] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                     "frac_of_8TBps": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    return res
+
+
+def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args):
+    """The same four LL entry points at 4096 tokens (8 ranks x 32 experts), where they are HBM-bound."""
+    t, h, k, e, r, rank = 4096, 7168, 8, 256, 8, 3
+    shape = ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8)
+    st = ll_runtime.LowLatencyState(shape)
+    world = loopback.LoopbackWorld(r, rank, seed=args.seed + 7)
+    world.synthesise(t, h, k, e)
+    x, topk = world.own_inputs()
+    weights = torch.softmax(torch.randn((t, k), generator=torch.Generator().manual_seed(1)), dim=-1).cuda()
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    epr, n_slots = e // r, r * t
+    y = torch.empty((epr, n_slots, h), dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    _capi.check(lib.deepep_synth_bf16_rows(_capi.ptr(y), epr * n_slots, h, h * 2, None, 0, 5, 0, stream))
+    st.dispatch_send(x, topk)
+    world.dispatch_from_peers(st)
+    st.dispatch_recv()
+    world.combine_from_peers(st, mode=1, seed=9)
+    torch.cuda.synchronize()
+    p = int((st.pair_slot[:t] >= 0).sum())
+    rv = int(st.packed_recv_count.sum())
+    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r)
+    calls = {
+        "dispatch_send": lambda: st.dispatch_send(x, topk),
+        "dispatch_recv": lambda: st.dispatch_recv(),
+        "combine_send": lambda: st.combine_send(y),
+        "combine_recv": lambda: st.combine_recv(topk, weights, out),
+    }
+    res = {"workload": "LL dispatch+combine at 4096 tokens x 7168, top-8 of 256 experts, 8 ranks x 32 experts",
+           "pairs_sent": p, "rows_received": rv}
+    for name, fn in calls.items():
+        us = time_calls(torch, fn, max(10, args.steps // 10))
+        res[name] = {"us": round(us, 2), "bytes": nbytes[name], "GBps": round(nbytes[name] / us / 1e3, 1),
+                     "frac_of_8TBps": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBS, 4)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -49,6 +196,9 @@ def main():
     ap.add_argument("--rank", type=int, default=5)
     ap.add_argument("--seed", type=int, default=2024)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-pack", action="store_true", help="skip the normal-mode layout + pack section")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a plain row copy of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--no-graph", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -62,6 +212,12 @@ def main():
     lib = _capi.load()
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     torch.cuda.set_device(0)
+    if args.calibrate_copy:
+        calibrate_copy(torch, _capi, lib)
+        return
+    if os.environ.get("DEEPEP_BENCH_ONLY_LARGE") == "1":  # tuning aid: the 4096-token section alone
+        print(json.dumps(bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args)))
+        return
     t, h, k, e, r, rank = args.tokens, args.hidden, args.topk, args.experts, args.ranks, args.rank
     shape = ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8)
     st = ll_runtime.LowLatencyState(shape)
@@ -175,6 +331,15 @@ def main():
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
     }
+
+    traffic = read_traffic_summary(dom)
+    if traffic is not None and (t, h, k, e, r) == (128, 7168, 8, 256, 32):
+        result["roofline"]["traffic"] = traffic
+    if not args.no_pack:
+        del st, y
+        torch.cuda.empty_cache()
+        result["normal_mode_pack"] = bench_pack(torch, _capi, lib, loopback, args)
+        result["ll_4096_tokens"] = bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args)
 
     if not args.no_cpu_baseline:
         from oracle import cpu_baseline
