@@ -1,7 +1,7 @@
 """MI355X-native MoE token dispatch/combine hot path behind the deep_ep.Buffer API.
 
 Importing the package loads the HIP library and the host module; both must have
-been built (`python -m deepep_efa_amd.build`).  There is no CPU fallback.
+been built (`python deepep_efa_amd/build.py`).  There is no CPU fallback.
 """
 import torch  # noqa: F401  (its HIP runtime must be the one loaded in this process)
 

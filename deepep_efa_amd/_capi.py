@@ -1,6 +1,6 @@
 """ctypes view of the C ABI declared in include/deepep_hip.h.
 
-The library must already be built (``python -m deepep_efa_amd.build`` or
+The library must already be built (``python deepep_efa_amd/build.py`` or
 ``__graft_entry__.build()``); a missing library is an error, never a fallback.
 """
 import ctypes
@@ -29,8 +29,9 @@ PROTOTYPES = {
     "deepep_per_token_cast_to_fp8": (_I, [_VP, _I, _I, _I, _VP, _VP, _VP]),
     "deepep_ll_dispatch_workspace_bytes": (_SZ, [_I, _I, _I]),
     "deepep_ll_dispatch_send": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
-    "deepep_ll_dispatch_recv": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
-    "deepep_ll_combine_send": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _VP]),
+    "deepep_ll_segment_workspace_bytes": (_SZ, [_I, _I]),
+    "deepep_ll_dispatch_recv": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _SZ, _VP]),
+    "deepep_ll_combine_send": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I64, _VP, _SZ, _VP]),
     "deepep_ll_combine_recv": (_I, [_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP, _VP]),
     "deepep_synth_topk_idx": (_I, [_VP, _VP, _I, _I, _I, _I, _U32, _VP, _VP]),
     "deepep_synth_bf16_rows": (_I, [_VP, _I64, _I, _I64, _VP, _U32, _U32, _I, _VP]),
@@ -50,7 +51,7 @@ def load() -> ctypes.CDLL:
     global _lib
     if _lib is None:
         if not os.path.exists(LIB_PATH):
-            raise ImportError(f"{LIB_PATH} is missing: build it with `python -m deepep_efa_amd.build`")
+            raise ImportError(f"{LIB_PATH} is missing: build it with `python deepep_efa_amd/build.py`")
         lib = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in PROTOTYPES.items():
             fn = getattr(lib, name)

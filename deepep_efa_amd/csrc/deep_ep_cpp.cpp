@@ -160,7 +160,7 @@ static void stream_wait(const HostStream& waiter, const EventHandle& event) {
 // ---------------------------------------------------------------------------
 struct LowLatencyCache {
     int max_tokens = 0, hidden = 0, num_topk = 0, num_experts = 0, row_format = -1;
-    torch::Tensor recv_staging, recv_count, send_slots, send_count, pair_slot, workspace;
+    torch::Tensor recv_staging, recv_count, send_slots, send_count, pair_slot, workspace, segment_workspace;
     torch::Tensor packed_recv_x, packed_recv_scales, packed_recv_count, packed_recv_src_info, packed_recv_layout_range;
     torch::Tensor combine_staging, combine_send_slots, combined_x;
     bool dispatched = false;
@@ -399,6 +399,9 @@ struct Buffer {
         ll.pair_slot = torch::full({m, num_topk}, -1, i32);
         ll.workspace = torch::empty(
             {std::max<int64_t>(256, int64_t(deepep_ll_dispatch_workspace_bytes(max_tokens, num_topk, num_experts)))}, u8);
+        if (e * m > (int64_t(1) << 18))  // index + flat-copy scratch, only used by large batches
+            ll.segment_workspace =
+                torch::empty({int64_t(deepep_ll_segment_workspace_bytes(num_experts, max_tokens))}, u8);
         if (fmt == DEEPEP_ROW_BF16) {
             ll.packed_recv_x = torch::empty({el, r * m, h}, bf16);
         } else {
@@ -487,7 +490,9 @@ struct Buffer {
             c.packed_recv_src_info.data_ptr<int>(), c.packed_recv_layout_range.data_ptr<int64_t>(),
             c.packed_recv_count.data_ptr<int>(),
             cumulative_local_expert_recv_stats.has_value() ? cumulative_local_expert_recv_stats->data_ptr<int>() : nullptr,
-            stream));
+            int64_t(num_max_dispatch_tokens_per_rank) * num_topk,
+            c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
+            c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));
         c.dispatched = true;
 
         std::optional<EventHandle> event;
@@ -555,7 +560,11 @@ struct Buffer {
 
         abi_check(deepep_ll_combine_send(src.data_ptr(), layout_range.data_ptr<int64_t>(), hidden, num_experts,
                                          num_ranks, rank, num_max_dispatch_tokens_per_rank, c.combine_staging.data_ptr(),
-                                         c.combine_send_slots.data_ptr(), stream));
+                                         c.combine_send_slots.data_ptr(),
+                                         int64_t(num_max_dispatch_tokens_per_rank) * num_topk,
+                                         c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
+                                         c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0,
+                                         stream));
         if (world_x.has_value())  // what the remote experts would have returned
             abi_check(deepep_loopback_combine_from_peers(c.send_slots.data_ptr(), c.send_count.data_ptr<int>(), hidden,
                                                          num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,

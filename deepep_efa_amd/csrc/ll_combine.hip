@@ -136,7 +136,8 @@ extern "C" {
 
 int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidden, int num_experts, int num_ranks,
                            int rank, int num_max_dispatch_tokens_per_rank, void* combine_staging,
-                           void* combine_send_slots, void* stream) {
+                           void* combine_send_slots, int64_t expected_rows, void* workspace, size_t workspace_bytes,
+                           void* stream) {
     clear_error();
     EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
     EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
@@ -150,12 +151,34 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
     const int num_local_experts = num_experts / num_ranks;
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     EP_HOST_ASSERT(max_rows < (int64_t(1) << 31));
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    if (max_rows > kLargeBatchRows && workspace != nullptr) {
+        EP_HOST_ASSERT(workspace_bytes >= size_t(segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank)));
+        EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
+        int32_t* flat = reinterpret_cast<int32_t*>(workspace);
+        RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) +
+                                                   (((int64_t(num_experts) + 1) * 4 + 255) & ~int64_t(255)));
+        ll_segment_index_kernel<<<num_experts, kIndexThreads, 0, hs>>>(
+            1, nullptr, layout_range, num_local_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank, nullptr,
+            nullptr, nullptr, flat, desc);
+        EP_LAUNCH_CHECK();
+        const int num_vec = hidden * 2 / 16;
+        int threads = ((num_vec + 63) / 64) * 64;
+        if (threads > 1024) threads = 1024;
+        ll_rows_flat_kernel<<<flat_grid_blocks(expected_rows, max_rows, num_max_dispatch_tokens_per_rank), threads, 0,
+                              hs>>>(flat, num_experts, desc, reinterpret_cast<const uint8_t*>(x), int64_t(hidden) * 2,
+                                    num_vec, reinterpret_cast<uint8_t*>(combine_send_slots),
+                                    reinterpret_cast<uint8_t*>(combine_staging), int64_t(hidden) * 2, 0, 0, nullptr, 0,
+                                    nullptr, 0);
+        EP_LAUNCH_CHECK();
+        return 0;
+    }
     const int parts = choose_row_parts(max_rows, int64_t(hidden) * 2);
     int64_t blocks = (max_rows * parts + 3) / 4;
-    const int64_t cap = max_rows > (int64_t(1) << 18) ? 4096 : 1024;
+    const int64_t cap = max_rows > kLargeBatchRows ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(2 * num_experts + 1) * sizeof(int32_t);
-    ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, lds, reinterpret_cast<hipStream_t>(stream)>>>(
+    ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, lds, hs>>>(
         reinterpret_cast<const uint8_t*>(x), layout_range, hidden, num_local_experts, num_ranks, rank,
         num_max_dispatch_tokens_per_rank, parts, reinterpret_cast<uint8_t*>(combine_staging),
         reinterpret_cast<uint8_t*>(combine_send_slots));

@@ -22,27 +22,21 @@
 namespace deepep {
 
 constexpr int kRouteChunk = 1024;  // (token,k) entries ranked by one workgroup
-constexpr int kRouteWaves = kRouteChunk / kWave;
 
 __host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
 
 struct RouteScratch {
-    int32_t* pair_rank;   // [n] rank of the pair inside its chunk, -1 = no selection
-    int32_t* chunk_base;  // [C][E] pairs of expert e in earlier chunks
-    int num_chunks;
-    int64_t bytes;
+    int num_chunks;  // 1024-entry chunks of the (token,k) list
+    int64_t bytes;   // per source: slot of every (token,k) entry, int32 [T*K]
 };
 
-static RouteScratch carve_route_scratch(void* base, int num_tokens, int num_topk, int num_experts) {
+static RouteScratch route_scratch(int num_tokens, int num_topk, int num_experts) {
+    (void)num_experts;
     RouteScratch s;
     const int64_t n = int64_t(num_tokens) * num_topk;
     s.num_chunks = int((n + kRouteChunk - 1) / kRouteChunk);
     if (s.num_chunks < 1) s.num_chunks = 1;
-    const int64_t rank_bytes = align256(n * 4 + 4);
-    const int64_t base_bytes = align256(int64_t(s.num_chunks) * num_experts * 4);
-    s.pair_rank = reinterpret_cast<int32_t*>(base);
-    s.chunk_base = reinterpret_cast<int32_t*>(reinterpret_cast<uint8_t*>(base) + rank_bytes);
-    s.bytes = rank_bytes + base_bytes;
+    s.bytes = align256(n * 4 + 4);
     return s;
 }
 
@@ -57,36 +51,59 @@ __device__ __forceinline__ void emit_expert_count(int e, int total, int num_expe
 }
 
 // ---------------------------------------------------------------------
-// Route ranking.  Entry i = t*K + k.  pair_rank[i] = number of entries i' < i
-// of the same chunk naming the same expert; chunk totals go to chunk_base for
-// the cross-chunk scan.  In-wave ranks come from ballots over the 64 lanes
-// (one ballot per distinct expert present in the wave), cross-wave offsets
-// from a 16 x E table in LDS.  Deterministic: no atomics anywhere.
+// Slot ranking for batches of more than one chunk, in one launch.  Entry
+// i = t*K + k lives in chunk i / 1024; workgroup c owns chunk c and writes the
+// final slot of each of its entries:
+//   base  — entries of earlier chunks naming the same expert: the workgroup
+//           re-reads them (L2-resident, at most T*K*8 bytes) into an LDS
+//           histogram, so no workgroup waits on another;
+//   rank  — earlier entries of the same chunk: in-wave by 64-lane ballots (one
+//           ballot per distinct expert present in the wave), across the 16 waves
+//           by a 16 x E table in LDS.
+// The last chunk's workgroup also publishes the per-expert totals.
+// Deterministic: integer adds and ballots only.
 // Reference semantics: the serial (token,k) scan of
-// csrc/kernels/efa_kernels.cu:617-637 and coop_dispatch_send.cuh's token_offset.
+// csrc/kernels/efa_kernels.cu:617-637 and token_offset / expert_offsets of
+// csrc/kernels/coop_dispatch_send.cuh:360-420.
 // ---------------------------------------------------------------------
-template <bool kSingleChunk>
-__global__ __launch_bounds__(kRouteChunk) void ll_route_rank_kernel(
+constexpr int kRouteWaves = kRouteChunk / kWave;
+
+__global__ __launch_bounds__(kRouteChunk) void ll_route_slots_kernel(
     const int64_t* __restrict__ topk_idx, int n, int num_experts, int num_ranks, int rank,
     const int32_t* __restrict__ src_ranks, int max_tokens, int64_t scratch_stride,
     uint8_t* __restrict__ scratch_base, int32_t* __restrict__ recv_count, int32_t* __restrict__ send_count) {
-    extern __shared__ int32_t wave_hist[];  // [kRouteWaves][E]
+    extern __shared__ int32_t route_lds[];
+    int32_t* base_hist = route_lds;               // [E] entries of earlier chunks
+    int32_t* wave_hist = route_lds + num_experts;  // [kRouteWaves][E]
     const int b = blockIdx.y, c = blockIdx.x;
     const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
-    const int num_chunks = gridDim.x;
+    const int64_t* my_topk = topk_idx + int64_t(b) * n;
+    int32_t* slots = reinterpret_cast<int32_t*>(scratch_base + int64_t(b) * scratch_stride);
 
-    uint8_t* my_scratch = scratch_base + int64_t(b) * scratch_stride;
-    int32_t* pair_rank = reinterpret_cast<int32_t*>(my_scratch);
-    int32_t* chunk_base = reinterpret_cast<int32_t*>(my_scratch + align256(int64_t(n) * 4 + 4));
-
+    for (int j = tid; j < (kRouteWaves + 1) * num_experts; j += kRouteChunk) route_lds[j] = 0;
     const int i = c * kRouteChunk + tid;
     int e = -1;
     if (i < n) {
-        const int64_t v = topk_idx[int64_t(b) * n + i];
+        const int64_t v = my_topk[i];
         if (v >= 0 && v < num_experts) e = int(v);
     }
-    for (int j = tid; j < kRouteWaves * num_experts; j += kRouteChunk) wave_hist[j] = 0;
+    __syncthreads();
 
+    // base: histogram of every earlier chunk, eight independent loads per thread per step
+    const int before = c * kRouteChunk;
+    for (int i0 = tid; i0 < before; i0 += kRouteChunk * 8) {
+        int64_t v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int j = i0 + u * kRouteChunk;
+            v[u] = j < before ? my_topk[j] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (v[u] >= 0 && v[u] < num_experts) atomicAdd(&base_hist[int(v[u])], 1);
+    }
+
+    // rank inside the wave
     uint64_t pending = __ballot(e >= 0);
     int my_rank = 0, my_count = 0;
     while (pending != 0) {
@@ -99,52 +116,24 @@ __global__ __launch_bounds__(kRouteChunk) void ll_route_rank_kernel(
         }
         pending &= ~same;
     }
-    __syncthreads();
     if (e >= 0 && my_rank == 0) wave_hist[w * num_experts + e] = my_count;
     __syncthreads();
+    // exclusive scan over the 16 waves, one thread per expert
+    const bool last_chunk = c == int(gridDim.x) - 1;
+    const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
     for (int x = tid; x < num_experts; x += kRouteChunk) {
-        int run = 0;
+        int run = base_hist[x];
 #pragma unroll
         for (int w2 = 0; w2 < kRouteWaves; ++w2) {
             const int cnt = wave_hist[w2 * num_experts + x];
             wave_hist[w2 * num_experts + x] = run;
             run += cnt;
         }
-        if constexpr (kSingleChunk) {
-            chunk_base[x] = 0;
-            const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
-            emit_expert_count(x, run, num_experts, num_ranks, rank, src_rank, max_tokens, recv_count,
-                              send_count);
-        } else {
-            chunk_base[int64_t(c) * num_experts + x] = run;
-        }
+        if (last_chunk)
+            emit_expert_count(x, run, num_experts, num_ranks, rank, src_rank, max_tokens, recv_count, send_count);
     }
     __syncthreads();
-    if (i < n) pair_rank[i] = e >= 0 ? wave_hist[w * num_experts + e] + my_rank : -1;
-    (void)num_chunks;
-}
-
-// Cross-chunk exclusive scan per expert (only launched when T*K > kRouteChunk).
-__global__ __launch_bounds__(256) void ll_route_scan_kernel(int n, int num_experts, int num_ranks, int rank,
-                                                            const int32_t* __restrict__ src_ranks,
-                                                            int max_tokens, int num_chunks,
-                                                            int64_t scratch_stride,
-                                                            uint8_t* __restrict__ scratch_base,
-                                                            int32_t* __restrict__ recv_count,
-                                                            int32_t* __restrict__ send_count) {
-    const int b = blockIdx.y;
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= num_experts) return;
-    uint8_t* my_scratch = scratch_base + int64_t(b) * scratch_stride;
-    int32_t* chunk_base = reinterpret_cast<int32_t*>(my_scratch + align256(int64_t(n) * 4 + 4));
-    int run = 0;
-    for (int c = 0; c < num_chunks; ++c) {
-        const int cnt = chunk_base[int64_t(c) * num_experts + e];
-        chunk_base[int64_t(c) * num_experts + e] = run;
-        run += cnt;
-    }
-    const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
-    emit_expert_count(e, run, num_experts, num_ranks, rank, src_rank, max_tokens, recv_count, send_count);
+    if (i < n) slots[i] = e >= 0 ? wave_hist[w * num_experts + e] + my_rank : -1;
 }
 
 // ---------------------------------------------------------------------
@@ -161,25 +150,25 @@ __global__ __launch_bounds__(256) void ll_route_scan_kernel(int n, int num_exper
 // waves through LDS, so a wave's own work is: two loads, the DPP quantise,
 // and per selection one 8-byte LDS read and two stores.
 //
-// kFusedRoute (small batches): no route kernel runs first.  While the row
-// loads are in flight the workgroup ranks the token's selections itself: its
-// threads sweep the (token,k) entries before the token, one entry per thread
-// per step, and bump an LDS counter for every entry that names one of the
-// token's experts.  The sweep is O(T*K) per token, which at T*K <= 2048 is one
-// or two loads per thread and costs less than a dependent launch.  The
-// per-expert totals come from one extra row of workgroups (blockIdx.y == T),
-// an LDS histogram per source.
+// A small batch (T*K <= 2048) needs no route kernel: while the row loads are
+// in flight the workgroup's threads sweep the (token,k) entries before the
+// token, one entry per thread per step, and bump an LDS counter for every entry
+// that names one of the token's experts (integer adds — order does not matter);
+// the per-expert totals come from one extra row of workgroups (blockIdx.y == T),
+// an LDS histogram per source.  Larger batches read the slots ranked by
+// ll_route_slots_kernel.
 // ---------------------------------------------------------------------
 constexpr int kMaxTopk = 64;
 constexpr int kFusedMaxEntries = 2048;
 constexpr int kSendMaxWaves = 16;
 
-template <int kFmt, bool kFusedRoute>
+template <int kFmt>
 __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(
     const uint8_t* __restrict__ x, const int64_t* __restrict__ topk_idx,
     const int32_t* __restrict__ src_ranks, int num_tokens, int hidden, int num_topk, int num_experts,
     int num_ranks, int rank, int max_tokens, int pieces_per_row, int split_log2, uint32_t rank_of_expert_magic,
-    int64_t scratch_stride, const uint8_t* __restrict__ scratch_base, uint8_t* __restrict__ recv_staging,
+    int num_chunks, int64_t scratch_stride, const uint8_t* __restrict__ scratch_base,
+    uint8_t* __restrict__ recv_staging,
     uint8_t* __restrict__ send_slots, int32_t* __restrict__ pair_slot, int32_t* __restrict__ recv_count,
     int32_t* __restrict__ send_count) {
     extern __shared__ int32_t lds_hist[];  // [E], counting workgroups only
@@ -192,21 +181,19 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(
     const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
     const int64_t* my_topk = topk_idx + int64_t(b) * n;
 
-    if constexpr (kFusedRoute) {
-        if (t == num_tokens) {  // the counting row of the grid: one workgroup per source
-            if (blockIdx.x != 0) return;
-            for (int j = tid; j < num_experts; j += blockDim.x) lds_hist[j] = 0;
-            __syncthreads();
-            for (int i = tid; i < n; i += blockDim.x) {
-                const int64_t v = my_topk[i];
-                if (v >= 0 && v < num_experts) atomicAdd(&lds_hist[int(v)], 1);
-            }
-            __syncthreads();
-            for (int e = tid; e < num_experts; e += blockDim.x)
-                emit_expert_count(e, lds_hist[e], num_experts, num_ranks, rank, src_rank, max_tokens, recv_count,
-                                  send_count);
-            return;
+    if (t == num_tokens) {  // the counting row of the grid (single-chunk batches): one workgroup per source
+        if (blockIdx.x != 0) return;
+        for (int j = tid; j < num_experts; j += blockDim.x) lds_hist[j] = 0;
+        __syncthreads();
+        for (int i = tid; i < n; i += blockDim.x) {
+            const int64_t v = my_topk[i];
+            if (v >= 0 && v < num_experts) atomicAdd(&lds_hist[int(v)], 1);
         }
+        __syncthreads();
+        for (int e = tid; e < num_experts; e += blockDim.x)
+            emit_expert_count(e, lds_hist[e], num_experts, num_ranks, rank, src_rank, max_tokens, recv_count,
+                              send_count);
+        return;
     }
 
     const int item = int(blockIdx.x) * int(blockDim.x >> 6) + wave_in_block();
@@ -245,19 +232,15 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(
     if (tid < num_topk) {
         const int64_t v = my_topk[entry0 + tid];
         if (v >= 0 && v < num_experts) my_expert = int(v);
-        if constexpr (kFusedRoute) {
+    }
+    if (num_chunks > 1) {  // slots were ranked by ll_route_slots_kernel
+        if (tid < num_topk && my_expert >= 0)
+            my_slot = reinterpret_cast<const int32_t*>(scratch_base + int64_t(b) * scratch_stride)[entry0 + tid];
+    } else {  // small batch: rank here, sweeping every earlier entry
+        if (tid < num_topk) {
             sel_expert[tid] = my_expert;
             sel_count[tid] = 0;
-        } else {
-            const int32_t* pair_rank = reinterpret_cast<const int32_t*>(scratch_base + int64_t(b) * scratch_stride);
-            const int32_t* chunk_base = reinterpret_cast<const int32_t*>(
-                scratch_base + int64_t(b) * scratch_stride + align256(int64_t(n) * 4 + 4));
-            const int in_chunk = pair_rank[entry0 + tid];
-            if (in_chunk >= 0 && my_expert >= 0)
-                my_slot = in_chunk + chunk_base[((entry0 + tid) / kRouteChunk) * num_experts + my_expert];
         }
-    }
-    if constexpr (kFusedRoute) {
         __syncthreads();
         for (int i = tid; i < entry0; i += blockDim.x) {
             const int64_t v = my_topk[i];
@@ -419,34 +402,20 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
                             int max_tokens, int row_format, void* recv_staging, int32_t* recv_count,
                             void* send_slots, int32_t* send_count, int32_t* pair_slot, void* workspace,
                             size_t workspace_bytes, hipStream_t stream) {
-    const RouteScratch rs = carve_route_scratch(workspace, num_tokens, num_topk, num_experts);
+    RouteScratch rs = route_scratch(num_tokens, num_topk, num_experts);
     EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(rs.bytes) * size_t(num_src));
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
     const int n = num_tokens * num_topk;
     uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
-    const bool fused = n <= kFusedMaxEntries;
+    const bool single_chunk = n <= kFusedMaxEntries;  // up to two nominal chunks are swept as one
+    if (single_chunk) rs.num_chunks = 1;
 
-    if (!fused) {
-        // Route kernels.  Counts are published even for an empty batch of tokens.
-        const size_t lds = size_t(kRouteWaves) * num_experts * sizeof(int32_t);
+    if (!single_chunk) {
+        const size_t lds = size_t(kRouteWaves + 1) * num_experts * sizeof(int32_t);
         EP_HOST_ASSERT(lds <= 64 * 1024);
-        dim3 rgrid(rs.num_chunks, num_src);
-        if (rs.num_chunks == 1) {
-            ll_route_rank_kernel<true><<<rgrid, kRouteChunk, lds, stream>>>(
-                topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count,
-                send_count);
-            EP_LAUNCH_CHECK();
-        } else {
-            ll_route_rank_kernel<false><<<rgrid, kRouteChunk, lds, stream>>>(
-                topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count,
-                send_count);
-            EP_LAUNCH_CHECK();
-            dim3 sgrid((num_experts + 255) / 256, num_src);
-            ll_route_scan_kernel<<<sgrid, 256, 0, stream>>>(n, num_experts, num_ranks, rank, src_ranks, max_tokens,
-                                                            rs.num_chunks, rs.bytes, ws, recv_count, send_count);
-            EP_LAUNCH_CHECK();
-        }
-        if (n == 0) return 0;
+        ll_route_slots_kernel<<<dim3(rs.num_chunks, num_src), kRouteChunk, lds, stream>>>(
+            topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count, send_count);
+        EP_LAUNCH_CHECK();
     }
 
     const int pieces = row_format == kRowBF16 ? (hidden * 2 + 1023) / 1024 : (hidden / kGroup + 7) / 8;
@@ -460,8 +429,9 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     const int waves = items < kSendMaxWaves ? items : kSendMaxWaves;
     const int blocks_per_token = (items + waves - 1) / waves;
     EP_HOST_ASSERT(num_tokens < 65535 && num_src <= 65535);
-    const dim3 grid(blocks_per_token, num_tokens + (fused ? 1 : 0), num_src);
-    const size_t lds = fused ? size_t(num_experts) * sizeof(int32_t) : 0;
+    const dim3 grid(blocks_per_token, num_tokens + (single_chunk ? 1 : 0), num_src);
+    if (grid.y == 0) return 0;
+    const size_t lds = single_chunk ? size_t(num_experts) * sizeof(int32_t) : 0;
     // floor(e / E_l) == umulhi(e, ceil(2^32 / E_l)) for every e below 2^16.
     const uint32_t experts_per_rank = uint32_t(num_experts / num_ranks);
     const uint32_t magic =
@@ -470,16 +440,10 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
     uint8_t* stg = reinterpret_cast<uint8_t*>(recv_staging);
     uint8_t* snd = reinterpret_cast<uint8_t*>(send_slots);
-#define DEEPEP_SEND_ARGS                                                                                       \
-    xb, topk_idx, src_ranks, num_tokens, hidden, num_topk, num_experts, num_ranks, rank, max_tokens, pieces,    \
-        split_log2, magic, rs.bytes, ws, stg, snd, pair_slot, recv_count, send_count
-#define DEEPEP_LAUNCH_SEND(FMT)                                                                     \
-    do {                                                                                             \
-        if (fused)                                                                                   \
-            ll_send_kernel<FMT, true><<<grid, waves * kWave, lds, stream>>>(DEEPEP_SEND_ARGS);       \
-        else                                                                                         \
-            ll_send_kernel<FMT, false><<<grid, waves * kWave, 0, stream>>>(DEEPEP_SEND_ARGS);        \
-    } while (0)
+#define DEEPEP_LAUNCH_SEND(FMT)                                                                                 \
+    ll_send_kernel<FMT><<<grid, waves * kWave, lds, stream>>>(                                                  \
+        xb, topk_idx, src_ranks, num_tokens, hidden, num_topk, num_experts, num_ranks, rank, max_tokens, pieces, \
+        split_log2, magic, rs.num_chunks, rs.bytes, ws, stg, snd, pair_slot, recv_count, send_count)
     switch (row_format) {
         case kRowBF16: DEEPEP_LAUNCH_SEND(kRowBF16); break;
         case kRowFP8: DEEPEP_LAUNCH_SEND(kRowFP8); break;
@@ -487,7 +451,6 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
         default: DEEPEP_LAUNCH_SEND(kRowFP8UE8M0); break;
     }
 #undef DEEPEP_LAUNCH_SEND
-#undef DEEPEP_SEND_ARGS
     EP_LAUNCH_CHECK();
     return 0;
 }
@@ -502,8 +465,12 @@ size_t deepep_ll_row_data_bytes(int hidden, int row_format) { return size_t(row_
 size_t deepep_ll_row_scale_bytes(int hidden, int row_format) { return size_t(row_scale_bytes(hidden, row_format)); }
 size_t deepep_ll_row_stride(int hidden, int row_format) { return size_t(row_stride_bytes(hidden, row_format)); }
 
+size_t deepep_ll_segment_workspace_bytes(int num_experts, int num_max_dispatch_tokens_per_rank) {
+    return size_t(segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank));
+}
+
 size_t deepep_ll_dispatch_workspace_bytes(int num_tokens, int num_topk, int num_experts) {
-    return size_t(carve_route_scratch(nullptr, num_tokens, num_topk, num_experts).bytes);
+    return size_t(route_scratch(num_tokens, num_topk, num_experts).bytes);
 }
 
 int deepep_ll_dispatch_send(const void* x, const int64_t* topk_idx, int num_tokens, int hidden, int num_topk,
@@ -551,7 +518,8 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
                             int num_ranks, int num_max_dispatch_tokens_per_rank, int row_format,
                             void* packed_recv_x, void* packed_recv_scales, int32_t* packed_recv_src_info,
                             int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
-                            int32_t* cumulative_local_expert_recv_stats, void* stream) {
+                            int32_t* cumulative_local_expert_recv_stats, int64_t expected_rows, void* workspace,
+                            size_t workspace_bytes, void* stream) {
     clear_error();
     EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
     EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
@@ -569,12 +537,40 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
     const int num_local_experts = num_experts / num_ranks;
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     EP_HOST_ASSERT(max_rows < (int64_t(1) << 31));
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    if (max_rows > kLargeBatchRows && workspace != nullptr) {
+        EP_HOST_ASSERT(workspace_bytes >= size_t(segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank)));
+        EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
+        int32_t* flat = reinterpret_cast<int32_t*>(workspace);
+        RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) +
+                                                   (((int64_t(num_experts) + 1) * 4 + 255) & ~int64_t(255)));
+        ll_segment_index_kernel<<<num_experts, kIndexThreads, 0, hs>>>(
+            0, recv_count, nullptr, num_local_experts, num_ranks, 0, num_max_dispatch_tokens_per_rank,
+            packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, flat, desc);
+        EP_LAUNCH_CHECK();
+        const int64_t data_bytes = row_data_bytes(hidden, row_format);
+        const int64_t scale_bytes = row_scale_bytes(hidden, row_format);
+        const int num_vec = int(data_bytes / 16);
+        int threads = ((num_vec + 63) / 64) * 64;
+        int extra = 64;  // one more wave for scales + source index
+        if (threads + extra > 1024) threads = 1024, extra = 0;
+        ll_rows_flat_kernel<<<flat_grid_blocks(expected_rows, max_rows, num_max_dispatch_tokens_per_rank),
+                              threads + extra, 0,
+                              hs>>>(flat, num_experts, desc, reinterpret_cast<const uint8_t*>(recv_staging),
+                                    row_stride_bytes(hidden, row_format), num_vec,
+                                    reinterpret_cast<uint8_t*>(packed_recv_x), nullptr, data_bytes,
+                                    int(scale_bytes / 4), align16(data_bytes),
+                                    scale_bytes > 0 ? reinterpret_cast<uint8_t*>(packed_recv_scales) : nullptr,
+                                    align16(data_bytes) + align16(scale_bytes), packed_recv_src_info, extra);
+        EP_LAUNCH_CHECK();
+        return 0;
+    }
     const int parts = choose_row_parts(max_rows, row_data_bytes(hidden, row_format));
     int64_t blocks = (max_rows * parts + 3) / 4;
-    const int64_t cap = max_rows > (int64_t(1) << 18) ? 4096 : 1024;
+    const int64_t cap = max_rows > kLargeBatchRows ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(num_experts + 1) * sizeof(int32_t);
-    ll_recv_kernel<<<dim3(unsigned(blocks)), 256, lds, reinterpret_cast<hipStream_t>(stream)>>>(
+    ll_recv_kernel<<<dim3(unsigned(blocks)), 256, lds, hs>>>(
         reinterpret_cast<const uint8_t*>(recv_staging), recv_count, hidden, num_local_experts, num_ranks,
         num_max_dispatch_tokens_per_rank, row_format, parts, reinterpret_cast<uint8_t*>(packed_recv_x),
         reinterpret_cast<uint8_t*>(packed_recv_scales), packed_recv_src_info, packed_recv_layout_range,

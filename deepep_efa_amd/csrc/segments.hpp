@@ -87,4 +87,154 @@ inline int choose_row_parts(int64_t max_rows, int64_t row_bytes) {
     return row_bytes > 8192 ? 4 : 2;
 }
 
+// ---------------------------------------------------------------------
+// Large batches.  A flat copy — one workgroup per row, one 16-byte vector per
+// thread, no loop — is what reaches the highest HBM rate on this GPU, but it
+// needs the row -> (source, destination) map up front.  ll_segment_index_kernel
+// builds it: one workgroup per segment scans the segment counts (<= 1024 ints)
+// and writes a descriptor {source row, destination row} for each of its rows.
+// ---------------------------------------------------------------------
+struct RowDesc {
+    int32_t src_row;  // row index in the source buffer
+    int32_t dst_row;  // >= 0: row index in the primary destination; < 0: -(1 + row) in the secondary one
+};
+
+constexpr int kIndexThreads = 1024;
+
+// Exclusive prefix over one value per thread of a 1024-thread workgroup; returns the prefix, sets total.
+__device__ __forceinline__ int block_exclusive_scan_1024(int v, int32_t* wave_totals, int& total) {
+    const int lane = lane_id(), w = int(threadIdx.x) >> 6;
+    const int incl = wave_inclusive_sum(v);
+    if (lane == kWave - 1) wave_totals[w] = incl;
+    __syncthreads();
+    int offset = incl - v;
+    total = 0;
+    for (int w2 = 0; w2 < kIndexThreads / kWave; ++w2) {
+        const int t = wave_totals[w2];
+        if (w2 < w) offset += t;
+        total += t;
+    }
+    return offset;
+}
+
+// mode 0 (dispatch receive): counts = recv_count; writes layout_range / packed_count / stats;
+//        descriptor = {staging row seg*M + j, packed row e_l*N + begin + j}.
+// mode 1 (combine send): counts and begins from layout_range;
+//        descriptor = {expert-output row e_l*N + begin + j, seg*M + j for other ranks or
+//        -(1 + (rank*E_l + e_l)*M + j) for this rank's own rows}.
+static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
+    int mode, const int32_t* __restrict__ counts32, const int64_t* __restrict__ layout_in, int num_local_experts,
+    int num_ranks, int rank, int max_tokens, int64_t* __restrict__ layout_out, int32_t* __restrict__ packed_count,
+    int32_t* __restrict__ stats, int32_t* __restrict__ flat_out, RowDesc* __restrict__ desc) {
+    __shared__ int32_t flat[kIndexThreads + 1];
+    __shared__ int32_t begin_in[kIndexThreads];
+    __shared__ int32_t wave_totals[kIndexThreads / kWave];
+    const int tid = threadIdx.x;
+    const int num_segments = num_local_experts * num_ranks;
+    int c = 0;
+    if (tid < num_segments) {
+        if (mode == 0) {
+            c = counts32[tid];
+        } else {
+            const int64_t lr = layout_in[tid];
+            c = int(lr & 0xffffffffll);
+            begin_in[tid] = int(lr >> 32);
+        }
+        c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+    }
+    int total;
+    const int prefix = block_exclusive_scan_1024(c, wave_totals, total);
+    if (tid < num_segments) flat[tid] = prefix;
+    if (tid == 0) flat[num_segments] = total;
+    __syncthreads();
+    const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
+    if (blockIdx.x == 0) {
+        for (int s = tid; s <= num_segments; s += kIndexThreads) flat_out[s] = flat[s];
+        if (mode == 0) {
+            if (tid < num_segments) {
+                const int le = tid / num_ranks;
+                const int64_t cnt = c, begin = flat[tid] - flat[le * num_ranks];
+                layout_out[tid] = cnt > 0 ? ((begin << 32) | cnt) : 0;
+            }
+            if (tid < num_local_experts) {
+                const int n = flat[(tid + 1) * num_ranks] - flat[tid * num_ranks];
+                packed_count[tid] = n;
+                if (stats != nullptr) stats[tid] += n;
+            }
+        }
+    }
+    const int seg = blockIdx.x;
+    const int le = seg / num_ranks, s = seg - le * num_ranks;
+    const int cnt = flat[seg + 1] - flat[seg];
+    const int64_t begin = mode == 0 ? flat[seg] - flat[le * num_ranks] : begin_in[seg];
+    if (mode == 1 && (begin < 0 || begin + cnt > slots_per_expert)) return;  // malformed range: emit nothing
+    for (int j = tid; j < cnt; j += kIndexThreads) {
+        RowDesc d;
+        if (mode == 0) {
+            d.src_row = seg * max_tokens + j;
+            d.dst_row = int32_t(le * slots_per_expert + begin + j);
+        } else {
+            d.src_row = int32_t(le * slots_per_expert + begin + j);
+            d.dst_row = s == rank ? -(1 + (rank * num_local_experts + le) * max_tokens + j) : seg * max_tokens + j;
+        }
+        desc[flat[seg] + j] = d;
+    }
+}
+
+// One workgroup per described row (looping only if there are more rows than workgroups).
+static __global__ __launch_bounds__(1024) void ll_rows_flat_kernel(
+    const int32_t* __restrict__ flat, int num_segments, const RowDesc* __restrict__ desc,
+    const uint8_t* __restrict__ src, int64_t src_stride, int num_vec, uint8_t* __restrict__ dst_primary,
+    uint8_t* __restrict__ dst_secondary, int64_t dst_stride, int scale_dwords, int64_t src_scale_off,
+    uint8_t* __restrict__ scale_dst, int64_t tail_off, int32_t* __restrict__ src_info, int extra_threads) {
+    const int total = flat[num_segments];
+    for (int row = blockIdx.x; row < total; row += gridDim.x) {
+        const RowDesc d = desc[row];
+        const uint8_t* s = src + int64_t(d.src_row) * src_stride;
+        uint8_t* o;
+        if (d.dst_row >= 0) {
+            if (dst_primary == nullptr) continue;
+            o = dst_primary + int64_t(d.dst_row) * dst_stride;
+        } else {
+            o = dst_secondary + int64_t(-(d.dst_row + 1)) * dst_stride;
+        }
+        const u32x4* sv = reinterpret_cast<const u32x4*>(s);
+        u32x4* ov = reinterpret_cast<u32x4*>(o);
+        // threads [0, data_threads) move the payload; when the launch carries extra threads beyond
+        // them, those move scales and the source index in the same pass instead of a second one
+        const int data_threads = extra_threads > 0 ? int(blockDim.x) - extra_threads : int(blockDim.x);
+        const int tid = threadIdx.x;
+        if (tid < data_threads)
+            for (int v = tid; v < num_vec; v += data_threads) ov[v] = sv[v];
+        if (extra_threads == 0 || tid >= data_threads) {
+            const int t2 = extra_threads > 0 ? tid - data_threads : tid;
+            const int step = extra_threads > 0 ? extra_threads : int(blockDim.x);
+            if (scale_dst != nullptr) {
+                const uint32_t* s32 = reinterpret_cast<const uint32_t*>(s + src_scale_off);
+                uint32_t* d32 = reinterpret_cast<uint32_t*>(scale_dst + int64_t(d.dst_row) * scale_dwords * 4);
+                for (int v = t2; v < scale_dwords; v += step) d32[v] = s32[v];
+            }
+            if (src_info != nullptr && t2 == step - 1)
+                src_info[d.dst_row] = *reinterpret_cast<const int32_t*>(s + tail_off);
+        }
+    }
+}
+
+__host__ __device__ inline int64_t segment_workspace_bytes(int num_experts, int max_tokens) {
+    const int64_t flat_bytes = ((int64_t(num_experts) + 1) * 4 + 255) & ~int64_t(255);
+    return flat_bytes + int64_t(num_experts) * max_tokens * int64_t(sizeof(RowDesc));
+}
+
+// Rows above this bound on E*M take the index + flat-copy pair instead of the single fused kernel.
+constexpr int64_t kLargeBatchRows = int64_t(1) << 18;
+
+inline unsigned flat_grid_blocks(int64_t expected_rows, int64_t max_rows, int max_tokens) {
+    int64_t want = expected_rows > 0 ? expected_rows : int64_t(max_tokens) * 8;
+    want += want / 8 + 64;
+    if (want > max_rows) want = max_rows;
+    if (want > (int64_t(1) << 22)) want = int64_t(1) << 22;
+    if (want < 1) want = 1;
+    return unsigned(want);
+}
+
 }  // namespace deepep

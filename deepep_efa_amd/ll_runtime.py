@@ -70,6 +70,10 @@ class LowLatencyState:
         self.send_count = torch.zeros(e, **i32)
         self.pair_slot = torch.full((m, s.num_topk), -1, **i32)
         self.workspace = torch.empty(max(256, lib.deepep_ll_dispatch_workspace_bytes(m, s.num_topk, e)), **u8)
+        # index + flat-copy scratch of the receive / combine-send kernels, only needed for large batches
+        self.segment_workspace = (torch.empty(lib.deepep_ll_segment_workspace_bytes(e, m), **u8)
+                                  if e * m > (1 << 18) else None)
+        self.expected_rows = m * s.num_topk
         if s.fmt == ROW_BF16:
             self.packed_recv_x = torch.empty((el, r * m, h), dtype=torch.bfloat16, device=device)
             self.packed_recv_scales = None
@@ -104,7 +108,9 @@ class LowLatencyState:
             _capi.ptr(self.recv_staging), _capi.ptr(self.recv_count), s.hidden, s.num_experts, s.num_ranks,
             s.max_tokens, s.fmt, _capi.ptr(self.packed_recv_x), _capi.ptr(self.packed_recv_scales),
             _capi.ptr(self.packed_recv_src_info), _capi.ptr(self.packed_recv_layout_range),
-            _capi.ptr(self.packed_recv_count), _capi.ptr(stats), current_stream_ptr()))
+            _capi.ptr(self.packed_recv_count), _capi.ptr(stats), self.expected_rows,
+            _capi.ptr(self.segment_workspace),
+            0 if self.segment_workspace is None else self.segment_workspace.numel(), current_stream_ptr()))
 
     # -- combine ----------------------------------------------------------
     def combine_send(self, x: torch.Tensor, layout_range: torch.Tensor = None) -> None:
@@ -112,7 +118,9 @@ class LowLatencyState:
         lr = self.packed_recv_layout_range if layout_range is None else layout_range
         _capi.check(self.lib.deepep_ll_combine_send(
             _capi.ptr(x), _capi.ptr(lr), s.hidden, s.num_experts, s.num_ranks, s.rank, s.max_tokens,
-            _capi.ptr(self.combine_staging), _capi.ptr(self.combine_send_slots), current_stream_ptr()))
+            _capi.ptr(self.combine_staging), _capi.ptr(self.combine_send_slots), self.expected_rows,
+            _capi.ptr(self.segment_workspace),
+            0 if self.segment_workspace is None else self.segment_workspace.numel(), current_stream_ptr()))
 
     def combine_recv(self, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor) -> None:
         s = self.shape

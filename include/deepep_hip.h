@@ -146,6 +146,9 @@ int deepep_per_token_cast_to_fp8(const void* x, int num_rows, int num_cols, int 
 /* Low-latency dispatch                                               */
 /* ------------------------------------------------------------------ */
 
+/* Bytes of the optional scratch of deepep_ll_dispatch_recv / deepep_ll_combine_send. */
+size_t deepep_ll_segment_workspace_bytes(int num_experts, int num_max_dispatch_tokens_per_rank);
+
 /* Bytes of scratch `deepep_ll_dispatch_send` needs. */
 size_t deepep_ll_dispatch_workspace_bytes(int num_tokens, int num_topk, int num_experts);
 
@@ -190,6 +193,10 @@ int deepep_ll_dispatch_send(const void* x, const int64_t* topk_idx,
  *   packed_recv_count        [E_l] int32 (out)
  *   cumulative_local_expert_recv_stats [E_l] int32, += count, or NULL
  * Rows at or beyond packed_recv_count[e] are left untouched.
+ *   expected_rows  launch-sizing hint only (0 = unknown); any value gives the same result.
+ *   workspace      deepep_ll_segment_workspace_bytes(E, M) bytes, or NULL.  With it, batches
+ *                  whose E*M exceeds 2^18 run as an index kernel plus a flat row copy (faster
+ *                  when bandwidth-bound); without it one fused kernel is used at every size.
  * Replaces ll_recv_unpack_v2 (csrc/kernels/efa_kernels.cu:2121-2231;
  * kernels :877-1389) and a2a_dispatch_recv (csrc/deep_ep.cpp:3709,
  * csrc/kernels/coop_dispatch_recv.cuh:39-304). */
@@ -199,7 +206,9 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
                             void* packed_recv_x, void* packed_recv_scales,
                             int32_t* packed_recv_src_info, int64_t* packed_recv_layout_range,
                             int32_t* packed_recv_count,
-                            int32_t* cumulative_local_expert_recv_stats, void* stream);
+                            int32_t* cumulative_local_expert_recv_stats,
+                            int64_t expected_rows, void* workspace, size_t workspace_bytes,
+                            void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Low-latency combine                                                */
@@ -214,12 +223,15 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
  *   layout_range        [E_l, R] int64 from the dispatch
  *   combine_staging     [E, M, H] bf16 (in/out)
  *   combine_send_slots  [E_l, R, M, H] bf16 (out) or NULL
+ *   expected_rows, workspace: as for deepep_ll_dispatch_recv.
  * Replaces the two torch gathers of deep_ep/buffer.py:2601-2608 and
  * a2a_combine_send (csrc/deep_ep.cpp:3804, csrc/kernels/coop_combine_send.cuh:34-275). */
 int deepep_ll_combine_send(const void* x, const int64_t* layout_range,
                            int hidden, int num_experts, int num_ranks, int rank,
                            int num_max_dispatch_tokens_per_rank,
-                           void* combine_staging, void* combine_send_slots, void* stream);
+                           void* combine_staging, void* combine_send_slots,
+                           int64_t expected_rows, void* workspace, size_t workspace_bytes,
+                           void* stream);
 
 /* Receive side: out[t,:] = bf16( sum_k [pair_slot[t,k] >= 0] * w[t,k] *
  * f32(combine_staging[topk_idx[t,k], pair_slot[t,k], :]) ), accumulated in

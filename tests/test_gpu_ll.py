@@ -89,6 +89,7 @@ def check_dispatch(st, want, fmt):
     (4, 1, 40, 512, 9, 64),    # K > 8: separate route kernel, one chunk
     (2, 1, 600, 512, 8, 16),   # T*K > 2048: chunked route + cross-chunk scan
     (4, 3, 300, 512, 11, 32),  # both
+    (8, 5, 4200, 512, 4, 64),  # E*M > 2^18: receive runs as index kernel + flat row copy
 ])
 def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e):
     x_all, topk_all, _ = make_world(r, t, h, k, e, seed=r * 100 + t, drop=min(5, t))
@@ -186,7 +187,8 @@ def test_reference_recipe_roundtrip(rt, use_fp8):
     assert diff < (9e-4 if use_fp8 else 1e-5), diff
 
 
-@pytest.mark.parametrize("r,rank,t,h,k,e", [(32, 5, 128, 7168, 8, 256), (4, 0, 16, 512, 3, 8)])
+@pytest.mark.parametrize("r,rank,t,h,k,e", [(32, 5, 128, 7168, 8, 256), (4, 0, 16, 512, 3, 8),
+                                            (8, 3, 4200, 512, 4, 64)])  # the last: large-batch combine-send path
 def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e):
     """Seeded expert outputs along the dispatch routing; combine vs the float32 chain and the float64 sum."""
     x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=31 + r, drop=10)
@@ -312,7 +314,7 @@ def test_ll_argument_errors(rt):
     assert rc != 0 and "num_tokens <= max_tokens" in lib.deepep_last_error().decode()
     # experts not divisible by ranks
     rc = lib.deepep_ll_dispatch_recv(capi.ptr(z), capi.ptr(z), 128, 9, 2, 8, 1, capi.ptr(z), capi.ptr(z), capi.ptr(z),
-                                     capi.ptr(z), capi.ptr(z), None, s)
+                                     capi.ptr(z), capi.ptr(z), None, 0, None, 0, s)
     assert rc != 0 and "num_experts % num_ranks == 0" in lib.deepep_last_error().decode()
     # workspace too small
     rc = lib.deepep_ll_dispatch_send(capi.ptr(z), capi.ptr(z), 8, 128, 2, 8, 2, 0, 8, 1, capi.ptr(z), capi.ptr(z),
