@@ -1,0 +1,114 @@
+"""Full-size skewed-routing stress on the GPU: 8192 tokens x 7168 per rank, EP=64 with 4 local experts,
+Zipf(1.2) expert popularity, 1 % of the rows scaled by 100, hot experts filling most of their slots;
+FP8 dispatch and BF16 combine round trip.
+
+The CPU oracle cannot replay 64 x 8192 x 7168 elements in seconds, so parity at this size is checked by
+(a) the integer outputs against the oracle in full (routing is regenerated from the seed on the CPU),
+(b) the payload of a random sample of received rows against the oracle's quantisation of the regenerated
+source rows, and (c) size-independent properties: segment order, count identities, and the
+identity-expert round trip combined == x * sum(w).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import deepep_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_skew_stress_full_size():
+    from deepep_efa_amd import _capi, ll_runtime, loopback
+    _capi.load()
+    assert torch.cuda.is_available(), "this test needs the MI355X"
+    free, _ = torch.cuda.mem_get_info()
+    if free < 170 * 2 ** 30:
+        pytest.skip("needs ~150 GB of free HBM")
+    r, rank, t, h, k, e, seed = 64, 0, 8192, 7168, 8, 256, 4242
+    epr, n_slots = e // r, r * t
+    shape = ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8)
+    st = ll_runtime.LowLatencyState(shape)
+    world = loopback.LoopbackWorld(r, rank, seed=seed)
+    world.synthesise(t, h, k, e, popularity="zipf", outlier_period=100)
+    x, topk = world.own_inputs()
+    st.dispatch_send(x, topk)
+    world.dispatch_from_peers(st)
+    st.dispatch_recv()
+    torch.cuda.synchronize()
+
+    # (a) integer outputs against the oracle, in full
+    topk_all = O.synth_topk_idx(O.zipf_cdf(e), np.arange(r), t, k, seed)
+    assert torch.equal(world.topk_idx_all.cpu(), topk_all)
+    flat = topk_all.numpy().reshape(r, t * k)
+    count = st.packed_recv_count.cpu()
+    layout = st.packed_recv_layout_range.cpu()
+    src_info = st.packed_recv_src_info.cpu().numpy()
+    seg_tokens = {}
+    for le in range(epr):
+        expert = rank * epr + le
+        begin = 0
+        for s in range(r):
+            tok = (np.nonzero(flat[s] == expert)[0] // k).astype(np.int32)
+            seg_tokens[(le, s)] = (begin, tok)
+            want = ((begin << 32) | len(tok)) if len(tok) else 0
+            assert int(layout[le, s]) == want, (le, s)
+            assert np.array_equal(src_info[le, begin:begin + len(tok)], tok), (le, s)
+            assert (np.diff(tok) >= 0).all()
+            begin += len(tok)
+        assert int(count[le]) == begin
+    assert int(count[0]) > n_slots // 2, "the hottest expert should fill over half of its slots"
+    send_count, pair_slot = O.route(topk_all[rank], e, t)
+    assert torch.equal(st.send_count.cpu(), send_count)
+    assert torch.equal(st.pair_slot.cpu(), pair_slot)
+
+    # (b) payload of a random sample of received rows
+    rng = np.random.default_rng(1)
+    picks = []
+    for _ in range(1500):
+        le, s = int(rng.integers(epr)), int(rng.integers(r))
+        begin, tok = seg_tokens[(le, s)]
+        if len(tok) == 0:
+            continue
+        j = int(rng.integers(len(tok)))
+        picks.append((le, begin + j, s, int(tok[j])))
+    keys = np.array([s * t + tk for (_, _, s, tk) in picks], dtype=np.uint32)
+    rows = O.synth_bf16_rows(keys, h, seed, outlier_period=100)
+    assert rows.float().abs().amax(1).max().item() > 100, "the sample should contain outlier rows"
+    wq, ws = O.per_token_cast_to_fp8(rows)
+    idx_le = torch.tensor([p[0] for p in picks])
+    idx_slot = torch.tensor([p[1] for p in picks])
+    got_q = st.packed_recv_x.view(torch.uint8)[idx_le.cuda(), idx_slot.cuda()].cpu()
+    got_s = st.packed_recv_scales[idx_le.cuda(), idx_slot.cuda()].cpu()
+    assert torch.equal(got_q, wq.view(torch.uint8))
+    assert torch.equal(got_s, ws)
+
+    # (c) identity experts: every pair gets back the dequantised row, combined == x * sum(w)
+    y = torch.empty((epr, n_slots, h), dtype=torch.bfloat16, device="cuda")
+    step = 32768
+    for le in range(epr):
+        n = int(count[le])
+        for b0 in range(0, n, step):
+            b1 = min(n, b0 + step)
+            q = st.packed_recv_x[le, b0:b1].float().view(b1 - b0, h // 128, 128)
+            y[le, b0:b1] = (q * st.packed_recv_scales[le, b0:b1].unsqueeze(-1)).view(b1 - b0, h).to(torch.bfloat16)
+    world.combine_from_peers(st, mode=0)
+    st.combine_send(y)
+    w = torch.softmax(torch.randn((t, k), generator=torch.Generator().manual_seed(2)), dim=-1).cuda()
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    st.combine_recv(topk, w, out)
+    torch.cuda.synchronize()
+    want = x.double() * w.double().sum(1, keepdim=True)
+    got = out.double()
+    assert not torch.isnan(got).any()
+    a, b = want + 1, got + 1
+    diff = float(1 - 2 * (a * b).sum() / (a * a + b * b).sum())
+    assert diff < 9e-4, diff
+    # the same rows through the float32 chain definition, on a sample of tokens
+    sample = torch.arange(0, t, 257)
+    pair_rows = torch.zeros((len(sample), k, h), dtype=torch.bfloat16)
+    xq, xs = O.per_token_cast_to_fp8(x[sample.cuda()].cpu())
+    back = O.per_token_cast_back(xq, xs)
+    live = (topk[sample.cuda()].cpu() >= 0)
+    pair_rows[:] = back.unsqueeze(1)
+    chain = O.ll_combine_f32_chain(pair_rows, w[sample.cuda()].cpu(), live)
+    assert torch.equal(out[sample.cuda()].cpu().view(torch.int16), chain.view(torch.int16))
