@@ -335,6 +335,10 @@ def main():
     traffic = read_traffic_summary(dom)
     if traffic is not None and (t, h, k, e, r) == (128, 7168, 8, 256, 32):
         result["roofline"]["traffic"] = traffic
+    cpu_inputs = None
+    if not args.no_cpu_baseline:  # host copies for the CPU leg, taken before the device buffers are released
+        cpu_inputs = (x.cpu(), topk.cpu(), weights.cpu(), st.recv_staging.view(epr, r, t, st.stride).cpu(),
+                      st.recv_count.view(epr, r).cpu())
     if not args.no_pack:
         del st, y
         torch.cuda.empty_cache()
@@ -344,9 +348,7 @@ def main():
     if not args.no_cpu_baseline:
         from oracle import cpu_baseline
         torch.cuda.synchronize()
-        staged = st.recv_staging.view(epr, r, t, st.stride).cpu()
-        cpu = cpu_baseline.CpuRankStep(x.cpu(), topk.cpu(), weights.cpu(), staged, st.recv_count.view(epr, r).cpu(),
-                                       e, r, rank, t)
+        cpu = cpu_baseline.CpuRankStep(*cpu_inputs, e, r, rank, t)
         med, threads, runs = cpu_baseline.time_cpu_step(cpu, budget_s=15.0)
         result["cpu_baseline"] = {"value": round(med * 1e6, 1), "unit": "us", "cores": threads, "kind": "port",
                                   "sample": f"the same rank-{rank} dispatch+combine step in torch on the host, "
