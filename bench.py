@@ -24,15 +24,22 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 
-def algorithmic_bytes(t, h, k, p, rv, stride, e, r):
-    """Bytes each kernel must move (reads + writes), from the generated routing.
-    p = live (token,k) pairs of this rank, rv = rows this rank receives."""
+def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0):
+    """Bytes each entry point must move (reads + writes), from the generated routing.
+    p = live (token,k) pairs of this rank, rv = rows this rank receives, own = rows it sends to itself.
+    The one-call entries handle the own rows once: quantised straight into the packed tensors on dispatch,
+    read straight from the expert outputs on combine."""
     g = h // 128
+    packed = h + 4 * g + 4
+    small = e * 4 + (e // r) * r * 8 + (e // r) * 4
     return {
         "dispatch_send": t * 2 * h + t * k * 8 + p * stride + t * k * 4 + e * 4,
-        "dispatch_recv": rv * stride + rv * (h + 4 * g + 4) + e * 4 + (e // r) * r * 8 + (e // r) * 4,
+        "dispatch_recv": rv * stride + rv * packed + small,
         "combine_send": rv * 2 * h * 2 + (e // r) * r * 8,
         "combine_recv": p * 2 * h + t * k * 16 + t * 2 * h,
+        "dispatch": (t * 2 * h + t * k * 8 + (p - own) * stride + own * packed + t * k * 4 + e * 4
+                     + (rv - own) * (stride + packed) + small),
+        "combine": (rv - own) * 2 * h * 2 + (e // r) * r * 8 + p * 2 * h + t * k * 16 + t * 2 * h,
     }
 
 
@@ -239,17 +246,26 @@ def main():
     torch.cuda.synchronize()
     p = int((st.pair_slot[:t] >= 0).sum())
     rv = int(st.packed_recv_count.sum())
+    own = int((st.packed_recv_layout_range[:, rank] & 0xFFFFFFFF).sum())
 
     calls = {
+        "dispatch": lambda: st.dispatch(x, topk),  # send + receive phase, one launch at this size
+        "combine": lambda: st.combine(y, topk, weights, out),  # row return + reduce, one launch at this size
         "dispatch_send": lambda: st.dispatch_send(x, topk),
         "dispatch_recv": lambda: st.dispatch_recv(),
         "combine_send": lambda: st.combine_send(y),
         "combine_recv": lambda: st.combine_recv(topk, weights, out),
     }
+    step_calls = ("dispatch", "combine")  # what deep_ep.Buffer.low_latency_dispatch / _combine launch
+    phase_calls = ("dispatch_send", "dispatch_recv", "combine_send", "combine_recv")
 
     def step():
-        for fn in calls.values():
-            fn()
+        for name in step_calls:
+            calls[name]()
+
+    def step_by_phase():
+        for name in phase_calls:
+            calls[name]()
 
     for _ in range(args.warmup):
         step()
@@ -263,6 +279,15 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
     us_per_step = ev0.elapsed_time(ev1) * 1e3 / args.steps
+    for _ in range(10):
+        step_by_phase()
+    torch.cuda.synchronize()
+    ev0.record()
+    for _ in range(args.steps):
+        step_by_phase()
+    ev1.record()
+    torch.cuda.synchronize()
+    us_per_phase_step = ev0.elapsed_time(ev1) * 1e3 / args.steps
 
     # per entry point: the same call `steps` times back to back between two events.  Consecutive
     # launches on one stream leave well under a microsecond between kernels on this GPU, so the
@@ -302,10 +327,10 @@ def main():
         except Exception as exc:  # graph capture is an extra, never the headline
             graph_us = f"unavailable: {type(exc).__name__}"
 
-    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r)
+    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r, own)
     kernels = {n: {"us": round(per_call[n], 2), "bytes": nbytes[n],
                    "GBps": round(nbytes[n] / per_call[n] / 1e3, 1)} for n in calls}
-    dom = max(per_call, key=per_call.get)
+    dom = max(step_calls, key=per_call.get)
     achieved = nbytes[dom] / per_call[dom] / 1e3
     result = {
         "metric": "us per LL dispatch+combine (128 tok,7168,top-8); pack/combine HBM GB/s",
@@ -323,8 +348,10 @@ def main():
         "config": {"workload": "LL dispatch+combine, one GPU's share of EP=32: 128 tokens x 7168, top-8 of 256 "
                                "experts, 8 local experts; 31 peers synthesised in HBM from a seed",
                    "tokens": t, "hidden": h, "topk": k, "experts": e, "ranks": r, "rank": rank,
-                   "pairs_sent": p, "rows_received": rv},
-        "kernel_time_us": round(sum(per_call.values()), 2),
+                   "pairs_sent": p, "rows_received": rv, "rows_to_own_experts": own,
+                   "launches_per_step": 2},
+        "kernel_time_us": round(sum(per_call[n] for n in step_calls), 2),
+        "step_by_phase_us": round(us_per_phase_step, 2),  # the same step as four launches
         "graph_replay_us": graph_us if not isinstance(graph_us, float) else round(graph_us, 2),
         "host_wall_us_per_step": round(wall * 1e6 / args.steps, 2),
         "kernels": kernels,

@@ -67,6 +67,13 @@ __device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u,
 // stays in SGPRs and row addresses become scalar loads.
 __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6); }
 
+// A 64-bit value every lane of the wave holds alike, moved to scalar registers.
+__device__ __forceinline__ uint64_t wave_uniform_u64(uint64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(uint32_t(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(uint32_t(v >> 32));
+    return (uint64_t(hi) << 32) | lo;
+}
+
 __device__ __forceinline__ uint64_t lanes_below(int lane) { return (uint64_t(1) << lane) - 1; }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }

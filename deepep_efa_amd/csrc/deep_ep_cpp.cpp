@@ -477,21 +477,18 @@ struct Buffer {
         auto& c = get_ll_cache(num_max_dispatch_tokens_per_rank, hidden, num_topk, num_experts, fmt);
         auto stream = current_stream();
 
-        abi_check(deepep_ll_dispatch_send(
+        stage_peer_rows(c);  // what the exchange would have delivered
+        // send and receive phase in one call (one kernel launch for decode-sized batches)
+        abi_check(deepep_ll_dispatch(
             x.data_ptr(), topk_idx.data_ptr<int64_t>(), num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
             num_max_dispatch_tokens_per_rank, fmt, c.recv_staging.data_ptr(), c.recv_count.data_ptr<int>(),
             c.send_slots.data_ptr(), c.send_count.data_ptr<int>(), c.pair_slot.data_ptr<int>(),
-            c.workspace.data_ptr(), size_t(c.workspace.numel()), stream));
-        stage_peer_rows(c);  // what the exchange would have delivered
-        abi_check(deepep_ll_dispatch_recv(
-            c.recv_staging.data_ptr(), c.recv_count.data_ptr<int>(), hidden, num_experts, num_ranks,
-            num_max_dispatch_tokens_per_rank, fmt, c.packed_recv_x.data_ptr(),
-            c.packed_recv_scales.defined() ? c.packed_recv_scales.data_ptr() : nullptr,
+            c.packed_recv_x.data_ptr(), c.packed_recv_scales.defined() ? c.packed_recv_scales.data_ptr() : nullptr,
             c.packed_recv_src_info.data_ptr<int>(), c.packed_recv_layout_range.data_ptr<int64_t>(),
             c.packed_recv_count.data_ptr<int>(),
             cumulative_local_expert_recv_stats.has_value() ? cumulative_local_expert_recv_stats->data_ptr<int>() : nullptr,
-            int64_t(num_max_dispatch_tokens_per_rank) * num_topk,
-            c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
+            int64_t(num_max_dispatch_tokens_per_rank) * num_topk, c.workspace.data_ptr(),
+            size_t(c.workspace.numel()), c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
             c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));
         c.dispatched = true;
 
@@ -558,22 +555,19 @@ struct Buffer {
             combined_x = c.combined_x.narrow(0, 0, num_combined_tokens);
         }
 
-        abi_check(deepep_ll_combine_send(src.data_ptr(), layout_range.data_ptr<int64_t>(), hidden, num_experts,
-                                         num_ranks, rank, num_max_dispatch_tokens_per_rank, c.combine_staging.data_ptr(),
-                                         c.combine_send_slots.data_ptr(),
-                                         int64_t(num_max_dispatch_tokens_per_rank) * num_topk,
-                                         c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
-                                         c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0,
-                                         stream));
         if (world_x.has_value())  // what the remote experts would have returned
             abi_check(deepep_loopback_combine_from_peers(c.send_slots.data_ptr(), c.send_count.data_ptr<int>(), hidden,
                                                          num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,
                                                          c.row_format, combine_peer_mode, combine_peer_seed,
                                                          c.combine_staging.data_ptr(), stream));
-        abi_check(deepep_ll_combine_recv(c.combine_staging.data_ptr(), topk_idx.data_ptr<int64_t>(),
-                                         topk_weights.data_ptr<float>(), c.pair_slot.data_ptr<int>(),
-                                         num_combined_tokens, hidden, num_topk, num_experts,
-                                         num_max_dispatch_tokens_per_rank, combined_x.data_ptr(), stream));
+        // row return and weighted reduce in one call (one kernel launch for decode-sized batches)
+        abi_check(deepep_ll_combine(src.data_ptr(), layout_range.data_ptr<int64_t>(), topk_idx.data_ptr<int64_t>(),
+                                    topk_weights.data_ptr<float>(), c.pair_slot.data_ptr<int>(), num_combined_tokens,
+                                    hidden, num_topk, num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,
+                                    c.combine_staging.data_ptr(), c.combine_send_slots.data_ptr(),
+                                    combined_x.data_ptr(), int64_t(num_max_dispatch_tokens_per_rank) * num_topk,
+                                    c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
+                                    c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));
 
         std::optional<EventHandle> event;
         if (async) event = EventHandle();

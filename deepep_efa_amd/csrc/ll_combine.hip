@@ -13,37 +13,48 @@
 namespace deepep {
 
 // ---------------------------------------------------------------------
-// Send side: one wave per live row, rows enumerated segment by segment in
+// Send side: one wave per live row part, rows enumerated segment by segment in
 // arrival order (reference: deep_ep/buffer.py:2601-2608 gathers
 // x[recv_expert_ids, recv_expert_pos] and un-sorts to arrival order).
+// skip_own: the rows owed to this rank itself are left where they are (the
+// single-launch combine reads them from x directly).
 // ---------------------------------------------------------------------
-__global__ __launch_bounds__(256) void ll_combine_send_kernel(
-    const uint8_t* __restrict__ x, const int64_t* __restrict__ layout_range, int hidden, int num_local_experts,
-    int num_ranks, int rank, int max_tokens, int parts, uint8_t* __restrict__ combine_staging,
-    uint8_t* __restrict__ combine_send_slots) {
-    extern __shared__ int32_t flat[];  // [num_segments + 1] then begin[num_segments]
-    __shared__ int32_t wave_totals[4];
+struct CombineSendArgs {
+    const uint8_t* x;
+    const int64_t* layout_range;
+    int hidden, num_local_experts, num_ranks, rank, max_tokens, parts;
+    uint8_t* combine_staging;
+    uint8_t* combine_send_slots;
+};
+
+// flat: [2 * num_segments + 1] ints; wave_totals: 16 ints.
+__device__ __forceinline__ void combine_send_rows(const CombineSendArgs& a, int block, int num_blocks, bool skip_own,
+                                                  int32_t* flat, int32_t* wave_totals) {
     const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
-    const int num_segments = num_local_experts * num_ranks;
+    const int threads = blockDim.x, waves = threads >> 6;
+    const int num_ranks = a.num_ranks, max_tokens = a.max_tokens;
+    const int num_segments = a.num_local_experts * num_ranks;
     int32_t* begin = flat + num_segments + 1;
 
-    for (int s = tid; s < num_segments; s += 256) {
-        const int64_t lr = layout_range[s];
+    for (int s = tid; s < num_segments; s += threads) {
+        const int64_t lr = a.layout_range[s];
         int c = int(lr & 0xffffffffll);
         c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+        if (skip_own && s % num_ranks == a.rank) c = 0;
         flat[s] = c;
         begin[s] = int(lr >> 32);
     }
     __syncthreads();
-    block_exclusive_scan_256(flat, num_segments, wave_totals);
+    block_exclusive_scan(flat, num_segments, wave_totals);
     const int total_rows = flat[num_segments];
 
-    const int64_t row_bytes = int64_t(hidden) * 2;
+    const int64_t row_bytes = int64_t(a.hidden) * 2;
     const int num_vec = int(row_bytes / 16);
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
-    const int64_t waves_total = int64_t(gridDim.x) * 4;
+    const int64_t waves_total = int64_t(num_blocks) * waves;
+    const int parts = a.parts;
 
-    for (int64_t item = blockIdx.x * 4 + w; item < int64_t(total_rows) * parts; item += waves_total) {
+    for (int64_t item = int64_t(block) * waves + w; item < int64_t(total_rows) * parts; item += waves_total) {
         const int row = int(item / parts), part = int(item - int64_t(row) * parts);
         const int seg = __builtin_amdgcn_readfirstlane(find_segment(flat, num_segments, row));
         const int j = row - __builtin_amdgcn_readfirstlane(flat[seg]);
@@ -51,12 +62,12 @@ __global__ __launch_bounds__(256) void ll_combine_send_kernel(
         const int s = seg - le * num_ranks;
         const int b = __builtin_amdgcn_readfirstlane(begin[seg]);
         if (b < 0 || int64_t(b) + j >= slots_per_expert) continue;  // malformed range: never read past the expert
-        const uint8_t* src = x + (int64_t(le) * slots_per_expert + b + j) * row_bytes;
+        const uint8_t* src = a.x + (int64_t(le) * slots_per_expert + b + j) * row_bytes;
         uint8_t* dst;
-        if (s == rank)
-            dst = combine_staging + ((int64_t(rank) * num_local_experts + le) * max_tokens + j) * row_bytes;
-        else if (combine_send_slots != nullptr)
-            dst = combine_send_slots + (int64_t(seg) * max_tokens + j) * row_bytes;
+        if (s == a.rank)
+            dst = a.combine_staging + ((int64_t(a.rank) * a.num_local_experts + le) * max_tokens + j) * row_bytes;
+        else if (a.combine_send_slots != nullptr)
+            dst = a.combine_send_slots + (int64_t(seg) * max_tokens + j) * row_bytes;
         else
             continue;
         int v_begin, v_end;
@@ -65,25 +76,42 @@ __global__ __launch_bounds__(256) void ll_combine_send_kernel(
     }
 }
 
+__global__ __launch_bounds__(256) void ll_combine_send_kernel(CombineSendArgs a) {
+    extern __shared__ int32_t flat[];  // [num_segments + 1] then begin[num_segments]
+    __shared__ int32_t wave_totals[kMaxBlockWaves];
+    combine_send_rows(a, blockIdx.x, gridDim.x, false, flat, wave_totals);
+}
+
 // ---------------------------------------------------------------------
 // Receive side: one wave = one (token, 1 KiB piece of the output row).
 // All K source vectors are loaded before the FMA chain so K 16-byte loads
 // are in flight per lane; accumulation order is k = 0..K-1, float32 FMA,
 // one rounding to bf16 at the end
 // (reference: csrc/kernels/coop_combine_recv.cuh:222-260).
+// own_begin != null (single-launch combine): the answers of this rank's own
+// experts are read from the expert-output tensor own_x at
+// [e_l][own_begin[e_l] + slot] instead of the staging area.
 // ---------------------------------------------------------------------
-__global__ __launch_bounds__(256) void ll_combine_recv_kernel(
-    const uint8_t* __restrict__ combine_staging, const int64_t* __restrict__ topk_idx,
-    const float* __restrict__ topk_weights, const int32_t* __restrict__ pair_slot, int num_tokens, int hidden,
-    int num_topk, int num_experts, int max_tokens, int pieces_per_row, uint8_t* __restrict__ out) {
+struct CombineRecvArgs {
+    const uint8_t* combine_staging;
+    const int64_t* topk_idx;
+    const float* topk_weights;
+    const int32_t* pair_slot;
+    int num_tokens, hidden, num_topk, num_experts, max_tokens, pieces_per_row;
+    uint8_t* out;
+};
+
+__device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int64_t item, const uint8_t* own_x,
+                                                   const int32_t* own_begin, int own_first_expert,
+                                                   int num_local_experts, int64_t slots_per_expert) {
     const int lane = lane_id();
-    const int64_t item = int64_t(blockIdx.x) * 4 + wave_in_block();
-    if (item >= int64_t(num_tokens) * pieces_per_row) return;
-    const int t = int(item / pieces_per_row);
-    const int piece = int(item - int64_t(t) * pieces_per_row);
-    const int64_t row_bytes = int64_t(hidden) * 2;
+    if (item >= int64_t(a.num_tokens) * a.pieces_per_row) return;
+    const int t = int(item / a.pieces_per_row);
+    const int piece = int(item - int64_t(t) * a.pieces_per_row);
+    const int64_t row_bytes = int64_t(a.hidden) * 2;
     const int64_t off = int64_t(piece) * 1024 + lane * 16;
     const bool lane_live = off < row_bytes;
+    const int num_topk = a.num_topk;
 
     float acc[8];
 #pragma unroll
@@ -99,14 +127,22 @@ __global__ __launch_bounds__(256) void ll_combine_recv_kernel(
             live[u] = false;
             wgt[u] = 0.0f;
             if (k < num_topk) {
-                const int slot = pair_slot[int64_t(t) * num_topk + k];
-                const int64_t e = topk_idx[int64_t(t) * num_topk + k];
-                if (slot >= 0 && slot < max_tokens && e >= 0 && e < num_experts) {
-                    live[u] = true;
-                    wgt[u] = topk_weights[int64_t(t) * num_topk + k];
-                    if (lane_live)
-                        v[u] = *reinterpret_cast<const u32x4*>(combine_staging +
-                                                               (e * max_tokens + slot) * row_bytes + off);
+                const int slot = a.pair_slot[int64_t(t) * num_topk + k];
+                const int64_t e = a.topk_idx[int64_t(t) * num_topk + k];
+                if (slot >= 0 && slot < a.max_tokens && e >= 0 && e < a.num_experts) {
+                    const uint8_t* row = a.combine_staging + (e * a.max_tokens + slot) * row_bytes;
+                    bool ok = true;
+                    const int64_t le = e - own_first_expert;
+                    if (own_begin != nullptr && le >= 0 && le < num_local_experts) {
+                        const int64_t pos = int64_t(own_begin[le]) + slot;
+                        ok = own_begin[le] >= 0 && pos < slots_per_expert;
+                        row = own_x + (le * slots_per_expert + pos) * row_bytes;
+                    }
+                    if (ok) {
+                        live[u] = true;
+                        wgt[u] = a.topk_weights[int64_t(t) * num_topk + k];
+                        if (lane_live) v[u] = *reinterpret_cast<const u32x4*>(row + off);
+                    }
                 }
             }
         }
@@ -124,8 +160,95 @@ __global__ __launch_bounds__(256) void ll_combine_recv_kernel(
         u32x4 o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
-        *reinterpret_cast<u32x4*>(out + int64_t(t) * row_bytes + off) = o;
+        *reinterpret_cast<u32x4*>(a.out + int64_t(t) * row_bytes + off) = o;
     }
+}
+
+__global__ __launch_bounds__(256) void ll_combine_recv_kernel(CombineRecvArgs a) {
+    combine_recv_piece(a, int64_t(blockIdx.x) * 4 + wave_in_block(), nullptr, nullptr, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------
+// Single-launch combine for small batches (E*M <= 2^18): the reduce workgroups
+// and the row-return workgroups of the two kernels above in one grid.  No
+// workgroup waits on another: the reduce reads the answers of this rank's own
+// experts straight from x (layout_range says where each segment begins), so the
+// row return only has to move the rows owed to other ranks.
+// (The reference's combine is one kernel with a send and a receive phase as
+// well: csrc/kernels/coop_combine_send.cuh:37, coop_combine_recv.cuh:72.)
+// ---------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ll_combine_fused_kernel(CombineSendArgs sa, CombineRecvArgs ra,
+                                                               int num_recv_blocks) {
+    extern __shared__ int32_t dyn_lds[];  // reduce: own_begin[E_l]; row return: [2 * segments + 1]
+    __shared__ int32_t wave_totals[kMaxBlockWaves];
+    const int block = blockIdx.x;
+    if (block < num_recv_blocks) {
+        for (int le = threadIdx.x; le < sa.num_local_experts; le += blockDim.x) {
+            const int64_t lr = sa.layout_range[le * sa.num_ranks + sa.rank];
+            dyn_lds[le] = (lr & 0xffffffffll) > 0 ? int(lr >> 32) : 0;
+        }
+        __syncthreads();
+        combine_recv_piece(ra, int64_t(block) * 4 + wave_in_block(), sa.x, dyn_lds, sa.rank * sa.num_local_experts,
+                           sa.num_local_experts, int64_t(sa.max_tokens) * sa.num_ranks);
+    } else {
+        combine_send_rows(sa, block - num_recv_blocks, int(gridDim.x) - num_recv_blocks, true, dyn_lds, wave_totals);
+    }
+}
+
+static CombineSendArgs make_combine_send_args(const void* x, const int64_t* layout_range, int hidden, int num_experts,
+                                              int num_ranks, int rank, int max_tokens, void* combine_staging,
+                                              void* combine_send_slots) {
+    CombineSendArgs sa;
+    sa.x = reinterpret_cast<const uint8_t*>(x);
+    sa.layout_range = layout_range;
+    sa.hidden = hidden, sa.num_local_experts = num_experts / num_ranks, sa.num_ranks = num_ranks, sa.rank = rank;
+    sa.max_tokens = max_tokens;
+    sa.parts = choose_row_parts(int64_t(num_experts) * max_tokens, int64_t(hidden) * 2);
+    sa.combine_staging = reinterpret_cast<uint8_t*>(combine_staging);
+    sa.combine_send_slots = reinterpret_cast<uint8_t*>(combine_send_slots);
+    return sa;
+}
+
+static CombineRecvArgs make_combine_recv_args(const void* combine_staging, const int64_t* topk_idx,
+                                              const float* topk_weights, const int32_t* pair_slot, int num_tokens,
+                                              int hidden, int num_topk, int num_experts, int max_tokens, void* out) {
+    CombineRecvArgs ra;
+    ra.combine_staging = reinterpret_cast<const uint8_t*>(combine_staging);
+    ra.topk_idx = topk_idx, ra.topk_weights = topk_weights, ra.pair_slot = pair_slot;
+    ra.num_tokens = num_tokens, ra.hidden = hidden, ra.num_topk = num_topk, ra.num_experts = num_experts;
+    ra.max_tokens = max_tokens, ra.pieces_per_row = (hidden * 2 + 1023) / 1024;
+    ra.out = reinterpret_cast<uint8_t*>(out);
+    return ra;
+}
+
+static int check_combine_send_args(const void* x, const int64_t* layout_range, int hidden, int num_experts,
+                                   int num_ranks, int rank, int max_tokens, const void* combine_staging,
+                                   const void* combine_send_slots) {
+    EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
+    EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
+    EP_HOST_ASSERT(rank >= 0 && rank < num_ranks);
+    EP_HOST_ASSERT(max_tokens > 0);
+    EP_HOST_ASSERT(num_experts <= 1024);
+    EP_HOST_ASSERT(x != nullptr && layout_range != nullptr && combine_staging != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combine_staging) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combine_send_slots) & 15) == 0);
+    EP_HOST_ASSERT(int64_t(num_experts) * max_tokens < (int64_t(1) << 31));
+    return 0;
+}
+
+static int check_combine_recv_args(const void* combine_staging, const int64_t* topk_idx, const float* topk_weights,
+                                   const int32_t* pair_slot, int num_tokens, int hidden, int num_topk,
+                                   int num_experts, int max_tokens, const void* out) {
+    EP_HOST_ASSERT(num_tokens >= 0 && hidden > 0 && hidden % 128 == 0 && num_topk > 0);
+    EP_HOST_ASSERT(num_experts > 0 && max_tokens > 0);
+    if (num_tokens == 0) return 0;
+    EP_HOST_ASSERT(combine_staging != nullptr && topk_idx != nullptr && topk_weights != nullptr &&
+                   pair_slot != nullptr && out != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combine_staging) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(out) & 15) == 0);
+    EP_HOST_ASSERT((int64_t(num_tokens) * ((hidden * 2 + 1023) / 1024) + 3) / 4 < (int64_t(1) << 31));
+    return 0;
 }
 
 }  // namespace deepep
@@ -139,18 +262,11 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
                            void* combine_send_slots, int64_t expected_rows, void* workspace, size_t workspace_bytes,
                            void* stream) {
     clear_error();
-    EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
-    EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
-    EP_HOST_ASSERT(rank >= 0 && rank < num_ranks);
-    EP_HOST_ASSERT(num_max_dispatch_tokens_per_rank > 0);
-    EP_HOST_ASSERT(num_experts <= 1024);
-    EP_HOST_ASSERT(x != nullptr && layout_range != nullptr && combine_staging != nullptr);
-    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
-    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combine_staging) & 15) == 0);
-    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combine_send_slots) & 15) == 0);
+    if (int rc = check_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
+                                         num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots))
+        return rc;
     const int num_local_experts = num_experts / num_ranks;
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
-    EP_HOST_ASSERT(max_rows < (int64_t(1) << 31));
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
     if (max_rows > kLargeBatchRows && workspace != nullptr) {
         EP_HOST_ASSERT(workspace_bytes >= size_t(segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank)));
@@ -173,15 +289,14 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
         EP_LAUNCH_CHECK();
         return 0;
     }
-    const int parts = choose_row_parts(max_rows, int64_t(hidden) * 2);
-    int64_t blocks = (max_rows * parts + 3) / 4;
+    const CombineSendArgs sa = make_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
+                                                      num_max_dispatch_tokens_per_rank, combine_staging,
+                                                      combine_send_slots);
+    int64_t blocks = (max_rows * sa.parts + 3) / 4;
     const int64_t cap = max_rows > kLargeBatchRows ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(2 * num_experts + 1) * sizeof(int32_t);
-    ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, lds, hs>>>(
-        reinterpret_cast<const uint8_t*>(x), layout_range, hidden, num_local_experts, num_ranks, rank,
-        num_max_dispatch_tokens_per_rank, parts, reinterpret_cast<uint8_t*>(combine_staging),
-        reinterpret_cast<uint8_t*>(combine_send_slots));
+    ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, lds, hs>>>(sa);
     EP_LAUNCH_CHECK();
     return 0;
 }
@@ -190,19 +305,58 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
                            const int32_t* pair_slot, int num_tokens, int hidden, int num_topk, int num_experts,
                            int num_max_dispatch_tokens_per_rank, void* out, void* stream) {
     clear_error();
-    EP_HOST_ASSERT(num_tokens >= 0 && hidden > 0 && hidden % 128 == 0 && num_topk > 0);
-    EP_HOST_ASSERT(num_experts > 0 && num_max_dispatch_tokens_per_rank > 0);
+    if (int rc = check_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden,
+                                         num_topk, num_experts, num_max_dispatch_tokens_per_rank, out))
+        return rc;
     if (num_tokens == 0) return 0;
-    EP_HOST_ASSERT(combine_staging != nullptr && topk_idx != nullptr && topk_weights != nullptr &&
-                   pair_slot != nullptr && out != nullptr);
-    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combine_staging) & 15) == 0);
-    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(out) & 15) == 0);
-    const int pieces = (hidden * 2 + 1023) / 1024;
-    const int64_t blocks = (int64_t(num_tokens) * pieces + 3) / 4;
-    EP_HOST_ASSERT(blocks < (int64_t(1) << 31));
-    ll_combine_recv_kernel<<<dim3(unsigned(blocks)), 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(
-        reinterpret_cast<const uint8_t*>(combine_staging), topk_idx, topk_weights, pair_slot, num_tokens, hidden,
-        num_topk, num_experts, num_max_dispatch_tokens_per_rank, pieces, reinterpret_cast<uint8_t*>(out));
+    const CombineRecvArgs ra = make_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens,
+                                                      hidden, num_topk, num_experts,
+                                                      num_max_dispatch_tokens_per_rank, out);
+    const int64_t blocks = (int64_t(num_tokens) * ra.pieces_per_row + 3) / 4;
+    ll_combine_recv_kernel<<<dim3(unsigned(blocks)), 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(ra);
+    EP_LAUNCH_CHECK();
+    return 0;
+}
+
+int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t* topk_idx, const float* topk_weights,
+                      const int32_t* pair_slot, int num_tokens, int hidden, int num_topk, int num_experts,
+                      int num_ranks, int rank, int num_max_dispatch_tokens_per_rank, void* combine_staging,
+                      void* combine_send_slots, void* out, int64_t expected_rows, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+    clear_error();
+    const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
+    if (max_rows > kLargeBatchRows) {  // the two phases back to back
+        if (int rc = deepep_ll_combine_send(x, layout_range, hidden, num_experts, num_ranks, rank,
+                                            num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots,
+                                            expected_rows, workspace, workspace_bytes, stream))
+            return rc;
+        return deepep_ll_combine_recv(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden, num_topk,
+                                      num_experts, num_max_dispatch_tokens_per_rank, out, stream);
+    }
+    if (int rc = check_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
+                                         num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots))
+        return rc;
+    if (int rc = check_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden,
+                                         num_topk, num_experts, num_max_dispatch_tokens_per_rank, out))
+        return rc;
+    const CombineSendArgs sa = make_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
+                                                      num_max_dispatch_tokens_per_rank, combine_staging,
+                                                      combine_send_slots);
+    const CombineRecvArgs ra = make_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens,
+                                                      hidden, num_topk, num_experts,
+                                                      num_max_dispatch_tokens_per_rank, out);
+    const int64_t recv_blocks = (int64_t(num_tokens) * ra.pieces_per_row + 3) / 4;
+    int64_t rows = expected_rows > 0 ? expected_rows : int64_t(num_max_dispatch_tokens_per_rank) * num_topk;
+    rows += rows / 8 + 16;
+    if (rows > max_rows) rows = max_rows;
+    int64_t send_blocks = combine_send_slots != nullptr ? (rows * sa.parts + 3) / 4 : 0;
+    if (send_blocks > 1024) send_blocks = 1024;
+    if (recv_blocks + send_blocks == 0) return 0;
+    const size_t need_send = size_t(2 * num_experts + 1) * sizeof(int32_t);
+    const size_t need_recv = size_t(sa.num_local_experts) * sizeof(int32_t);
+    const size_t lds = need_send > need_recv ? need_send : need_recv;
+    ll_combine_fused_kernel<<<dim3(unsigned(recv_blocks + send_blocks)), 256, lds,
+                              reinterpret_cast<hipStream_t>(stream)>>>(sa, ra, int(recv_blocks));
     EP_LAUNCH_CHECK();
     return 0;
 }

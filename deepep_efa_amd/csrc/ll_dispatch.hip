@@ -162,51 +162,79 @@ constexpr int kMaxTopk = 64;
 constexpr int kFusedMaxEntries = 2048;
 constexpr int kSendMaxWaves = 16;
 
-template <int kFmt>
-__global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(
-    const uint8_t* __restrict__ x, const int64_t* __restrict__ topk_idx,
-    const int32_t* __restrict__ src_ranks, int num_tokens, int hidden, int num_topk, int num_experts,
-    int num_ranks, int rank, int max_tokens, int pieces_per_row, int split_log2, uint32_t rank_of_expert_magic,
-    int num_chunks, int64_t scratch_stride, const uint8_t* __restrict__ scratch_base,
-    uint8_t* __restrict__ recv_staging,
-    uint8_t* __restrict__ send_slots, int32_t* __restrict__ pair_slot, int32_t* __restrict__ recv_count,
-    int32_t* __restrict__ send_count) {
-    extern __shared__ int32_t lds_hist[];  // [E], counting workgroups only
-    __shared__ int32_t sel_expert[kMaxTopk];
-    __shared__ int32_t sel_count[kMaxTopk];
-    __shared__ uint64_t sel_row[kMaxTopk];
-    const int lane = lane_id(), tid = threadIdx.x;
-    const int b = blockIdx.z, t = blockIdx.y;
-    const int n = num_tokens * num_topk;
-    const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
-    const int64_t* my_topk = topk_idx + int64_t(b) * n;
+struct SendArgs {
+    const uint8_t* x;
+    const int64_t* topk_idx;
+    const int32_t* src_ranks;  // null: the rows are this rank's own
+    int num_tokens, hidden, num_topk, num_experts, num_ranks, rank, max_tokens;
+    int pieces_per_row, split_log2;
+    uint32_t rank_of_expert_magic;
+    int num_chunks;
+    int64_t scratch_stride;
+    const uint8_t* scratch_base;
+    uint8_t* recv_staging;
+    uint8_t* send_slots;
+    int32_t* pair_slot;
+    int32_t* recv_count;
+    int32_t* send_count;
+};
 
-    if (t == num_tokens) {  // the counting row of the grid (single-chunk batches): one workgroup per source
-        if (blockIdx.x != 0) return;
-        for (int j = tid; j < num_experts; j += blockDim.x) lds_hist[j] = 0;
-        __syncthreads();
-        for (int i = tid; i < n; i += blockDim.x) {
-            const int64_t v = my_topk[i];
-            if (v >= 0 && v < num_experts) atomicAdd(&lds_hist[int(v)], 1);
-        }
-        __syncthreads();
-        for (int e = tid; e < num_experts; e += blockDim.x)
-            emit_expert_count(e, lds_hist[e], num_experts, num_ranks, rank, src_rank, max_tokens, recv_count,
-                              send_count);
-        return;
+// Final destination of the rows a rank sends to its own experts, used by the
+// single-launch dispatch: they skip the staging area and land where the
+// receive side would have copied them.
+struct DirectOut {
+    uint8_t* packed_x;  // null: stage own rows like everyone else's
+    uint8_t* packed_scales;
+    int32_t* src_info;
+};
+
+struct SendLds {
+    int32_t sel_expert[kMaxTopk];
+    int32_t sel_count[kMaxTopk];
+    uint64_t sel_row[kMaxTopk];    // where selection k's payload goes (0: nowhere)
+    uint64_t sel_scale[kMaxTopk];  // where its scales go
+};
+
+// The per-source counting workgroup of a single-chunk batch.
+__device__ __forceinline__ void send_count_block(const SendArgs& a, int b, int32_t* lds_hist) {
+    const int tid = threadIdx.x;
+    const int n = a.num_tokens * a.num_topk;
+    const int src_rank = a.src_ranks != nullptr ? a.src_ranks[b] : a.rank;
+    const int64_t* my_topk = a.topk_idx + int64_t(b) * n;
+    for (int j = tid; j < a.num_experts; j += blockDim.x) lds_hist[j] = 0;
+    __syncthreads();
+    for (int i = tid; i < n; i += blockDim.x) {
+        const int64_t v = my_topk[i];
+        if (v >= 0 && v < a.num_experts) atomicAdd(&lds_hist[int(v)], 1);
     }
+    __syncthreads();
+    for (int e = tid; e < a.num_experts; e += blockDim.x)
+        emit_expert_count(e, lds_hist[e], a.num_experts, a.num_ranks, a.rank, src_rank, a.max_tokens, a.recv_count,
+                          a.send_count);
+}
 
-    const int item = int(blockIdx.x) * int(blockDim.x >> 6) + wave_in_block();
-    const int split = 1 << split_log2;
-    const bool wave_live = item < (pieces_per_row << split_log2);
+// One workgroup's share of token t of source b.
+template <int kFmt>
+__device__ __forceinline__ void send_token_block(const SendArgs& a, const DirectOut& direct, int b, int t,
+                                                 int block_in_token, SendLds& lds) {
+    const int lane = lane_id(), tid = threadIdx.x;
+    const int num_topk = a.num_topk, num_experts = a.num_experts;
+    const int n = a.num_tokens * num_topk;
+    const int src_rank = a.src_ranks != nullptr ? a.src_ranks[b] : a.rank;
+    const int64_t* my_topk = a.topk_idx + int64_t(b) * n;
+
+    const int item = block_in_token * int(blockDim.x >> 6) + wave_in_block();
+    const int split = 1 << a.split_log2;
+    const bool wave_live = item < (a.pieces_per_row << a.split_log2);
     const int part = item & (split - 1);
-    const int piece = item >> split_log2;
-    const int64_t row_id = int64_t(b) * num_tokens + t;
+    const int piece = item >> a.split_log2;
+    const int64_t row_id = int64_t(b) * a.num_tokens + t;
     const int entry0 = t * num_topk;
 
-    const int64_t data_bytes = row_data_bytes(hidden, kFmt);
+    const int64_t data_bytes = row_data_bytes(a.hidden, kFmt);
     const int64_t data_pad = align16(data_bytes);
-    const int64_t scale_pad = align16(row_scale_bytes(hidden, kFmt));
+    const int64_t scale_bytes = row_scale_bytes(a.hidden, kFmt);
+    const int64_t scale_pad = align16(scale_bytes);
     const int64_t stride = data_pad + scale_pad + kRowTailBytes;
 
     // ---- issue this wave's row loads ------------------------------------
@@ -216,63 +244,84 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(
     if constexpr (kFmt == kRowBF16) {
         const int64_t off = int64_t(piece) * 1024 + lane * 16;
         lane_live = wave_live && off < data_bytes;
-        if (lane_live) lo = *reinterpret_cast<const u32x4*>(x + row_id * data_bytes + off);
+        if (lane_live) lo = *reinterpret_cast<const u32x4*>(a.x + row_id * data_bytes + off);
     } else {
         group = piece * 8 + (lane >> 3);
-        lane_live = wave_live && group < hidden / kGroup;
+        lane_live = wave_live && group < a.hidden / kGroup;
         if (lane_live) {
-            const uint8_t* src = x + (row_id * hidden + int64_t(group) * kGroup + (lane & 7) * 16) * 2;
+            const uint8_t* src = a.x + (row_id * a.hidden + int64_t(group) * kGroup + (lane & 7) * 16) * 2;
             lo = *reinterpret_cast<const u32x4*>(src);
             hi = *reinterpret_cast<const u32x4*>(src + 16);
         }
     }
 
     // ---- per-selection bookkeeping, once per token --------------------------
-    int my_expert = -1, my_slot = -1;  // threads 0..K-1: selection k = tid
+    int my_expert = -1, my_slot = -1, dst_rank = -1, local = 0;  // threads 0..K-1: selection k = tid
+    int direct_begin = 0;
     if (tid < num_topk) {
         const int64_t v = my_topk[entry0 + tid];
-        if (v >= 0 && v < num_experts) my_expert = int(v);
+        if (v >= 0 && v < num_experts) {
+            my_expert = int(v);
+            // my_expert / E_l by multiply-high; magic 0 stands for E_l == 1
+            dst_rank = a.rank_of_expert_magic != 0 ? int(__umulhi(uint32_t(my_expert), a.rank_of_expert_magic))
+                                                   : my_expert;
+            local = my_expert - dst_rank * (num_experts / a.num_ranks);
+            if (direct.packed_x != nullptr && dst_rank == a.rank) {
+                // rows of the ranks below come first in the expert's packed range
+                for (int s = 0; s < a.rank; ++s) {
+                    const int c = a.recv_count[local * a.num_ranks + s];
+                    direct_begin += c < 0 ? 0 : (c > a.max_tokens ? a.max_tokens : c);
+                }
+            }
+        }
     }
-    if (num_chunks > 1) {  // slots were ranked by ll_route_slots_kernel
+    if (a.num_chunks > 1) {  // slots were ranked by ll_route_slots_kernel
         if (tid < num_topk && my_expert >= 0)
-            my_slot = reinterpret_cast<const int32_t*>(scratch_base + int64_t(b) * scratch_stride)[entry0 + tid];
+            my_slot = reinterpret_cast<const int32_t*>(a.scratch_base + int64_t(b) * a.scratch_stride)[entry0 + tid];
     } else {  // small batch: rank here, sweeping every earlier entry
         if (tid < num_topk) {
-            sel_expert[tid] = my_expert;
-            sel_count[tid] = 0;
+            lds.sel_expert[tid] = my_expert;
+            lds.sel_count[tid] = 0;
         }
         __syncthreads();
         for (int i = tid; i < entry0; i += blockDim.x) {
             const int64_t v = my_topk[i];
             if (v < 0 || v >= num_experts) continue;
             for (int k = 0; k < num_topk; ++k)
-                if (int(v) == sel_expert[k]) atomicAdd(&sel_count[k], 1);
+                if (int(v) == lds.sel_expert[k]) atomicAdd(&lds.sel_count[k], 1);
         }
         __syncthreads();
         if (tid < num_topk && my_expert >= 0) {
-            my_slot = sel_count[tid];
+            my_slot = lds.sel_count[tid];
             for (int k2 = 0; k2 < tid; ++k2)  // the same expert named earlier in this token
-                if (sel_expert[k2] == my_expert) my_slot += 1;
+                if (lds.sel_expert[k2] == my_expert) my_slot += 1;
         }
     }
     if (tid < num_topk) {
-        if (my_slot >= max_tokens) my_slot = -1;
+        if (my_slot >= a.max_tokens) my_slot = -1;
         uint8_t* row = nullptr;
+        uint8_t* scale_row = nullptr;
+        bool staged = false;
         if (my_slot >= 0) {
-            // my_expert / E_l by multiply-high; magic 0 stands for E_l == 1
-            const int dst_rank = rank_of_expert_magic != 0
-                                     ? int(__umulhi(uint32_t(my_expert), rank_of_expert_magic))
-                                     : my_expert;
-            const int local = my_expert - dst_rank * (num_experts / num_ranks);
-            if (dst_rank == rank)
-                row = recv_staging + ((int64_t(local) * num_ranks + src_rank) * max_tokens + my_slot) * stride;
-            else if (send_slots != nullptr)
-                row = send_slots + (int64_t(my_expert) * max_tokens + my_slot) * stride;
+            if (dst_rank == a.rank && direct.packed_x != nullptr) {
+                const int64_t out_row = int64_t(local) * a.num_ranks * a.max_tokens + direct_begin + my_slot;
+                row = direct.packed_x + out_row * data_bytes;
+                scale_row = direct.packed_scales + out_row * scale_bytes;
+                if (block_in_token == 0) direct.src_info[out_row] = t;
+            } else if (dst_rank == a.rank) {
+                row = a.recv_staging + ((int64_t(local) * a.num_ranks + src_rank) * a.max_tokens + my_slot) * stride;
+                staged = true;
+            } else if (a.send_slots != nullptr) {
+                row = a.send_slots + (int64_t(my_expert) * a.max_tokens + my_slot) * stride;
+                staged = true;
+            }
+            if (staged) scale_row = row + data_pad;
         }
-        sel_row[tid] = reinterpret_cast<uint64_t>(row);
-        if (blockIdx.x == 0) {
-            if (pair_slot != nullptr) pair_slot[entry0 + tid] = my_slot;
-            if (row != nullptr) {
+        lds.sel_row[tid] = reinterpret_cast<uint64_t>(row);
+        lds.sel_scale[tid] = reinterpret_cast<uint64_t>(scale_row);
+        if (block_in_token == 0) {
+            if (a.pair_slot != nullptr) a.pair_slot[entry0 + tid] = my_slot;
+            if (staged) {
                 u32x4 tail = {uint32_t(t), uint32_t(tid), uint32_t(src_rank), 0u};
                 *reinterpret_cast<u32x4*>(row + data_pad + scale_pad) = tail;
             }
@@ -287,88 +336,172 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(
     if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
     const int64_t lane_off = int64_t(piece) * 1024 + lane * 16;
     for (int k = part; k < num_topk; k += split) {
-        const uint64_t row_bits = sel_row[k];
-        const uint32_t lo32 = __builtin_amdgcn_readfirstlane(uint32_t(row_bits));
-        const uint32_t hi32 = __builtin_amdgcn_readfirstlane(uint32_t(row_bits >> 32));
-        uint8_t* row = reinterpret_cast<uint8_t*>((uint64_t(hi32) << 32) | lo32);
+        uint8_t* row = reinterpret_cast<uint8_t*>(wave_uniform_u64(lds.sel_row[k]));
         if (row == nullptr) continue;
         if (lane_live) *reinterpret_cast<u32x4*>(row + lane_off) = payload;
-        if constexpr (kFmt == kRowFP8 || kFmt == kRowFP8Pow2) {
-            if (lane_live && (lane & 7) == 0)
-                *reinterpret_cast<uint32_t*>(row + data_pad + int64_t(group) * 4) = scale_bits;
-        } else if constexpr (kFmt == kRowFP8UE8M0) {
-            if (lane_live && (lane & 7) == 0) row[data_pad + group] = uint8_t(scale_bits >> 23);
+        if constexpr (kFmt != kRowBF16) {
+            uint8_t* scale_row = reinterpret_cast<uint8_t*>(wave_uniform_u64(lds.sel_scale[k]));
+            if constexpr (kFmt == kRowFP8UE8M0) {
+                if (lane_live && (lane & 7) == 0) scale_row[group] = uint8_t(scale_bits >> 23);
+            } else {
+                if (lane_live && (lane & 7) == 0)
+                    *reinterpret_cast<uint32_t*>(scale_row + int64_t(group) * 4) = scale_bits;
+            }
         }
     }
+}
+
+template <int kFmt>
+__global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs a) {
+    extern __shared__ int32_t lds_hist[];  // [E], counting workgroups only
+    __shared__ SendLds lds;
+    if (int(blockIdx.y) == a.num_tokens) {  // the counting row of the grid (single-chunk batches)
+        if (blockIdx.x == 0) send_count_block(a, blockIdx.z, lds_hist);
+        return;
+    }
+    const DirectOut none = {nullptr, nullptr, nullptr};
+    send_token_block<kFmt>(a, none, blockIdx.z, blockIdx.y, blockIdx.x, lds);
 }
 
 // ---------------------------------------------------------------------
 // Receive side.  Every workgroup rebuilds the segment prefix from the E
 // counts (a few hundred ints) in LDS, then its waves walk the flat row index
-// space: row -> (segment, j) by binary search, one wave per row.
+// space: row -> (segment, j) by binary search, one wave per row part.
 // Slot order is fixed by the staging order, not by atomics
 // (reference: csrc/kernels/efa_kernels.cu:1017-1052 for the ranges,
 // :1059-1213 for the deterministic scatter).
+//
+// own_topk != null (single-launch dispatch): the rows this rank sends to its own
+// experts are not in the staging area — the send workgroups of the same launch
+// put them straight into the packed tensors — so the own segments' counts are
+// recounted here from the rank's own indices, and their rows are skipped.
 // ---------------------------------------------------------------------
-__global__ __launch_bounds__(256) void ll_recv_kernel(
-    const uint8_t* __restrict__ recv_staging, const int32_t* __restrict__ recv_count, int hidden,
-    int num_local_experts, int num_ranks, int max_tokens, int fmt, int parts, uint8_t* __restrict__ packed_x,
-    uint8_t* __restrict__ packed_scales, int32_t* __restrict__ src_info, int64_t* __restrict__ layout_range,
-    int32_t* __restrict__ packed_count, int32_t* __restrict__ stats) {
-    extern __shared__ int32_t flat[];  // [num_segments + 1]
-    __shared__ int32_t wave_totals[4];
-    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
-    const int num_segments = num_local_experts * num_ranks;
+struct RecvArgs {
+    const uint8_t* recv_staging;
+    const int32_t* recv_count;
+    int hidden, num_local_experts, num_ranks, max_tokens, fmt, parts;
+    uint8_t* packed_x;
+    uint8_t* packed_scales;
+    int32_t* src_info;
+    int64_t* layout_range;
+    int32_t* packed_count;
+    int32_t* stats;
+};
 
-    for (int s = tid; s < num_segments; s += 256) {
-        int c = recv_count[s];
-        c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
-        flat[s] = c;
+// flat: [num_segments + 1] ints (+ num_local_experts when own_topk != null); wave_totals: 16 ints.
+__device__ __forceinline__ void recv_rows(const RecvArgs& a, int block, int num_blocks, const int64_t* own_topk,
+                                          int own_entries, int own_rank, int32_t* flat, int32_t* wave_totals) {
+    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
+    const int threads = blockDim.x, waves = threads >> 6;
+    const int num_segments = a.num_local_experts * a.num_ranks;
+    const int num_ranks = a.num_ranks, max_tokens = a.max_tokens;
+
+    if (own_topk != nullptr) {
+        int32_t* own_cnt = flat + num_segments + 1;
+        for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
+        __syncthreads();
+        const int64_t first = int64_t(own_rank) * a.num_local_experts;
+        for (int i = tid; i < own_entries; i += threads) {
+            const int64_t v = own_topk[i] - first;
+            if (v >= 0 && v < a.num_local_experts) atomicAdd(&own_cnt[int(v)], 1);
+        }
+        for (int s = tid; s < num_segments; s += threads) {
+            if (s % num_ranks == own_rank) continue;
+            const int c = a.recv_count[s];
+            flat[s] = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+        }
+        __syncthreads();
+        for (int le = tid; le < a.num_local_experts; le += threads) {
+            const int c = own_cnt[le];
+            flat[le * num_ranks + own_rank] = c > max_tokens ? max_tokens : c;
+        }
+    } else {
+        for (int s = tid; s < num_segments; s += threads) {
+            const int c = a.recv_count[s];
+            flat[s] = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+        }
     }
     __syncthreads();
-    block_exclusive_scan_256(flat, num_segments, wave_totals);
+    block_exclusive_scan(flat, num_segments, wave_totals);
     const int total_rows = flat[num_segments];
 
-    if (blockIdx.x == 0) {
-        for (int s = tid; s < num_segments; s += 256) {
+    if (block == 0) {
+        for (int s = tid; s < num_segments; s += threads) {
             const int le = s / num_ranks;
             const int64_t cnt = flat[s + 1] - flat[s];
             const int64_t begin = flat[s] - flat[le * num_ranks];
-            layout_range[s] = cnt > 0 ? ((begin << 32) | cnt) : 0;
+            a.layout_range[s] = cnt > 0 ? ((begin << 32) | cnt) : 0;
         }
-        for (int le = tid; le < num_local_experts; le += 256) {
+        for (int le = tid; le < a.num_local_experts; le += threads) {
             const int c = flat[(le + 1) * num_ranks] - flat[le * num_ranks];
-            packed_count[le] = c;
-            if (stats != nullptr) stats[le] += c;
+            a.packed_count[le] = c;
+            if (a.stats != nullptr) a.stats[le] += c;
         }
     }
 
-    const int64_t data_bytes = row_data_bytes(hidden, fmt);
+    const int64_t data_bytes = row_data_bytes(a.hidden, a.fmt);
     const int64_t data_pad = align16(data_bytes);
-    const int64_t scale_bytes = row_scale_bytes(hidden, fmt);
+    const int64_t scale_bytes = row_scale_bytes(a.hidden, a.fmt);
     const int64_t stride = data_pad + align16(scale_bytes) + kRowTailBytes;
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
-    const int64_t waves_total = int64_t(gridDim.x) * 4;
+    const int64_t waves_total = int64_t(num_blocks) * waves;
     const int num_vec = int(data_bytes / 16);
-    for (int64_t item = blockIdx.x * 4 + w; item < int64_t(total_rows) * parts; item += waves_total) {
+    const int parts = a.parts;
+    for (int64_t item = int64_t(block) * waves + w; item < int64_t(total_rows) * parts; item += waves_total) {
         const int row = int(item / parts), part = int(item - int64_t(row) * parts);
         const int seg = __builtin_amdgcn_readfirstlane(find_segment(flat, num_segments, row));
-        const int j = row - __builtin_amdgcn_readfirstlane(flat[seg]);
         const int le = seg / num_ranks;
+        if (own_topk != nullptr && seg - le * num_ranks == own_rank) continue;
+        const int j = row - __builtin_amdgcn_readfirstlane(flat[seg]);
         const int64_t slot = int64_t(row) - __builtin_amdgcn_readfirstlane(flat[le * num_ranks]);
-        const uint8_t* src = recv_staging + (int64_t(seg) * max_tokens + j) * stride;
+        const uint8_t* src = a.recv_staging + (int64_t(seg) * max_tokens + j) * stride;
         const int64_t out_row = int64_t(le) * slots_per_expert + slot;
         int v_begin, v_end;
         row_part_range(num_vec, parts, part, v_begin, v_end);
-        wave_copy_vec16(src, packed_x + out_row * data_bytes, v_begin, v_end, lane);
+        wave_copy_vec16(src, a.packed_x + out_row * data_bytes, v_begin, v_end, lane);
         if (part != parts - 1) continue;  // the last part is the shortest: it also carries scales and source index
-        if (packed_scales != nullptr && scale_bytes > 0) {
+        if (a.packed_scales != nullptr && scale_bytes > 0) {
             const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src + data_pad);
-            uint32_t* d32 = reinterpret_cast<uint32_t*>(packed_scales + out_row * scale_bytes);
+            uint32_t* d32 = reinterpret_cast<uint32_t*>(a.packed_scales + out_row * scale_bytes);
             for (int v = lane; v < int(scale_bytes / 4); v += kWave) d32[v] = s32[v];
         }
         if (lane == 0)
-            src_info[out_row] = *reinterpret_cast<const int32_t*>(src + data_pad + align16(scale_bytes));
+            a.src_info[out_row] = *reinterpret_cast<const int32_t*>(src + data_pad + align16(scale_bytes));
+    }
+}
+
+__global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a) {
+    extern __shared__ int32_t flat[];  // [num_segments + 1]
+    __shared__ int32_t wave_totals[kMaxBlockWaves];
+    recv_rows(a, blockIdx.x, gridDim.x, nullptr, 0, 0, flat, wave_totals);
+}
+
+// ---------------------------------------------------------------------
+// Single-launch dispatch for small batches (T*K <= 2048, E*M <= 2^18): the send
+// workgroups, the counting workgroup and the receive workgroups of the two
+// kernels above in one grid.  No workgroup waits on another: the receive
+// workgroups copy only the peers' rows (already in the staging area when the
+// launch starts) and recount the own segments from topk_idx; the send
+// workgroups place the rank's rows for its own experts at their final packed
+// position, which they find from the peers' counts.
+// (The reference's dispatch is one kernel with a send and a receive phase as
+// well: csrc/kernels/coop_dispatch_send.cuh:304, coop_dispatch_recv.cuh:42.)
+// ---------------------------------------------------------------------
+template <int kFmt>
+__global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_dispatch_fused_kernel(SendArgs sa, RecvArgs ra, int blocks_per_token,
+                                                                                 int num_send_blocks) {
+    extern __shared__ int32_t dyn_lds[];  // counting: [E]; receive: [segments + 1 + E_l]
+    __shared__ SendLds lds;
+    __shared__ int32_t wave_totals[kMaxBlockWaves];
+    const int block = blockIdx.x;
+    if (block < num_send_blocks) {
+        const DirectOut direct = {ra.packed_x, ra.packed_scales, ra.src_info};
+        send_token_block<kFmt>(sa, direct, 0, block / blocks_per_token, block % blocks_per_token, lds);
+    } else if (block == num_send_blocks) {
+        send_count_block(sa, 0, dyn_lds);
+    } else {
+        recv_rows(ra, block - num_send_blocks - 1, int(gridDim.x) - num_send_blocks - 1, sa.topk_idx,
+                  sa.num_tokens * sa.num_topk, sa.rank, dyn_lds, wave_totals);
     }
 }
 
@@ -401,7 +534,8 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
                             int num_tokens, int hidden, int num_topk, int num_experts, int num_ranks, int rank,
                             int max_tokens, int row_format, void* recv_staging, int32_t* recv_count,
                             void* send_slots, int32_t* send_count, int32_t* pair_slot, void* workspace,
-                            size_t workspace_bytes, hipStream_t stream) {
+                            size_t workspace_bytes, hipStream_t stream, const RecvArgs* fused_recv = nullptr,
+                            int64_t fused_recv_wave_items = 0) {
     RouteScratch rs = route_scratch(num_tokens, num_topk, num_experts);
     EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(rs.bytes) * size_t(num_src));
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
@@ -429,21 +563,54 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     const int waves = items < kSendMaxWaves ? items : kSendMaxWaves;
     const int blocks_per_token = (items + waves - 1) / waves;
     EP_HOST_ASSERT(num_tokens < 65535 && num_src <= 65535);
-    const dim3 grid(blocks_per_token, num_tokens + (single_chunk ? 1 : 0), num_src);
-    if (grid.y == 0) return 0;
-    const size_t lds = single_chunk ? size_t(num_experts) * sizeof(int32_t) : 0;
     // floor(e / E_l) == umulhi(e, ceil(2^32 / E_l)) for every e below 2^16.
     const uint32_t experts_per_rank = uint32_t(num_experts / num_ranks);
     const uint32_t magic =
         experts_per_rank == 1 ? 0u : uint32_t(((uint64_t(1) << 32) + experts_per_rank - 1) / experts_per_rank);
     EP_HOST_ASSERT(num_experts < 65536);
-    const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
-    uint8_t* stg = reinterpret_cast<uint8_t*>(recv_staging);
-    uint8_t* snd = reinterpret_cast<uint8_t*>(send_slots);
-#define DEEPEP_LAUNCH_SEND(FMT)                                                                                 \
-    ll_send_kernel<FMT><<<grid, waves * kWave, lds, stream>>>(                                                  \
-        xb, topk_idx, src_ranks, num_tokens, hidden, num_topk, num_experts, num_ranks, rank, max_tokens, pieces, \
-        split_log2, magic, rs.num_chunks, rs.bytes, ws, stg, snd, pair_slot, recv_count, send_count)
+    SendArgs sa;
+    sa.x = reinterpret_cast<const uint8_t*>(x);
+    sa.topk_idx = topk_idx;
+    sa.src_ranks = src_ranks;
+    sa.num_tokens = num_tokens, sa.hidden = hidden, sa.num_topk = num_topk, sa.num_experts = num_experts;
+    sa.num_ranks = num_ranks, sa.rank = rank, sa.max_tokens = max_tokens;
+    sa.pieces_per_row = pieces, sa.split_log2 = split_log2;
+    sa.rank_of_expert_magic = magic;
+    sa.num_chunks = rs.num_chunks, sa.scratch_stride = rs.bytes, sa.scratch_base = ws;
+    sa.recv_staging = reinterpret_cast<uint8_t*>(recv_staging);
+    sa.send_slots = reinterpret_cast<uint8_t*>(send_slots);
+    sa.pair_slot = pair_slot, sa.recv_count = recv_count, sa.send_count = send_count;
+
+    if (fused_recv != nullptr) {  // single launch: send workgroups, the counting workgroup, receive workgroups
+        EP_HOST_ASSERT(single_chunk && num_src == 1 && src_ranks == nullptr);
+        const int num_send_blocks = blocks_per_token * num_tokens;
+        int64_t fused_recv_blocks = (fused_recv_wave_items + waves - 1) / waves;
+        fused_recv_blocks = fused_recv_blocks < 1 ? 1 : (fused_recv_blocks > 1024 ? 1024 : fused_recv_blocks);
+        const int64_t total = int64_t(num_send_blocks) + 1 + fused_recv_blocks;
+        EP_HOST_ASSERT(total < (int64_t(1) << 31));
+        const int num_segments = fused_recv->num_local_experts * fused_recv->num_ranks;
+        const size_t need_recv = size_t(num_segments + 1 + fused_recv->num_local_experts) * sizeof(int32_t);
+        const size_t need_count = size_t(num_experts) * sizeof(int32_t);
+        const size_t lds = need_recv > need_count ? need_recv : need_count;
+        const RecvArgs ra = *fused_recv;
+#define DEEPEP_LAUNCH_FUSED(FMT)                                                                        \
+    ll_dispatch_fused_kernel<FMT><<<dim3(unsigned(total)), waves * kWave, lds, stream>>>(sa, ra, blocks_per_token, \
+                                                                                         num_send_blocks)
+        switch (row_format) {
+            case kRowBF16: DEEPEP_LAUNCH_FUSED(kRowBF16); break;
+            case kRowFP8: DEEPEP_LAUNCH_FUSED(kRowFP8); break;
+            case kRowFP8Pow2: DEEPEP_LAUNCH_FUSED(kRowFP8Pow2); break;
+            default: DEEPEP_LAUNCH_FUSED(kRowFP8UE8M0); break;
+        }
+#undef DEEPEP_LAUNCH_FUSED
+        EP_LAUNCH_CHECK();
+        return 0;
+    }
+
+    const dim3 grid(blocks_per_token, num_tokens + (single_chunk ? 1 : 0), num_src);
+    if (grid.y == 0) return 0;
+    const size_t lds = single_chunk ? size_t(num_experts) * sizeof(int32_t) : 0;
+#define DEEPEP_LAUNCH_SEND(FMT) ll_send_kernel<FMT><<<grid, waves * kWave, lds, stream>>>(sa)
     switch (row_format) {
         case kRowBF16: DEEPEP_LAUNCH_SEND(kRowBF16); break;
         case kRowFP8: DEEPEP_LAUNCH_SEND(kRowFP8); break;
@@ -514,16 +681,13 @@ int deepep_loopback_dispatch_from_peers(const void* x, const int64_t* topk_idx, 
                             nullptr, nullptr, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
 }
 
-int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
-                            int num_ranks, int num_max_dispatch_tokens_per_rank, int row_format,
-                            void* packed_recv_x, void* packed_recv_scales, int32_t* packed_recv_src_info,
-                            int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
-                            int32_t* cumulative_local_expert_recv_stats, int64_t expected_rows, void* workspace,
-                            size_t workspace_bytes, void* stream) {
-    clear_error();
+static int check_recv_args(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
+                           int num_ranks, int max_tokens, int row_format, void* packed_recv_x,
+                           void* packed_recv_scales, int32_t* packed_recv_src_info, int64_t* packed_recv_layout_range,
+                           int32_t* packed_recv_count) {
     EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
     EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
-    EP_HOST_ASSERT(num_max_dispatch_tokens_per_rank > 0);
+    EP_HOST_ASSERT(max_tokens > 0);
     EP_HOST_ASSERT(row_format >= kRowBF16 && row_format <= kRowFP8UE8M0);
     EP_HOST_ASSERT(row_format != kRowFP8UE8M0 || (hidden / 128) % 4 == 0);
     EP_HOST_ASSERT(num_experts <= 1024);
@@ -534,9 +698,40 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_staging) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_x) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_scales) & 3) == 0);
+    EP_HOST_ASSERT(int64_t(num_experts) * max_tokens < (int64_t(1) << 31));
+    return 0;
+}
+
+static RecvArgs make_recv_args(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
+                               int num_ranks, int max_tokens, int row_format, void* packed_recv_x,
+                               void* packed_recv_scales, int32_t* packed_recv_src_info,
+                               int64_t* packed_recv_layout_range, int32_t* packed_recv_count, int32_t* stats) {
+    RecvArgs ra;
+    ra.recv_staging = reinterpret_cast<const uint8_t*>(recv_staging);
+    ra.recv_count = recv_count;
+    ra.hidden = hidden, ra.num_local_experts = num_experts / num_ranks, ra.num_ranks = num_ranks;
+    ra.max_tokens = max_tokens, ra.fmt = row_format;
+    ra.parts = choose_row_parts(int64_t(num_experts) * max_tokens, row_data_bytes(hidden, row_format));
+    ra.packed_x = reinterpret_cast<uint8_t*>(packed_recv_x);
+    ra.packed_scales = reinterpret_cast<uint8_t*>(packed_recv_scales);
+    ra.src_info = packed_recv_src_info, ra.layout_range = packed_recv_layout_range;
+    ra.packed_count = packed_recv_count, ra.stats = stats;
+    return ra;
+}
+
+int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
+                            int num_ranks, int num_max_dispatch_tokens_per_rank, int row_format,
+                            void* packed_recv_x, void* packed_recv_scales, int32_t* packed_recv_src_info,
+                            int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
+                            int32_t* cumulative_local_expert_recv_stats, int64_t expected_rows, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+    clear_error();
+    if (int rc = check_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
+                                 num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
+                                 packed_recv_src_info, packed_recv_layout_range, packed_recv_count))
+        return rc;
     const int num_local_experts = num_experts / num_ranks;
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
-    EP_HOST_ASSERT(max_rows < (int64_t(1) << 31));
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
     if (max_rows > kLargeBatchRows && workspace != nullptr) {
         EP_HOST_ASSERT(workspace_bytes >= size_t(segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank)));
@@ -565,18 +760,63 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
         EP_LAUNCH_CHECK();
         return 0;
     }
-    const int parts = choose_row_parts(max_rows, row_data_bytes(hidden, row_format));
-    int64_t blocks = (max_rows * parts + 3) / 4;
+    const RecvArgs ra = make_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
+                                       num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
+                                       packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
+                                       cumulative_local_expert_recv_stats);
+    int64_t blocks = (max_rows * ra.parts + 3) / 4;
     const int64_t cap = max_rows > kLargeBatchRows ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(num_experts + 1) * sizeof(int32_t);
-    ll_recv_kernel<<<dim3(unsigned(blocks)), 256, lds, hs>>>(
-        reinterpret_cast<const uint8_t*>(recv_staging), recv_count, hidden, num_local_experts, num_ranks,
-        num_max_dispatch_tokens_per_rank, row_format, parts, reinterpret_cast<uint8_t*>(packed_recv_x),
-        reinterpret_cast<uint8_t*>(packed_recv_scales), packed_recv_src_info, packed_recv_layout_range,
-        packed_recv_count, cumulative_local_expert_recv_stats);
+    ll_recv_kernel<<<dim3(unsigned(blocks)), 256, lds, hs>>>(ra);
     EP_LAUNCH_CHECK();
     return 0;
+}
+
+int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, int hidden, int num_topk,
+                       int num_experts, int num_ranks, int rank, int num_max_dispatch_tokens_per_rank, int row_format,
+                       void* recv_staging, int32_t* recv_count, void* send_slots, int32_t* send_count,
+                       int32_t* pair_slot, void* packed_recv_x, void* packed_recv_scales,
+                       int32_t* packed_recv_src_info, int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
+                       int32_t* cumulative_local_expert_recv_stats, int64_t expected_rows, void* workspace,
+                       size_t workspace_bytes, void* segment_workspace, size_t segment_workspace_bytes,
+                       void* stream) {
+    clear_error();
+    const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
+    const bool fused = int64_t(num_tokens) * num_topk <= kFusedMaxEntries && max_rows <= kLargeBatchRows;
+    if (!fused) {  // the two phases back to back
+        if (int rc = deepep_ll_dispatch_send(x, topk_idx, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                                             num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count,
+                                             send_slots, send_count, pair_slot, workspace, workspace_bytes, stream))
+            return rc;
+        return deepep_ll_dispatch_recv(recv_staging, recv_count, hidden, num_experts, num_ranks,
+                                       num_max_dispatch_tokens_per_rank, row_format, packed_recv_x,
+                                       packed_recv_scales, packed_recv_src_info, packed_recv_layout_range,
+                                       packed_recv_count, cumulative_local_expert_recv_stats, expected_rows,
+                                       segment_workspace, segment_workspace_bytes, stream);
+    }
+    if (int rc = check_ll_shape(num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                                num_max_dispatch_tokens_per_rank, row_format))
+        return rc;
+    EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
+    EP_HOST_ASSERT(send_count != nullptr && pair_slot != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(send_slots) & 15) == 0);
+    if (int rc = check_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
+                                 num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
+                                 packed_recv_src_info, packed_recv_layout_range, packed_recv_count))
+        return rc;
+    const RecvArgs ra = make_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
+                                       num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
+                                       packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
+                                       cumulative_local_expert_recv_stats);
+    int64_t rows = expected_rows > 0 ? expected_rows : int64_t(num_max_dispatch_tokens_per_rank) * num_topk;
+    rows += rows / 8 + 16;
+    if (rows > max_rows) rows = max_rows;
+    return launch_send_side(x, topk_idx, nullptr, 1, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                            num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count, send_slots,
+                            send_count, pair_slot, workspace, workspace_bytes,
+                            reinterpret_cast<hipStream_t>(stream), &ra, rows * ra.parts);
 }
 
 }  // extern "C"

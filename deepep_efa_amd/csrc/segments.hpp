@@ -1,5 +1,5 @@
 // Helpers for kernels that walk a list of variable-length row segments with
-// one wavefront per row: a 256-thread exclusive scan in LDS, the row ->
+// one wavefront per row: a workgroup-wide exclusive scan in LDS, the row ->
 // segment search, and the 16-byte-per-lane row copy.
 #pragma once
 
@@ -10,12 +10,16 @@
 namespace deepep {
 
 // ---------------------------------------------------------------------
-// Exclusive prefix of n ints held in LDS, by a 256-thread workgroup.
-// data[n] receives the total.
+// Exclusive prefix of n ints held in LDS, by the whole workgroup (a multiple
+// of 64 threads, at most 1024).  data[n] receives the total; wave_totals has
+// room for 16 ints.
 // ---------------------------------------------------------------------
-__device__ __forceinline__ void block_exclusive_scan_256(int32_t* data, int n, int32_t* wave_totals) {
+constexpr int kMaxBlockWaves = 16;
+
+__device__ __forceinline__ void block_exclusive_scan(int32_t* data, int n, int32_t* wave_totals) {
     const int tid = threadIdx.x, lane = lane_id(), w = tid >> 6;
-    const int per = (n + 255) / 256;
+    const int threads = blockDim.x, waves = threads >> 6;
+    const int per = (n + threads - 1) / threads;
     const int lo = tid * per;
     int sum = 0;
     for (int j = 0; j < per; ++j)
@@ -23,10 +27,12 @@ __device__ __forceinline__ void block_exclusive_scan_256(int32_t* data, int n, i
     const int incl = wave_inclusive_sum(sum);
     if (lane == kWave - 1) wave_totals[w] = incl;
     __syncthreads();
-    int offset = incl - sum;
-    for (int w2 = 0; w2 < w; ++w2) offset += wave_totals[w2];
-    int total = 0;
-    for (int w2 = 0; w2 < 4; ++w2) total += wave_totals[w2];
+    int offset = incl - sum, total = 0;
+    for (int w2 = 0; w2 < waves; ++w2) {
+        const int t = wave_totals[w2];
+        if (w2 < w) offset += t;
+        total += t;
+    }
     int run = offset;
     for (int j = 0; j < per; ++j)
         if (lo + j < n) {

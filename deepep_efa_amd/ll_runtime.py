@@ -112,6 +112,21 @@ class LowLatencyState:
             _capi.ptr(self.segment_workspace),
             0 if self.segment_workspace is None else self.segment_workspace.numel(), current_stream_ptr()))
 
+    def dispatch(self, x: torch.Tensor, topk_idx: torch.Tensor, stats: torch.Tensor = None) -> None:
+        """Send + receive in one call; the peers' rows must already be staged."""
+        s = self.shape
+        t = x.shape[0]
+        sw = self.segment_workspace
+        _capi.check(self.lib.deepep_ll_dispatch(
+            _capi.ptr(x), _capi.ptr(topk_idx), t, s.hidden, s.num_topk, s.num_experts, s.num_ranks, s.rank,
+            s.max_tokens, s.fmt, _capi.ptr(self.recv_staging), _capi.ptr(self.recv_count),
+            _capi.ptr(self.send_slots), _capi.ptr(self.send_count), _capi.ptr(self.pair_slot),
+            _capi.ptr(self.packed_recv_x), _capi.ptr(self.packed_recv_scales),
+            _capi.ptr(self.packed_recv_src_info), _capi.ptr(self.packed_recv_layout_range),
+            _capi.ptr(self.packed_recv_count), _capi.ptr(stats), self.expected_rows,
+            _capi.ptr(self.workspace), self.workspace.numel(), _capi.ptr(sw), 0 if sw is None else sw.numel(),
+            current_stream_ptr()))
+
     # -- combine ----------------------------------------------------------
     def combine_send(self, x: torch.Tensor, layout_range: torch.Tensor = None) -> None:
         s = self.shape
@@ -128,3 +143,16 @@ class LowLatencyState:
         _capi.check(self.lib.deepep_ll_combine_recv(
             _capi.ptr(self.combine_staging), _capi.ptr(topk_idx), _capi.ptr(topk_weights), _capi.ptr(self.pair_slot),
             t, s.hidden, s.num_topk, s.num_experts, s.max_tokens, _capi.ptr(out), current_stream_ptr()))
+
+    def combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor,
+                layout_range: torch.Tensor = None) -> None:
+        """Row return + weighted reduce in one call; the remote experts' answers must already be staged."""
+        s = self.shape
+        t = topk_idx.shape[0]
+        lr = self.packed_recv_layout_range if layout_range is None else layout_range
+        sw = self.segment_workspace
+        _capi.check(self.lib.deepep_ll_combine(
+            _capi.ptr(x), _capi.ptr(lr), _capi.ptr(topk_idx), _capi.ptr(topk_weights), _capi.ptr(self.pair_slot),
+            t, s.hidden, s.num_topk, s.num_experts, s.num_ranks, s.rank, s.max_tokens,
+            _capi.ptr(self.combine_staging), _capi.ptr(self.combine_send_slots), _capi.ptr(out),
+            self.expected_rows, _capi.ptr(sw), 0 if sw is None else sw.numel(), current_stream_ptr()))

@@ -248,6 +248,54 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
                            int num_max_dispatch_tokens_per_rank, void* out, void* stream);
 
 /* ------------------------------------------------------------------ */
+/* Whole dispatch / whole combine in one call                          */
+/* ------------------------------------------------------------------ */
+
+/* deepep_ll_dispatch_send followed by deepep_ll_dispatch_recv, for a caller
+ * whose peers' rows and counts are already in recv_staging / recv_count when
+ * the call is made (the reference's dispatch is one call too:
+ * Buffer::low_latency_dispatch, csrc/deep_ep.cpp:1622-1799; its kernel has a
+ * send and a receive phase, csrc/kernels/coop_dispatch_send.cuh:304,
+ * coop_dispatch_recv.cuh:42).  Arguments are those of the two calls; outputs
+ * are identical, with one difference: for small batches
+ * (num_tokens * num_topk <= 2048 and num_experts * M <= 2^18) both phases run
+ * as one kernel launch, and then this rank's rows for its own experts go
+ * straight to their packed position — the own segment of recv_staging is not
+ * written (recv_count, send_count, send_slots, pair_slot are written as by
+ * deepep_ll_dispatch_send).  Larger batches launch the phases back to back.
+ *   workspace          as for deepep_ll_dispatch_send
+ *   segment_workspace  as the workspace of deepep_ll_dispatch_recv */
+int deepep_ll_dispatch(const void* x, const int64_t* topk_idx,
+                       int num_tokens, int hidden, int num_topk, int num_experts,
+                       int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                       int row_format,
+                       void* recv_staging, int32_t* recv_count,
+                       void* send_slots, int32_t* send_count, int32_t* pair_slot,
+                       void* packed_recv_x, void* packed_recv_scales,
+                       int32_t* packed_recv_src_info, int64_t* packed_recv_layout_range,
+                       int32_t* packed_recv_count, int32_t* cumulative_local_expert_recv_stats,
+                       int64_t expected_rows, void* workspace, size_t workspace_bytes,
+                       void* segment_workspace, size_t segment_workspace_bytes, void* stream);
+
+/* deepep_ll_combine_send followed by deepep_ll_combine_recv, for a caller
+ * whose remote experts' answers are already in combine_staging when the call
+ * is made (the reference: Buffer::low_latency_combine,
+ * csrc/deep_ep.cpp:1801-1939; kernel phases csrc/kernels/coop_combine_send.cuh:37,
+ * coop_combine_recv.cuh:72).  `out` is identical to the two calls'.  For
+ * num_experts * M <= 2^18 both phases run as one kernel launch, and then the
+ * answers of this rank's own experts are read from x directly — the own
+ * experts' part of combine_staging is neither written nor read.  Larger
+ * batches launch the phases back to back. */
+int deepep_ll_combine(const void* x, const int64_t* layout_range,
+                      const int64_t* topk_idx, const float* topk_weights,
+                      const int32_t* pair_slot,
+                      int num_tokens, int hidden, int num_topk, int num_experts,
+                      int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                      void* combine_staging, void* combine_send_slots, void* out,
+                      int64_t expected_rows, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
+/* ------------------------------------------------------------------ */
 /* Single-GPU loopback: peers synthesised in HBM                      */
 /* These stand where the reference has its transport                  */
 /* (csrc/transport/, dist.all_to_all_single at deep_ep/buffer.py:2268,2297,2735). */

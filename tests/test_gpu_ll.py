@@ -52,7 +52,45 @@ def make_world(r, t, h, k, e, seed, drop=10, recipe="randn"):
     return x_all, topk, w
 
 
-def dispatch_on_gpu(rt, x_all, topk_all, rank, e, m, fmt, stats=None):
+ONE_CALL = pytest.mark.parametrize("one_call", [False, True], ids=["two_calls", "one_call"])
+
+
+def poison_outputs(st):
+    """Fresh tensors may reuse memory that an earlier test left holding the right answer."""
+    st.packed_recv_x.view(torch.uint8).fill_(0xEE)
+    if st.packed_recv_scales is not None:
+        st.packed_recv_scales.view(torch.uint8).fill_(0xEE)
+    st.packed_recv_src_info.fill_(-7)
+    st.packed_recv_count.fill_(-7)
+    st.packed_recv_layout_range.fill_(-7)
+    st.pair_slot.fill_(-7)
+
+
+def run_dispatch(st, world, x, topk, stats=None, one_call=False):
+    poison_outputs(st)
+    if one_call:
+        world.dispatch_from_peers(st)
+        st.dispatch(x, topk, stats)
+    else:
+        st.dispatch_send(x, topk)
+        world.dispatch_from_peers(st)
+        st.dispatch_recv(stats)
+    torch.cuda.synchronize()
+
+
+def run_combine(st, world, y, topk, w, out, mode, seed=0, one_call=False):
+    out.view(torch.int16).fill_(0x7FC0)  # NaN
+    if one_call:
+        world.combine_from_peers(st, mode=mode, seed=seed)
+        st.combine(y, topk, w, out)
+    else:
+        world.combine_from_peers(st, mode=mode, seed=seed)
+        st.combine_send(y)
+        st.combine_recv(topk, w, out)
+    torch.cuda.synchronize()
+
+
+def dispatch_on_gpu(rt, x_all, topk_all, rank, e, m, fmt, stats=None, one_call=False):
     r, t, h = x_all.shape
     k = topk_all.shape[2]
     shape = rt.ll.LLShape(num_ranks=r, rank=rank, num_experts=e, max_tokens=m, hidden=h, num_topk=k, fmt=fmt)
@@ -60,10 +98,7 @@ def dispatch_on_gpu(rt, x_all, topk_all, rank, e, m, fmt, stats=None):
     world = rt.lb.LoopbackWorld(r, rank, seed=0)
     world.set_inputs(x_all.cuda(), topk_all.cuda())
     x, topk = world.own_inputs()
-    st.dispatch_send(x, topk)
-    world.dispatch_from_peers(st)
-    st.dispatch_recv(stats)
-    torch.cuda.synchronize()
+    run_dispatch(st, world, x, topk, stats, one_call)
     return st, world
 
 
@@ -91,11 +126,15 @@ def check_dispatch(st, want, fmt):
     (4, 3, 300, 512, 11, 32),  # both
     (8, 5, 4200, 512, 4, 64),  # E*M > 2^18: receive runs as index kernel + flat row copy
 ])
-def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e):
+@ONE_CALL
+def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
     x_all, topk_all, _ = make_world(r, t, h, k, e, seed=r * 100 + t, drop=min(5, t))
-    st, _ = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt)
+    st, _ = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt, one_call=one_call)
     want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
     check_dispatch(st, want, fmt)
+    send_count, pair_slot = O.route(topk_all[rank], e, t)
+    assert torch.equal(st.send_count.cpu(), send_count)
+    assert torch.equal(st.pair_slot[:t].cpu(), pair_slot)
 
 
 def test_dispatch_send_staging_and_send_slots(rt):
@@ -131,14 +170,15 @@ def test_dispatch_send_staging_and_send_slots(rt):
     assert (rc[:, [s for s in range(r) if s != rank]] == 0).all()
 
 
+@ONE_CALL
 @pytest.mark.parametrize("use_fp8", [True, False])
-def test_reference_recipe_roundtrip(rt, use_fp8):
+def test_reference_recipe_roundtrip(rt, use_fp8, one_call):
     """tests/test_low_latency.py:59-60,113-147,181-184 on one rank of an 8-rank world."""
     r, rank, t, h, k, e = 8, 3, 64, 2048, 6, 64
     fmt = O.ROW_FP8 if use_fp8 else O.ROW_BF16
     x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=77, drop=10, recipe="rank_const")
     stats = torch.zeros(e // r, dtype=torch.int32, device="cuda")
-    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt, stats)
+    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt, stats, one_call=one_call)
     epr = e // r
     count = st.packed_recv_count.cpu()
     lr_all = st.packed_recv_layout_range.cpu()
@@ -174,12 +214,9 @@ def test_reference_recipe_roundtrip(rt, use_fp8):
         y = y.view(el, n_slots, h).cuda()
     else:
         y = st.packed_recv_x.clone()
-    world.combine_from_peers(st, mode=0)
-    st.combine_send(y)
     out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
     topk, w = topk_all[rank].cuda(), w_all[rank].cuda()
-    st.combine_recv(topk, w, out)
-    torch.cuda.synchronize()
+    run_combine(st, world, y, topk, w, out, mode=0, one_call=one_call)
     x = x_all[rank]
     wsum = w_all[rank].masked_fill(topk_all[rank] == -1, 0).sum(1).view(-1, 1)
     diff = O.calc_diff(x.float() * wsum, out.cpu())
@@ -189,21 +226,20 @@ def test_reference_recipe_roundtrip(rt, use_fp8):
 
 @pytest.mark.parametrize("r,rank,t,h,k,e", [(32, 5, 128, 7168, 8, 256), (4, 0, 16, 512, 3, 8),
                                             (8, 3, 4200, 512, 4, 64)])  # the last: large-batch combine-send path
-def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e):
+@ONE_CALL
+def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e, one_call):
     """Seeded expert outputs along the dispatch routing; combine vs the float32 chain and the float64 sum."""
     x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=31 + r, drop=10)
-    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, O.ROW_FP8)
+    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, O.ROW_FP8, one_call=one_call)
     epr, n_slots, lib, capi = e // r, r * t, rt.capi.load(), rt.capi
     seed_local, seed_remote = 1234, 4321
     # local experts' outputs: row key = local_expert * N + slot
     y = torch.zeros((epr, n_slots, h), dtype=torch.bfloat16, device="cuda")
     capi.check(lib.deepep_synth_bf16_rows(capi.ptr(y), epr * n_slots, h, h * 2, None, 0, seed_local, 0,
                                           torch.cuda.current_stream().cuda_stream))
-    world.combine_from_peers(st, mode=1, seed=seed_remote)
-    st.combine_send(y)
     out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
-    st.combine_recv(topk_all[rank].cuda(), w_all[rank].cuda(), out)
-    torch.cuda.synchronize()
+    run_combine(st, world, y, topk_all[rank].cuda(), w_all[rank].cuda(), out, mode=1, seed=seed_remote,
+                one_call=one_call)
     # oracle: which row does each of this rank's pairs get back?
     topk, w = topk_all[rank], w_all[rank]
     _, pair_slot = O.route(topk, e, t)
@@ -245,7 +281,8 @@ def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e):
     assert O.calc_diff(got, ref) < 1e-5
 
 
-def test_ll_config_full_size(rt):
+@ONE_CALL
+def test_ll_config_full_size(rt, one_call):
     """One GPU's share of EP=32 at 128 tokens x 7168, top-8 of 256 experts, seeded world."""
     r, rank, t, h, k, e = 32, 11, 128, 7168, 8, 256
     shape = rt.ll.LLShape(r, rank, e, t, h, k, O.ROW_FP8)
@@ -253,10 +290,7 @@ def test_ll_config_full_size(rt):
     world = rt.lb.LoopbackWorld(r, rank, seed=2024)
     world.synthesise(t, h, k, e)
     x, topk = world.own_inputs()
-    st.dispatch_send(x, topk)
-    world.dispatch_from_peers(st)
-    st.dispatch_recv()
-    torch.cuda.synchronize()
+    run_dispatch(st, world, x, topk, one_call=one_call)
     # the oracle regenerates the same world from the seed
     topk_all = O.synth_topk_idx(O.uniform_cdf(e), np.arange(r), t, k, 2024)
     assert torch.equal(world.topk_idx_all.cpu(), topk_all)
@@ -267,7 +301,8 @@ def test_ll_config_full_size(rt):
     assert int(st.packed_recv_count.sum()) == int(((topk_all // (e // r)) == rank).sum())
 
 
-def test_skewed_routing_roundtrip(rt):
+@ONE_CALL
+def test_skewed_routing_roundtrip(rt, one_call):
     """Zipf(1.2) popularity, 1 % outlier rows, EP=64 with 4 local experts, hot experts past half their slots."""
     r, rank, t, h, k, e = 64, 0, 256, 1024, 8, 256
     shape = rt.ll.LLShape(r, rank, e, t, h, k, O.ROW_FP8)
@@ -275,10 +310,7 @@ def test_skewed_routing_roundtrip(rt):
     world = rt.lb.LoopbackWorld(r, rank, seed=99)
     world.synthesise(t, h, k, e, popularity="zipf", outlier_period=100)
     x, topk = world.own_inputs()
-    st.dispatch_send(x, topk)
-    world.dispatch_from_peers(st)
-    st.dispatch_recv()
-    torch.cuda.synchronize()
+    run_dispatch(st, world, x, topk, one_call=one_call)
     topk_all = O.synth_topk_idx(O.zipf_cdf(e), np.arange(r), t, k, 99)
     x_all = O.synth_bf16_rows(np.arange(r * t, dtype=np.uint32), h, 99, outlier_period=100).view(r, t, h)
     assert torch.equal(world.topk_idx_all.cpu(), topk_all)
@@ -293,13 +325,10 @@ def test_skewed_routing_roundtrip(rt):
     for i in range(el):
         n = int(count[i])
         y[i, :n] = O.per_token_cast_back(st.packed_recv_x[i, :n].cpu(), st.packed_recv_scales[i, :n].cpu())
-    world.combine_from_peers(st, mode=0)
-    st.combine_send(y.cuda())
     g = torch.Generator().manual_seed(1)
     w = torch.softmax(torch.randn((t, k), generator=g), dim=-1)
     out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
-    st.combine_recv(topk, w.cuda(), out)
-    torch.cuda.synchronize()
+    run_combine(st, world, y.cuda(), topk, w.cuda(), out, mode=0, one_call=one_call)
     diff = O.calc_diff(x_all[rank].float() * w.sum(1, keepdim=True), out.cpu())
     assert diff < 9e-4, diff
 
@@ -323,7 +352,8 @@ def test_ll_argument_errors(rt):
     torch.cuda.synchronize()
 
 
-def test_empty_batch(rt):
+@ONE_CALL
+def test_empty_batch(rt, one_call):
     """No tokens on this rank: counts come from the peers alone, combine returns nothing."""
     r, rank, t, h, k, e = 4, 2, 6, 512, 2, 8
     x_all, topk_all, _ = make_world(r, t, h, k, e, seed=8, drop=0)
@@ -331,10 +361,7 @@ def test_empty_batch(rt):
     st = rt.ll.LowLatencyState(shape)
     world = rt.lb.LoopbackWorld(r, rank)
     world.set_inputs(x_all.cuda(), topk_all.cuda())
-    st.dispatch_send(x_all[rank, :0].cuda(), topk_all[rank, :0].cuda())
-    world.dispatch_from_peers(st)
-    st.dispatch_recv()
-    torch.cuda.synchronize()
+    run_dispatch(st, world, x_all[rank, :0].cuda(), topk_all[rank, :0].cuda(), one_call=one_call)
     xs, tks = list(x_all), list(topk_all)
     xs[rank], tks[rank] = xs[rank][:0], tks[rank][:0]
     want = O.ll_dispatch(xs, tks, rank, e, t, O.ROW_FP8)
