@@ -37,6 +37,12 @@ void clear_error();
 // Row formats; values are part of the C ABI.
 enum RowFormat : int { kRowBF16 = 0, kRowFP8 = 1, kRowFP8Pow2 = 2, kRowFP8UE8M0 = 3 };
 
+// Hook for a timing build: a harness that wants per-phase timestamps defines DEEPEP_PHASE(i)
+// before including the kernels; the library compiles it away.
+#ifndef DEEPEP_PHASE
+#define DEEPEP_PHASE(i)
+#endif
+
 constexpr int kWave = 64;
 constexpr int kGroup = 128;        // channels per FP8 scale group
 constexpr int kRowTailBytes = 16;  // {src_token, topk_slot, src_rank, 0}
@@ -66,6 +72,15 @@ __device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u,
 // Wave index inside the workgroup as a scalar, so everything derived from it
 // stays in SGPRs and row addresses become scalar loads.
 __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6); }
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load and store of the wave, which stalls kernels that keep row loads in
+// flight across the barrier; use this one where threads exchange data through LDS alone.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 
 // A 64-bit value every lane of the wave holds alike, moved to scalar registers.
 __device__ __forceinline__ uint64_t wave_uniform_u64(uint64_t v) {
@@ -104,14 +119,16 @@ __device__ __forceinline__ float max_over_8_lanes(float v) {
     return v;
 }
 
-// Inclusive sum over the wave (lane i gets sum of lanes 0..i).
+// Inclusive sum over the wave (lane i gets sum of lanes 0..i), all DPP: a log-step shift-add inside
+// each row of 16 lanes, then lane 15 of rows 0 and 2 broadcast into rows 1 and 3, then lane 31 into
+// rows 2 and 3.
 __device__ __forceinline__ int wave_inclusive_sum(int v) {
-    const int lane = lane_id();
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        int o = __shfl_up(v, d, kWave);
-        if (lane >= d) v += o;
-    }
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1, 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2, 3
     return v;
 }
 

@@ -22,45 +22,48 @@ namespace deepep {
 struct CombineSendArgs {
     const uint8_t* x;
     const int64_t* layout_range;
-    int hidden, num_local_experts, num_ranks, rank, max_tokens, parts;
+    int hidden, num_local_experts, num_ranks, rank, max_tokens, parts_log2;
     uint8_t* combine_staging;
     uint8_t* combine_send_slots;
 };
 
-// flat: [2 * num_segments + 1] ints; wave_totals: 16 ints.
-__device__ __forceinline__ void combine_send_rows(const CombineSendArgs& a, int block, int num_blocks, bool skip_own,
-                                                  int32_t* flat, int32_t* wave_totals) {
-    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
-    const int threads = blockDim.x, waves = threads >> 6;
+// No LDS and no barrier: each wave holds the segment counts and begins in registers.
+template <int kPer>
+__device__ __forceinline__ void combine_send_rows_impl(const CombineSendArgs& a, int block, int num_blocks,
+                                                       bool skip_own) {
+    const int lane = lane_id(), w = wave_in_block();
+    const int waves = int(blockDim.x) >> 6;
     const int num_ranks = a.num_ranks, max_tokens = a.max_tokens;
     const int num_segments = a.num_local_experts * num_ranks;
-    int32_t* begin = flat + num_segments + 1;
 
-    for (int s = tid; s < num_segments; s += threads) {
-        const int64_t lr = a.layout_range[s];
-        int c = int(lr & 0xffffffffll);
+    WaveSegments<kPer> seg_table;
+    int64_t ranges[kPer];
+    wave_load_int64<kPer>(a.layout_range, num_segments, lane, ranges);
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+        const int s = lane * kPer + u;
+        int c = int(ranges[u] & 0xffffffffll);
         c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
         if (skip_own && s % num_ranks == a.rank) c = 0;
-        flat[s] = c;
-        begin[s] = int(lr >> 32);
+        seg_table.cnt[u] = c;
+        seg_table.aux[u] = int(ranges[u] >> 32);
     }
-    __syncthreads();
-    block_exclusive_scan(flat, num_segments, wave_totals);
-    const int total_rows = flat[num_segments];
+    wave_segments_finish(seg_table);
 
     const int64_t row_bytes = int64_t(a.hidden) * 2;
     const int num_vec = int(row_bytes / 16);
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
-    const int64_t waves_total = int64_t(num_blocks) * waves;
-    const int parts = a.parts;
+    const int waves_total = num_blocks * waves;
+    const int parts = 1 << a.parts_log2;
+    const int num_items = seg_table.total << a.parts_log2;
 
-    for (int64_t item = int64_t(block) * waves + w; item < int64_t(total_rows) * parts; item += waves_total) {
-        const int row = int(item / parts), part = int(item - int64_t(row) * parts);
-        const int seg = __builtin_amdgcn_readfirstlane(find_segment(flat, num_segments, row));
-        const int j = row - __builtin_amdgcn_readfirstlane(flat[seg]);
+    for (int item = block * waves + w; item < num_items; item += waves_total) {
+        const int row = item >> a.parts_log2, part = item & (parts - 1);
+        int seg_first, b;
+        const int seg = wave_segments_find(seg_table, row, seg_first, b);
+        const int j = row - seg_first;
         const int le = seg / num_ranks;
         const int s = seg - le * num_ranks;
-        const int b = __builtin_amdgcn_readfirstlane(begin[seg]);
         if (b < 0 || int64_t(b) + j >= slots_per_expert) continue;  // malformed range: never read past the expert
         const uint8_t* src = a.x + (int64_t(le) * slots_per_expert + b + j) * row_bytes;
         uint8_t* dst;
@@ -76,10 +79,15 @@ __device__ __forceinline__ void combine_send_rows(const CombineSendArgs& a, int 
     }
 }
 
+__device__ __forceinline__ void combine_send_rows(const CombineSendArgs& a, int block, int num_blocks, bool skip_own) {
+    if (a.num_local_experts * a.num_ranks <= 4 * kWave)
+        combine_send_rows_impl<4>(a, block, num_blocks, skip_own);
+    else
+        combine_send_rows_impl<16>(a, block, num_blocks, skip_own);
+}
+
 __global__ __launch_bounds__(256) void ll_combine_send_kernel(CombineSendArgs a) {
-    extern __shared__ int32_t flat[];  // [num_segments + 1] then begin[num_segments]
-    __shared__ int32_t wave_totals[kMaxBlockWaves];
-    combine_send_rows(a, blockIdx.x, gridDim.x, false, flat, wave_totals);
+    combine_send_rows(a, blockIdx.x, gridDim.x, false);
 }
 
 // ---------------------------------------------------------------------
@@ -113,6 +121,32 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
     const bool lane_live = off < row_bytes;
     const int num_topk = a.num_topk;
 
+    DEEPEP_PHASE(0);
+    // Lane k fetches selection k's (slot, expert, weight) and works out where its row is: one round
+    // of loads for the whole token instead of one per selection.  The loop below reads the results
+    // back lane by lane, as wave-uniform values.
+    uint64_t my_row = 0;
+    float my_weight = 0.0f;
+    bool my_live = false;
+    if (lane < num_topk) {
+        const int64_t idx = int64_t(t) * num_topk + lane;
+        const int slot = a.pair_slot[idx];
+        const int64_t e = a.topk_idx[idx];
+        my_weight = a.topk_weights[idx];
+        if (slot >= 0 && slot < a.max_tokens && e >= 0 && e < a.num_experts) {
+            const uint8_t* row = a.combine_staging + (e * a.max_tokens + slot) * row_bytes;
+            my_live = true;
+            const int64_t le = e - own_first_expert;
+            if (own_begin != nullptr && le >= 0 && le < num_local_experts) {
+                const int64_t pos = int64_t(own_begin[le]) + slot;
+                my_live = own_begin[le] >= 0 && pos < slots_per_expert;
+                row = own_x + (le * slots_per_expert + pos) * row_bytes;
+            }
+            my_row = reinterpret_cast<uint64_t>(row);
+        }
+    }
+    const uint64_t live_mask = __ballot(my_live);
+
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
@@ -124,28 +158,17 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int k = k0 + u;
-            live[u] = false;
+            live[u] = k < num_topk && ((live_mask >> k) & 1) != 0;
             wgt[u] = 0.0f;
-            if (k < num_topk) {
-                const int slot = a.pair_slot[int64_t(t) * num_topk + k];
-                const int64_t e = a.topk_idx[int64_t(t) * num_topk + k];
-                if (slot >= 0 && slot < a.max_tokens && e >= 0 && e < a.num_experts) {
-                    const uint8_t* row = a.combine_staging + (e * a.max_tokens + slot) * row_bytes;
-                    bool ok = true;
-                    const int64_t le = e - own_first_expert;
-                    if (own_begin != nullptr && le >= 0 && le < num_local_experts) {
-                        const int64_t pos = int64_t(own_begin[le]) + slot;
-                        ok = own_begin[le] >= 0 && pos < slots_per_expert;
-                        row = own_x + (le * slots_per_expert + pos) * row_bytes;
-                    }
-                    if (ok) {
-                        live[u] = true;
-                        wgt[u] = a.topk_weights[int64_t(t) * num_topk + k];
-                        if (lane_live) v[u] = *reinterpret_cast<const u32x4*>(row + off);
-                    }
-                }
+            if (live[u]) {
+                const uint32_t lo32 = __builtin_amdgcn_readlane(uint32_t(my_row), k);
+                const uint32_t hi32 = __builtin_amdgcn_readlane(uint32_t(my_row >> 32), k);
+                wgt[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_weight), k));
+                const uint8_t* row = reinterpret_cast<const uint8_t*>((uint64_t(hi32) << 32) | lo32);
+                if (lane_live) v[u] = *reinterpret_cast<const u32x4*>(row + off);
             }
         }
+        DEEPEP_PHASE(1);
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             if (!live[u] || !lane_live) continue;
@@ -156,6 +179,7 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
             }
         }
     }
+    DEEPEP_PHASE(2);
     if (lane_live) {
         u32x4 o;
 #pragma unroll
@@ -179,19 +203,18 @@ __global__ __launch_bounds__(256) void ll_combine_recv_kernel(CombineRecvArgs a)
 // ---------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ll_combine_fused_kernel(CombineSendArgs sa, CombineRecvArgs ra,
                                                                int num_recv_blocks) {
-    extern __shared__ int32_t dyn_lds[];  // reduce: own_begin[E_l]; row return: [2 * segments + 1]
-    __shared__ int32_t wave_totals[kMaxBlockWaves];
+    extern __shared__ int32_t dyn_lds[];  // reduce workgroups: own_begin[E_l]
     const int block = blockIdx.x;
     if (block < num_recv_blocks) {
         for (int le = threadIdx.x; le < sa.num_local_experts; le += blockDim.x) {
             const int64_t lr = sa.layout_range[le * sa.num_ranks + sa.rank];
             dyn_lds[le] = (lr & 0xffffffffll) > 0 ? int(lr >> 32) : 0;
         }
-        __syncthreads();
+        lds_barrier();
         combine_recv_piece(ra, int64_t(block) * 4 + wave_in_block(), sa.x, dyn_lds, sa.rank * sa.num_local_experts,
                            sa.num_local_experts, int64_t(sa.max_tokens) * sa.num_ranks);
     } else {
-        combine_send_rows(sa, block - num_recv_blocks, int(gridDim.x) - num_recv_blocks, true, dyn_lds, wave_totals);
+        combine_send_rows(sa, block - num_recv_blocks, int(gridDim.x) - num_recv_blocks, true);
     }
 }
 
@@ -203,7 +226,7 @@ static CombineSendArgs make_combine_send_args(const void* x, const int64_t* layo
     sa.layout_range = layout_range;
     sa.hidden = hidden, sa.num_local_experts = num_experts / num_ranks, sa.num_ranks = num_ranks, sa.rank = rank;
     sa.max_tokens = max_tokens;
-    sa.parts = choose_row_parts(int64_t(num_experts) * max_tokens, int64_t(hidden) * 2);
+    sa.parts_log2 = choose_row_parts_log2(int64_t(num_experts) * max_tokens, int64_t(hidden) * 2);
     sa.combine_staging = reinterpret_cast<uint8_t*>(combine_staging);
     sa.combine_send_slots = reinterpret_cast<uint8_t*>(combine_send_slots);
     return sa;
@@ -231,6 +254,7 @@ static int check_combine_send_args(const void* x, const int64_t* layout_range, i
     EP_HOST_ASSERT(num_experts <= 1024);
     EP_HOST_ASSERT(x != nullptr && layout_range != nullptr && combine_staging != nullptr);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(layout_range) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combine_staging) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combine_send_slots) & 15) == 0);
     EP_HOST_ASSERT(int64_t(num_experts) * max_tokens < (int64_t(1) << 31));
@@ -292,11 +316,10 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
     const CombineSendArgs sa = make_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
                                                       num_max_dispatch_tokens_per_rank, combine_staging,
                                                       combine_send_slots);
-    int64_t blocks = (max_rows * sa.parts + 3) / 4;
+    int64_t blocks = ((max_rows << sa.parts_log2) + 3) / 4;
     const int64_t cap = max_rows > kLargeBatchRows ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
-    const size_t lds = size_t(2 * num_experts + 1) * sizeof(int32_t);
-    ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, lds, hs>>>(sa);
+    ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, 0, hs>>>(sa);
     EP_LAUNCH_CHECK();
     return 0;
 }
@@ -349,12 +372,10 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
     int64_t rows = expected_rows > 0 ? expected_rows : int64_t(num_max_dispatch_tokens_per_rank) * num_topk;
     rows += rows / 8 + 16;
     if (rows > max_rows) rows = max_rows;
-    int64_t send_blocks = combine_send_slots != nullptr ? (rows * sa.parts + 3) / 4 : 0;
+    int64_t send_blocks = combine_send_slots != nullptr ? ((rows << sa.parts_log2) + 3) / 4 : 0;
     if (send_blocks > 1024) send_blocks = 1024;
     if (recv_blocks + send_blocks == 0) return 0;
-    const size_t need_send = size_t(2 * num_experts + 1) * sizeof(int32_t);
-    const size_t need_recv = size_t(sa.num_local_experts) * sizeof(int32_t);
-    const size_t lds = need_send > need_recv ? need_send : need_recv;
+    const size_t lds = size_t(sa.num_local_experts) * sizeof(int32_t);
     ll_combine_fused_kernel<<<dim3(unsigned(recv_blocks + send_blocks)), 256, lds,
                               reinterpret_cast<hipStream_t>(stream)>>>(sa, ra, int(recv_blocks));
     EP_LAUNCH_CHECK();

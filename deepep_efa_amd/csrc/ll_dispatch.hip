@@ -202,12 +202,12 @@ __device__ __forceinline__ void send_count_block(const SendArgs& a, int b, int32
     const int src_rank = a.src_ranks != nullptr ? a.src_ranks[b] : a.rank;
     const int64_t* my_topk = a.topk_idx + int64_t(b) * n;
     for (int j = tid; j < a.num_experts; j += blockDim.x) lds_hist[j] = 0;
-    __syncthreads();
+    lds_barrier();
     for (int i = tid; i < n; i += blockDim.x) {
         const int64_t v = my_topk[i];
         if (v >= 0 && v < a.num_experts) atomicAdd(&lds_hist[int(v)], 1);
     }
-    __syncthreads();
+    lds_barrier();
     for (int e = tid; e < a.num_experts; e += blockDim.x)
         emit_expert_count(e, lds_hist[e], a.num_experts, a.num_ranks, a.rank, src_rank, a.max_tokens, a.recv_count,
                           a.send_count);
@@ -237,6 +237,7 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
     const int64_t scale_pad = align16(scale_bytes);
     const int64_t stride = data_pad + scale_pad + kRowTailBytes;
 
+    DEEPEP_PHASE(0);
     // ---- issue this wave's row loads ------------------------------------
     u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
     bool lane_live;
@@ -275,6 +276,18 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             }
         }
     }
+    DEEPEP_PHASE(1);
+    // small batch: the entries before this token, fetched now so that their latency overlaps the
+    // loads above (each thread takes every blockDim-th entry; four cover 2048 entries at 512 threads)
+    constexpr int kSweepAhead = 4;
+    int64_t ahead[kSweepAhead];
+    if (a.num_chunks <= 1) {
+#pragma unroll
+        for (int r = 0; r < kSweepAhead; ++r) {
+            const int i = tid + r * int(blockDim.x);
+            ahead[r] = i < entry0 ? my_topk[i] : -1;
+        }
+    }
     if (a.num_chunks > 1) {  // slots were ranked by ll_route_slots_kernel
         if (tid < num_topk && my_expert >= 0)
             my_slot = reinterpret_cast<const int32_t*>(a.scratch_base + int64_t(b) * a.scratch_stride)[entry0 + tid];
@@ -283,14 +296,23 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             lds.sel_expert[tid] = my_expert;
             lds.sel_count[tid] = 0;
         }
-        __syncthreads();
-        for (int i = tid; i < entry0; i += blockDim.x) {
+        lds_barrier();
+        DEEPEP_PHASE(2);
+#pragma unroll
+        for (int r = 0; r < kSweepAhead; ++r) {
+            const int64_t v = ahead[r];
+            if (v < 0 || v >= num_experts) continue;
+            for (int k = 0; k < num_topk; ++k)
+                if (int(v) == lds.sel_expert[k]) atomicAdd(&lds.sel_count[k], 1);
+        }
+        for (int i = tid + kSweepAhead * int(blockDim.x); i < entry0; i += blockDim.x) {
             const int64_t v = my_topk[i];
             if (v < 0 || v >= num_experts) continue;
             for (int k = 0; k < num_topk; ++k)
                 if (int(v) == lds.sel_expert[k]) atomicAdd(&lds.sel_count[k], 1);
         }
-        __syncthreads();
+        lds_barrier();
+        DEEPEP_PHASE(3);
         if (tid < num_topk && my_expert >= 0) {
             my_slot = lds.sel_count[tid];
             for (int k2 = 0; k2 < tid; ++k2)  // the same expert named earlier in this token
@@ -327,7 +349,8 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             }
         }
     }
-    __syncthreads();
+    lds_barrier();
+    DEEPEP_PHASE(4);
     if (!wave_live) return;
 
     // ---- quantise, then one store per selection ---------------------------
@@ -335,6 +358,7 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
     uint32_t scale_bits = 0;
     if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
     const int64_t lane_off = int64_t(piece) * 1024 + lane * 16;
+    DEEPEP_PHASE(5);
     for (int k = part; k < num_topk; k += split) {
         uint8_t* row = reinterpret_cast<uint8_t*>(wave_uniform_u64(lds.sel_row[k]));
         if (row == nullptr) continue;
@@ -349,6 +373,7 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             }
         }
     }
+    DEEPEP_PHASE(6);
 }
 
 template <int kFmt>
@@ -379,7 +404,7 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs 
 struct RecvArgs {
     const uint8_t* recv_staging;
     const int32_t* recv_count;
-    int hidden, num_local_experts, num_ranks, max_tokens, fmt, parts;
+    int hidden, num_local_experts, num_ranks, max_tokens, fmt, parts_log2;
     uint8_t* packed_x;
     uint8_t* packed_scales;
     int32_t* src_info;
@@ -388,77 +413,97 @@ struct RecvArgs {
     int32_t* stats;
 };
 
-// flat: [num_segments + 1] ints (+ num_local_experts when own_topk != null); wave_totals: 16 ints.
-__device__ __forceinline__ void recv_rows(const RecvArgs& a, int block, int num_blocks, const int64_t* own_topk,
-                                          int own_entries, int own_rank, int32_t* flat, int32_t* wave_totals) {
+__device__ __forceinline__ int clamp_count(int c, int max_tokens) {
+    return c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+}
+
+// Workgroups [0, num_copy_blocks) copy rows; workgroup num_copy_blocks writes layout_range,
+// packed_count and stats and copies nothing, so the copying waves never wait for a barrier:
+// each builds the segment prefix in its own registers (WaveSegments) from the E counts.
+// lds: [num_segments + 1 + num_local_experts] ints; wave_totals: 16 ints.
+template <int kPer>
+__device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int num_copy_blocks,
+                                               const int64_t* own_topk, int own_entries, int own_rank, int32_t* lds,
+                                               int32_t* wave_totals) {
     const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
     const int threads = blockDim.x, waves = threads >> 6;
-    const int num_segments = a.num_local_experts * a.num_ranks;
     const int num_ranks = a.num_ranks, max_tokens = a.max_tokens;
+    const int num_segments = a.num_local_experts * num_ranks;
+    const bool recount_own = own_topk != nullptr;
 
-    if (own_topk != nullptr) {
-        int32_t* own_cnt = flat + num_segments + 1;
+    WaveSegments<kPer> seg_table;
+    DEEPEP_PHASE(0);
+    wave_load_int32<kPer>(a.recv_count, num_segments, lane, seg_table.cnt);
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+        seg_table.aux[u] = 0;
+        seg_table.cnt[u] = clamp_count(seg_table.cnt[u], max_tokens);
+    }
+    int32_t* own_cnt = lds + num_segments + 1;
+    if (recount_own) {  // rows from this rank itself: recount them from its own indices
         for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
-        __syncthreads();
+        lds_barrier();
         const int64_t first = int64_t(own_rank) * a.num_local_experts;
         for (int i = tid; i < own_entries; i += threads) {
             const int64_t v = own_topk[i] - first;
             if (v >= 0 && v < a.num_local_experts) atomicAdd(&own_cnt[int(v)], 1);
         }
-        for (int s = tid; s < num_segments; s += threads) {
-            if (s % num_ranks == own_rank) continue;
-            const int c = a.recv_count[s];
-            flat[s] = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
-        }
-        __syncthreads();
-        for (int le = tid; le < a.num_local_experts; le += threads) {
-            const int c = own_cnt[le];
-            flat[le * num_ranks + own_rank] = c > max_tokens ? max_tokens : c;
-        }
-    } else {
-        for (int s = tid; s < num_segments; s += threads) {
-            const int c = a.recv_count[s];
-            flat[s] = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+        lds_barrier();
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {  // whatever recv_count holds for the own segments is stale
+            const int s = lane * kPer + u;
+            if (s < num_segments && s % num_ranks == own_rank)
+                seg_table.cnt[u] = clamp_count(own_cnt[s / num_ranks], max_tokens);
         }
     }
-    __syncthreads();
-    block_exclusive_scan(flat, num_segments, wave_totals);
-    const int total_rows = flat[num_segments];
 
-    if (block == 0) {
+    if (block == num_copy_blocks) {  // the metadata workgroup
+        for (int s = tid; s < num_segments; s += threads) {
+            const bool own = recount_own && s % num_ranks == own_rank;
+            lds[s] = clamp_count(own ? own_cnt[s / num_ranks] : a.recv_count[s], max_tokens);
+        }
+        lds_barrier();
+        block_exclusive_scan(lds, num_segments, wave_totals);
         for (int s = tid; s < num_segments; s += threads) {
             const int le = s / num_ranks;
-            const int64_t cnt = flat[s + 1] - flat[s];
-            const int64_t begin = flat[s] - flat[le * num_ranks];
+            const int64_t cnt = lds[s + 1] - lds[s];
+            const int64_t begin = lds[s] - lds[le * num_ranks];
             a.layout_range[s] = cnt > 0 ? ((begin << 32) | cnt) : 0;
         }
         for (int le = tid; le < a.num_local_experts; le += threads) {
-            const int c = flat[(le + 1) * num_ranks] - flat[le * num_ranks];
+            const int c = lds[(le + 1) * num_ranks] - lds[le * num_ranks];
             a.packed_count[le] = c;
             if (a.stats != nullptr) a.stats[le] += c;
         }
+        return;
     }
 
+    wave_segments_finish(seg_table);
+    DEEPEP_PHASE(1);
     const int64_t data_bytes = row_data_bytes(a.hidden, a.fmt);
     const int64_t data_pad = align16(data_bytes);
     const int64_t scale_bytes = row_scale_bytes(a.hidden, a.fmt);
     const int64_t stride = data_pad + align16(scale_bytes) + kRowTailBytes;
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
-    const int64_t waves_total = int64_t(num_blocks) * waves;
+    const int waves_total = num_copy_blocks * waves;
     const int num_vec = int(data_bytes / 16);
-    const int parts = a.parts;
-    for (int64_t item = int64_t(block) * waves + w; item < int64_t(total_rows) * parts; item += waves_total) {
-        const int row = int(item / parts), part = int(item - int64_t(row) * parts);
-        const int seg = __builtin_amdgcn_readfirstlane(find_segment(flat, num_segments, row));
+    const int parts = 1 << a.parts_log2;
+    const int num_items = seg_table.total << a.parts_log2;
+    for (int item = block * waves + w; item < num_items; item += waves_total) {
+        const int row = item >> a.parts_log2, part = item & (parts - 1);
+        int seg_first, unused;
+        const int seg = wave_segments_find(seg_table, row, seg_first, unused);
         const int le = seg / num_ranks;
-        if (own_topk != nullptr && seg - le * num_ranks == own_rank) continue;
-        const int j = row - __builtin_amdgcn_readfirstlane(flat[seg]);
-        const int64_t slot = int64_t(row) - __builtin_amdgcn_readfirstlane(flat[le * num_ranks]);
+        if (recount_own && seg - le * num_ranks == own_rank) continue;  // placed by the send workgroups
+        const int j = row - seg_first;
+        const int slot = row - wave_segments_prefix(seg_table, le * num_ranks);
         const uint8_t* src = a.recv_staging + (int64_t(seg) * max_tokens + j) * stride;
         const int64_t out_row = int64_t(le) * slots_per_expert + slot;
         int v_begin, v_end;
         row_part_range(num_vec, parts, part, v_begin, v_end);
+        DEEPEP_PHASE(2);
         wave_copy_vec16(src, a.packed_x + out_row * data_bytes, v_begin, v_end, lane);
+        DEEPEP_PHASE(3);
         if (part != parts - 1) continue;  // the last part is the shortest: it also carries scales and source index
         if (a.packed_scales != nullptr && scale_bytes > 0) {
             const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src + data_pad);
@@ -470,10 +515,18 @@ __device__ __forceinline__ void recv_rows(const RecvArgs& a, int block, int num_
     }
 }
 
+__device__ __forceinline__ void recv_rows(const RecvArgs& a, int block, int num_copy_blocks, const int64_t* own_topk,
+                                          int own_entries, int own_rank, int32_t* lds, int32_t* wave_totals) {
+    if (a.num_local_experts * a.num_ranks <= 4 * kWave)
+        recv_rows_impl<4>(a, block, num_copy_blocks, own_topk, own_entries, own_rank, lds, wave_totals);
+    else
+        recv_rows_impl<16>(a, block, num_copy_blocks, own_topk, own_entries, own_rank, lds, wave_totals);
+}
+
 __global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a) {
-    extern __shared__ int32_t flat[];  // [num_segments + 1]
+    extern __shared__ int32_t flat[];  // [num_segments + 1], used by the metadata workgroup (the last one)
     __shared__ int32_t wave_totals[kMaxBlockWaves];
-    recv_rows(a, blockIdx.x, gridDim.x, nullptr, 0, 0, flat, wave_totals);
+    recv_rows(a, blockIdx.x, int(gridDim.x) - 1, nullptr, 0, 0, flat, wave_totals);
 }
 
 // ---------------------------------------------------------------------
@@ -500,7 +553,7 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_dispatch_fused_kernel
     } else if (block == num_send_blocks) {
         send_count_block(sa, 0, dyn_lds);
     } else {
-        recv_rows(ra, block - num_send_blocks - 1, int(gridDim.x) - num_send_blocks - 1, sa.topk_idx,
+        recv_rows(ra, block - num_send_blocks - 1, int(gridDim.x) - num_send_blocks - 2, sa.topk_idx,
                   sa.num_tokens * sa.num_topk, sa.rank, dyn_lds, wave_totals);
     }
 }
@@ -586,7 +639,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
         const int num_send_blocks = blocks_per_token * num_tokens;
         int64_t fused_recv_blocks = (fused_recv_wave_items + waves - 1) / waves;
         fused_recv_blocks = fused_recv_blocks < 1 ? 1 : (fused_recv_blocks > 1024 ? 1024 : fused_recv_blocks);
-        const int64_t total = int64_t(num_send_blocks) + 1 + fused_recv_blocks;
+        const int64_t total = int64_t(num_send_blocks) + 1 + fused_recv_blocks + 1;  // + counting, + metadata
         EP_HOST_ASSERT(total < (int64_t(1) << 31));
         const int num_segments = fused_recv->num_local_experts * fused_recv->num_ranks;
         const size_t need_recv = size_t(num_segments + 1 + fused_recv->num_local_experts) * sizeof(int32_t);
@@ -696,6 +749,7 @@ static int check_recv_args(const void* recv_staging, const int32_t* recv_count, 
     EP_HOST_ASSERT(packed_recv_src_info != nullptr && packed_recv_layout_range != nullptr &&
                    packed_recv_count != nullptr);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_staging) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_count) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_x) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_scales) & 3) == 0);
     EP_HOST_ASSERT(int64_t(num_experts) * max_tokens < (int64_t(1) << 31));
@@ -711,7 +765,7 @@ static RecvArgs make_recv_args(const void* recv_staging, const int32_t* recv_cou
     ra.recv_count = recv_count;
     ra.hidden = hidden, ra.num_local_experts = num_experts / num_ranks, ra.num_ranks = num_ranks;
     ra.max_tokens = max_tokens, ra.fmt = row_format;
-    ra.parts = choose_row_parts(int64_t(num_experts) * max_tokens, row_data_bytes(hidden, row_format));
+    ra.parts_log2 = choose_row_parts_log2(int64_t(num_experts) * max_tokens, row_data_bytes(hidden, row_format));
     ra.packed_x = reinterpret_cast<uint8_t*>(packed_recv_x);
     ra.packed_scales = reinterpret_cast<uint8_t*>(packed_recv_scales);
     ra.src_info = packed_recv_src_info, ra.layout_range = packed_recv_layout_range;
@@ -764,11 +818,11 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
                                        num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                                        packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
                                        cumulative_local_expert_recv_stats);
-    int64_t blocks = (max_rows * ra.parts + 3) / 4;
+    int64_t blocks = ((max_rows << ra.parts_log2) + 3) / 4;
     const int64_t cap = max_rows > kLargeBatchRows ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(num_experts + 1) * sizeof(int32_t);
-    ll_recv_kernel<<<dim3(unsigned(blocks)), 256, lds, hs>>>(ra);
+    ll_recv_kernel<<<dim3(unsigned(blocks) + 1), 256, lds, hs>>>(ra);  // + the metadata workgroup
     EP_LAUNCH_CHECK();
     return 0;
 }
@@ -816,7 +870,7 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, i
     return launch_send_side(x, topk_idx, nullptr, 1, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
                             num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count, send_slots,
                             send_count, pair_slot, workspace, workspace_bytes,
-                            reinterpret_cast<hipStream_t>(stream), &ra, rows * ra.parts);
+                            reinterpret_cast<hipStream_t>(stream), &ra, rows << ra.parts_log2);
 }
 
 }  // extern "C"

@@ -26,7 +26,7 @@ __device__ __forceinline__ void block_exclusive_scan(int32_t* data, int n, int32
         if (lo + j < n) sum += data[lo + j];
     const int incl = wave_inclusive_sum(sum);
     if (lane == kWave - 1) wave_totals[w] = incl;
-    __syncthreads();
+    lds_barrier();
     int offset = incl - sum, total = 0;
     for (int w2 = 0; w2 < waves; ++w2) {
         const int t = wave_totals[w2];
@@ -41,7 +41,7 @@ __device__ __forceinline__ void block_exclusive_scan(int32_t* data, int n, int32
             run += v;
         }
     if (tid == 0) data[n] = total;
-    __syncthreads();
+    lds_barrier();
 }
 
 // Largest seg with flat[seg] <= row, for flat[] non-decreasing, flat[0] = 0.
@@ -52,6 +52,101 @@ __device__ __forceinline__ int find_segment(const int32_t* flat, int num_segment
         if (flat[mid] <= row) lo = mid; else hi = mid;
     }
     return lo;
+}
+
+// ---------------------------------------------------------------------
+// The same prefix, held by one wave in registers: no LDS and no barrier, so a
+// wave can start looking up rows as soon as its own loads of the counts are
+// back.  Lane l holds the counts of segments [l * kPer, (l + 1) * kPer) and the
+// number of rows in all lower lanes' segments.  kPer is a compile-time 4 (up to
+// 256 segments) or 16 (up to 1024) so that every index below is static and the
+// arrays stay in registers.
+// ---------------------------------------------------------------------
+template <int kPer>
+struct WaveSegments {
+    int cnt[kPer];
+    int aux[kPer];  // one caller-defined value per segment, returned by the lookup
+    int lane_base;  // rows in the segments held by lower lanes
+    int total;      // rows in all segments
+};
+
+// Lane l's kPer consecutive values p[l * kPer + u] (0 beyond n), as 16-byte loads where a whole
+// vector lies inside the array.  p must be 16-byte aligned.
+template <int kPer>
+__device__ __forceinline__ void wave_load_int32(const int32_t* __restrict__ p, int n, int lane, int (&out)[kPer]) {
+    static_assert(kPer % 4 == 0, "whole 16-byte vectors per lane");
+#pragma unroll
+    for (int v = 0; v < kPer / 4; ++v) {
+        const int s0 = lane * kPer + v * 4;
+        if (s0 + 3 < n) {
+            const u32x4 q = *reinterpret_cast<const u32x4*>(p + s0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[v * 4 + i] = int(q[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) out[v * 4 + i] = s0 + i < n ? p[s0 + i] : 0;
+        }
+    }
+}
+
+template <int kPer>
+__device__ __forceinline__ void wave_load_int64(const int64_t* __restrict__ p, int n, int lane,
+                                                int64_t (&out)[kPer]) {
+    static_assert(kPer % 2 == 0, "whole 16-byte vectors per lane");
+#pragma unroll
+    for (int v = 0; v < kPer / 2; ++v) {
+        const int s0 = lane * kPer + v * 2;
+        if (s0 + 1 < n) {
+            const u32x4 q = *reinterpret_cast<const u32x4*>(p + s0);
+            out[v * 2] = int64_t((uint64_t(q[1]) << 32) | q[0]);
+            out[v * 2 + 1] = int64_t((uint64_t(q[3]) << 32) | q[2]);
+        } else {
+            out[v * 2] = s0 < n ? p[s0] : 0;
+            out[v * 2 + 1] = 0;
+        }
+    }
+}
+
+// Finishes a table whose cnt[] the caller has filled (zero beyond the last segment).
+template <int kPer>
+__device__ __forceinline__ void wave_segments_finish(WaveSegments<kPer>& t) {
+    int mine = 0;
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) mine += t.cnt[u];
+    const int incl = wave_inclusive_sum(mine);
+    t.lane_base = incl - mine;
+    t.total = __builtin_amdgcn_readlane(incl, kWave - 1);
+}
+
+// Rows before segment q (wave-uniform q in [0, 64 * kPer]).
+template <int kPer>
+__device__ __forceinline__ int wave_segments_prefix(const WaveSegments<kPer>& t, int q) {
+    q = __builtin_amdgcn_readfirstlane(q);
+    const int owner = q / kPer, within = q % kPer;
+    if (owner >= kWave) return t.total;
+    int run = t.lane_base;
+#pragma unroll
+    for (int u = 0; u < kPer; ++u)
+        if (u < within) run += t.cnt[u];
+    return __builtin_amdgcn_readlane(run, owner);
+}
+
+// Segment holding row (wave-uniform, 0 <= row < total); seg_first receives the rows before it,
+// seg_aux the segment's aux value.
+template <int kPer>
+__device__ __forceinline__ int wave_segments_find(const WaveSegments<kPer>& t, int row, int& seg_first,
+                                                  int& seg_aux) {
+    // the last lane whose base is <= row owns the row (empty lanes share their successor's base)
+    const int owner = __builtin_amdgcn_readfirstlane(__popcll(__ballot(t.lane_base <= row)) - 1);
+    int run = t.lane_base, found = 0, first = t.lane_base, aux = 0;
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+        if (run <= row && row < run + t.cnt[u]) found = u, first = run, aux = t.aux[u];
+        run += t.cnt[u];
+    }
+    seg_first = __builtin_amdgcn_readlane(first, owner);
+    seg_aux = __builtin_amdgcn_readlane(aux, owner);
+    return owner * kPer + __builtin_amdgcn_readlane(found, owner);
 }
 
 // Copies 16-byte vectors [v_begin, v_end) of a row with one wave, eight loads
@@ -83,14 +178,18 @@ __device__ __forceinline__ void row_part_range(int num_vec, int parts, int part,
     v_end = min(v_begin + per * kWave, num_vec);
 }
 
-// Host-side choice of `parts`: small problems cannot fill the chip with one wave per row.
-inline int choose_row_parts(int64_t max_rows, int64_t row_bytes) {
+// Host-side choice of the row split (log2 of the parts): small problems cannot fill the chip with
+// one wave per row.
+inline int choose_row_parts_log2(int64_t max_rows, int64_t row_bytes) {
+    if (max_rows > (int64_t(1) << 18)) return 0;
     if (const char* s = getenv("DEEPEP_ROW_PARTS")) {
         const int v = atoi(s);
-        if (v >= 1 && v <= 8) return v;
+        if (v == 1) return 0;
+        if (v == 2) return 1;
+        if (v == 4) return 2;
+        if (v == 8) return 3;
     }
-    if (max_rows > (int64_t(1) << 18)) return 1;
-    return row_bytes > 8192 ? 4 : 2;
+    return row_bytes > 8192 ? 2 : 1;
 }
 
 // ---------------------------------------------------------------------
