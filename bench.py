@@ -1,15 +1,18 @@
 """Bench of the low-latency dispatch + combine hot path on one MI355X.
 
-A step is one pass of the hot path for one rank of an EP=32 world:
-dispatch_send (route + quantise + pack) -> dispatch_recv -> combine_send ->
-combine_recv, for 128 tokens x 7168 hidden, top-8 of 256 experts, FP8
-dispatch and BF16 combine.  The 31 peer ranks' rows are synthesised in HBM
-from a seed before the timed region and stay resident.
+A step is one pass of the hot path for one rank of an EP=32 world: dispatch
+(route + quantise + pack into per-expert slots, then compaction of the rows
+received) and combine (return of the expert outputs, then the top-k weighted
+reduce), for 128 tokens x 7168 hidden, top-8 of 256 experts, FP8 dispatch and
+BF16 combine.  At this size each of the two is one kernel launch.  The 31 peer
+ranks' rows are synthesised in HBM from a seed before the timed region and
+stay resident.
 
-Prints ONE JSON line.  `value` is microseconds per dispatch+combine measured
-over K back-to-back steps on one stream (launch gaps included); the
-per-kernel durations, measured with events around each entry point, and the
-roofline of the slowest kernel are in the same line.
+Prints ONE JSON line.  `value` is microseconds of stream time per step over K
+steps: the steps are enqueued by HIP-graph replays so the GPU never waits for
+the host (launching call by call from Python costs more than the kernels take;
+that figure is reported beside it).  Per-entry durations are measured the same
+way; the roofline of the slower of the two step kernels is in the same line.
 """
 import argparse
 import json
@@ -267,65 +270,66 @@ def main():
         for name in phase_calls:
             calls[name]()
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    wall0 = time.perf_counter()
-    ev0.record()
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - wall0
-    us_per_step = ev0.elapsed_time(ev1) * 1e3 / args.steps
-    for _ in range(10):
-        step_by_phase()
-    torch.cuda.synchronize()
-    ev0.record()
-    for _ in range(args.steps):
-        step_by_phase()
-    ev1.record()
-    torch.cuda.synchronize()
-    us_per_phase_step = ev0.elapsed_time(ev1) * 1e3 / args.steps
 
-    # per entry point: the same call `steps` times back to back between two events.  Consecutive
-    # launches on one stream leave well under a microsecond between kernels on this GPU, so the
-    # mean is the kernel's duration (the rocprofv3 summary under profiles/ is the cross-check).
-    per_call = {}
-    for name, fn in calls.items():
-        for _ in range(10):
+    def time_eager(fn, warmup, reps):
+        """`reps` calls launched one by one from Python: includes the host's launch cost when that
+        is longer than the kernels (it is, at this size: ~9 us per call through ctypes)."""
+        for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
+        wall0 = time.perf_counter()
         ev0.record()
-        for _ in range(args.steps):
+        for _ in range(reps):
             fn()
         ev1.record()
         torch.cuda.synchronize()
-        per_call[name] = ev0.elapsed_time(ev1) * 1e3 / args.steps
+        return ev0.elapsed_time(ev1) * 1e3 / reps, (time.perf_counter() - wall0) * 1e6 / reps
 
-    graph_us = None
+    def time_graph(fn, warmup, reps):
+        """The same `reps` calls, enqueued by HIP-graph replays of `per_graph` calls each, so that the
+        GPU never waits for the host: the time is the stream's, kernels plus the gaps between them."""
+        per_graph = max(d for d in range(1, 26) if reps % d == 0)
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        with torch.cuda.graph(g):
+            for _ in range(per_graph):
+                fn()
+        for _ in range(max(1, warmup // per_graph)):
+            g.replay()
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(reps // per_graph):
+            g.replay()
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) * 1e3 / reps, per_graph
+
+    eager_us, host_wall_us = time_eager(step, args.warmup, args.steps)
+    eager_phase_us, _ = time_eager(step_by_phase, 10, args.steps)
+    graph_us = graph_phase_us = per_graph = None
+    per_call = {}
+    timing = "eager launches"
     if not args.no_graph:
         try:
-            g = torch.cuda.CUDAGraph()
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                step()
-            torch.cuda.current_stream().wait_stream(side)
-            with torch.cuda.graph(g):
-                step()
-            for _ in range(10):
-                g.replay()
-            torch.cuda.synchronize()
-            ev0.record()
-            for _ in range(args.steps):
-                g.replay()
-            ev1.record()
-            torch.cuda.synchronize()
-            graph_us = ev0.elapsed_time(ev1) * 1e3 / args.steps
-        except Exception as exc:  # graph capture is an extra, never the headline
-            graph_us = f"unavailable: {type(exc).__name__}"
+            graph_us, per_graph = time_graph(step, args.warmup, args.steps)
+            graph_phase_us, _ = time_graph(step_by_phase, 10, args.steps)
+            for name, fn in calls.items():
+                per_call[name], _ = time_graph(fn, 10, args.steps)
+            timing = f"HIP graphs of {per_graph} steps each, replayed back to back"
+        except Exception as exc:  # fall back to eager timing, and say so
+            graph_us = None
+            timing = f"eager launches (graph capture unavailable: {type(exc).__name__})"
+    if graph_us is None:
+        # the same call `steps` times back to back between two events
+        for name, fn in calls.items():
+            per_call[name], _ = time_eager(fn, 10, args.steps)
+    us_per_step = graph_us if graph_us is not None else eager_us
+    us_per_phase_step = graph_phase_us if graph_phase_us is not None else eager_phase_us
 
     nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r, own)
     kernels = {n: {"us": round(per_call[n], 2), "bytes": nbytes[n],
@@ -352,8 +356,9 @@ def main():
                    "launches_per_step": 2},
         "kernel_time_us": round(sum(per_call[n] for n in step_calls), 2),
         "step_by_phase_us": round(us_per_phase_step, 2),  # the same step as four launches
-        "graph_replay_us": graph_us if not isinstance(graph_us, float) else round(graph_us, 2),
-        "host_wall_us_per_step": round(wall * 1e6 / args.steps, 2),
+        "timing": timing,
+        "eager_us_per_step": round(eager_us, 2),  # launched call by call from Python: host-bound
+        "eager_host_wall_us_per_step": round(host_wall_us, 2),
         "kernels": kernels,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},

@@ -73,6 +73,16 @@ __device__ __forceinline__ int lane_id() { return __builtin_amdgcn_mbcnt_hi(~0u,
 // stays in SGPRs and row addresses become scalar loads.
 __device__ __forceinline__ int wave_in_block() { return __builtin_amdgcn_readfirstlane(int(threadIdx.x) >> 6); }
 
+// Stores through a pointer the compiler cannot prove to be global memory (one rebuilt from
+// integers, say) are emitted as flat stores, which also tick the LDS counter; these say "global".
+typedef __attribute__((address_space(1))) u32x4 global_u32x4;
+typedef __attribute__((address_space(1))) uint32_t global_u32;
+typedef __attribute__((address_space(1))) uint8_t global_u8;
+__device__ __forceinline__ void store_global(uint8_t* p, u32x4 v) { *(global_u32x4*)(p) = v; }
+__device__ __forceinline__ void store_global(uint8_t* p, uint32_t v) { *(global_u32*)(p) = v; }
+__device__ __forceinline__ u32x4 load_global_u32x4(const uint8_t* p) { return *(const global_u32x4*)(p); }
+__device__ __forceinline__ void store_global_byte(uint8_t* p, uint8_t v) { *(global_u8*)(p) = v; }
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load and store of the wave, which stalls kernels that keep row loads in
 // flight across the barrier; use this one where threads exchange data through LDS alone.

@@ -75,7 +75,7 @@ __device__ __forceinline__ void combine_send_rows_impl(const CombineSendArgs& a,
             continue;
         int v_begin, v_end;
         row_part_range(num_vec, parts, part, v_begin, v_end);
-        wave_copy_vec16(src, dst, v_begin, v_end, lane);
+        wave_copy_vec16<4>(src, dst, v_begin, v_end, lane);
     }
 }
 
@@ -165,7 +165,7 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
                 const uint32_t hi32 = __builtin_amdgcn_readlane(uint32_t(my_row >> 32), k);
                 wgt[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_weight), k));
                 const uint8_t* row = reinterpret_cast<const uint8_t*>((uint64_t(hi32) << 32) | lo32);
-                if (lane_live) v[u] = *reinterpret_cast<const u32x4*>(row + off);
+                if (lane_live) v[u] = load_global_u32x4(row + off);
             }
         }
         DEEPEP_PHASE(1);

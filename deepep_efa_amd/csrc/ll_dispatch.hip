@@ -188,11 +188,10 @@ struct DirectOut {
     int32_t* src_info;
 };
 
-struct SendLds {
-    int32_t sel_expert[kMaxTopk];
-    int32_t sel_count[kMaxTopk];
-    uint64_t sel_row[kMaxTopk];    // where selection k's payload goes (0: nowhere)
-    uint64_t sel_scale[kMaxTopk];  // where its scales go
+struct alignas(16) SendLds {
+    int32_t wave_count[kMaxTopk][kSendMaxWaves];  // [k][wave]: the wave's earlier entries naming selection k's expert
+    uint64_t sel_row[kMaxTopk];                   // where selection k's payload goes (0: nowhere)
+    uint64_t sel_scale[kMaxTopk];                 // where its scales go
 };
 
 // The per-source counting workgroup of a single-chunk batch.
@@ -269,54 +268,76 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             local = my_expert - dst_rank * (num_experts / a.num_ranks);
             if (direct.packed_x != nullptr && dst_rank == a.rank) {
                 // rows of the ranks below come first in the expert's packed range
-                for (int s = 0; s < a.rank; ++s) {
-                    const int c = a.recv_count[local * a.num_ranks + s];
-                    direct_begin += c < 0 ? 0 : (c > a.max_tokens ? a.max_tokens : c);
+                for (int s0 = 0; s0 < a.rank; s0 += 8) {  // eight loads in flight
+                    int c[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u)
+                        c[u] = s0 + u < a.rank ? a.recv_count[local * a.num_ranks + s0 + u] : 0;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) direct_begin += c[u] < 0 ? 0 : (c[u] > a.max_tokens ? a.max_tokens : c[u]);
                 }
             }
         }
     }
     DEEPEP_PHASE(1);
-    // small batch: the entries before this token, fetched now so that their latency overlaps the
-    // loads above (each thread takes every blockDim-th entry; four cover 2048 entries at 512 threads)
-    constexpr int kSweepAhead = 4;
-    int64_t ahead[kSweepAhead];
-    if (a.num_chunks <= 1) {
-#pragma unroll
-        for (int r = 0; r < kSweepAhead; ++r) {
-            const int i = tid + r * int(blockDim.x);
-            ahead[r] = i < entry0 ? my_topk[i] : -1;
-        }
-    }
     if (a.num_chunks > 1) {  // slots were ranked by ll_route_slots_kernel
         if (tid < num_topk && my_expert >= 0)
             my_slot = reinterpret_cast<const int32_t*>(a.scratch_base + int64_t(b) * a.scratch_stride)[entry0 + tid];
-    } else {  // small batch: rank here, sweeping every earlier entry
-        if (tid < num_topk) {
-            lds.sel_expert[tid] = my_expert;
-            lds.sel_count[tid] = 0;
-        }
-        lds_barrier();
-        DEEPEP_PHASE(2);
+    } else {
+        // Small batch: rank here.  Each thread takes every blockDim-th entry before this token (four of
+        // them fetched up front, so their latency overlaps the loads above); each wave counts, per
+        // selection, how many of its entries name that selection's expert (a ballot and a popcount,
+        // against the token's own entries read as wave-uniform values) and leaves the counts in LDS.
+        constexpr int kSweepAhead = 4;
+        int ahead[kSweepAhead];  // -1: no entry
 #pragma unroll
         for (int r = 0; r < kSweepAhead; ++r) {
-            const int64_t v = ahead[r];
-            if (v < 0 || v >= num_experts) continue;
-            for (int k = 0; k < num_topk; ++k)
-                if (int(v) == lds.sel_expert[k]) atomicAdd(&lds.sel_count[k], 1);
+            const int i = tid + r * int(blockDim.x);
+            const int64_t v = i < entry0 ? my_topk[i] : -1;
+            ahead[r] = v >= 0 && v < num_experts ? int(v) : -1;
         }
-        for (int i = tid + kSweepAhead * int(blockDim.x); i < entry0; i += blockDim.x) {
-            const int64_t v = my_topk[i];
-            if (v < 0 || v >= num_experts) continue;
-            for (int k = 0; k < num_topk; ++k)
-                if (int(v) == lds.sel_expert[k]) atomicAdd(&lds.sel_count[k], 1);
+        // lane k of every wave holds the token's selection k (-2: none, matches no entry)
+        int sel = -2;
+        if (lane < num_topk) {
+            const int64_t v = my_topk[entry0 + lane];
+            if (v >= 0 && v < num_experts) sel = int(v);
         }
+        const int w = wave_in_block();
+        int my_count = 0;  // lane k: this wave's entries naming selection k's expert
+        for (int k = 0; k < num_topk; ++k) {
+            const int e = __builtin_amdgcn_readlane(sel, k);
+            int count = 0;
+#pragma unroll
+            for (int r = 0; r < kSweepAhead; ++r) count += __popcll(__ballot(ahead[r] == e));
+            if (lane == k) my_count = count;
+        }
+        for (int base = kSweepAhead * int(blockDim.x); base < entry0; base += blockDim.x) {
+            const int64_t v = base + tid < entry0 ? my_topk[base + tid] : -1;
+            const int e32 = v >= 0 && v < num_experts ? int(v) : -1;
+            for (int k = 0; k < num_topk; ++k) {
+                const int count = __popcll(__ballot(e32 == __builtin_amdgcn_readlane(sel, k)));
+                if (lane == k) my_count += count;
+            }
+        }
+        if (lane < num_topk) lds.wave_count[lane][w] = my_count;
         lds_barrier();
         DEEPEP_PHASE(3);
-        if (tid < num_topk && my_expert >= 0) {
-            my_slot = lds.sel_count[tid];
-            for (int k2 = 0; k2 < tid; ++k2)  // the same expert named earlier in this token
-                if (lds.sel_expert[k2] == my_expert) my_slot += 1;
+        if (tid < kWave) {  // wave 0: lane k finishes selection k
+            const int waves = int(blockDim.x) >> 6;
+            int total = 0;
+            if (tid < num_topk) {  // one wide read of the row; entries of absent waves are never summed
+                static_assert(kSendMaxWaves == 16, "four 16-byte LDS reads");
+                u32x4 c[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) c[q] = reinterpret_cast<const u32x4*>(lds.wave_count[tid])[q];
+#pragma unroll
+                for (int w2 = 0; w2 < kSendMaxWaves; ++w2) total += w2 < waves ? int(c[w2 >> 2][w2 & 3]) : 0;
+            }
+            for (int k2 = 0; k2 < num_topk; ++k2) {  // the same expert named earlier in this token
+                const int other = __builtin_amdgcn_readlane(my_expert, k2);
+                if (k2 < tid && other == my_expert) total += 1;
+            }
+            if (tid < num_topk && my_expert >= 0) my_slot = total;
         }
     }
     if (tid < num_topk) {
@@ -359,17 +380,26 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
     if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
     const int64_t lane_off = int64_t(piece) * 1024 + lane * 16;
     DEEPEP_PHASE(5);
+    // lane k reads selection k's destinations once; the loop takes them back as wave-uniform values
+    uint64_t my_row = 0, my_scale_row = 0;
+    if (lane < num_topk) {
+        my_row = lds.sel_row[lane];
+        my_scale_row = lds.sel_scale[lane];
+    }
     for (int k = part; k < num_topk; k += split) {
-        uint8_t* row = reinterpret_cast<uint8_t*>(wave_uniform_u64(lds.sel_row[k]));
+        uint8_t* row = reinterpret_cast<uint8_t*>(
+            (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_row >> 32), k))) << 32) |
+            uint32_t(__builtin_amdgcn_readlane(int(uint32_t(my_row)), k)));
         if (row == nullptr) continue;
-        if (lane_live) *reinterpret_cast<u32x4*>(row + lane_off) = payload;
+        if (lane_live) store_global(row + lane_off, payload);
         if constexpr (kFmt != kRowBF16) {
-            uint8_t* scale_row = reinterpret_cast<uint8_t*>(wave_uniform_u64(lds.sel_scale[k]));
+            uint8_t* scale_row = reinterpret_cast<uint8_t*>(
+                (uint64_t(uint32_t(__builtin_amdgcn_readlane(int(my_scale_row >> 32), k))) << 32) |
+                uint32_t(__builtin_amdgcn_readlane(int(uint32_t(my_scale_row)), k)));
             if constexpr (kFmt == kRowFP8UE8M0) {
-                if (lane_live && (lane & 7) == 0) scale_row[group] = uint8_t(scale_bits >> 23);
+                if (lane_live && (lane & 7) == 0) store_global_byte(scale_row + group, uint8_t(scale_bits >> 23));
             } else {
-                if (lane_live && (lane & 7) == 0)
-                    *reinterpret_cast<uint32_t*>(scale_row + int64_t(group) * 4) = scale_bits;
+                if (lane_live && (lane & 7) == 0) store_global(scale_row + int64_t(group) * 4, scale_bits);
             }
         }
     }
@@ -441,19 +471,41 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
     }
     int32_t* own_cnt = lds + num_segments + 1;
     if (recount_own) {  // rows from this rank itself: recount them from its own indices
+        const int64_t first = int64_t(own_rank) * a.num_local_experts;
+        constexpr int kAhead = 4;  // four loads in flight per thread: 2048 entries at 512 threads
+        int64_t ahead[kAhead];
+#pragma unroll
+        for (int r = 0; r < kAhead; ++r) {
+            const int i = tid + r * threads;
+            ahead[r] = i < own_entries ? own_topk[i] - first : -1;
+        }
         for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
         lds_barrier();
-        const int64_t first = int64_t(own_rank) * a.num_local_experts;
-        for (int i = tid; i < own_entries; i += threads) {
+#pragma unroll
+        for (int r = 0; r < kAhead; ++r)
+            if (ahead[r] >= 0 && ahead[r] < a.num_local_experts) atomicAdd(&own_cnt[int(ahead[r])], 1);
+        for (int i = tid + kAhead * threads; i < own_entries; i += threads) {
             const int64_t v = own_topk[i] - first;
             if (v >= 0 && v < a.num_local_experts) atomicAdd(&own_cnt[int(v)], 1);
         }
         lds_barrier();
+        // whatever recv_count holds for the own segments (le * R + own_rank) is stale
+        if (a.num_local_experts <= 64) {  // few own segments: visit them, no division per table entry
+            for (int le = 0; le < a.num_local_experts; ++le) {
+                const int s = le * num_ranks + own_rank;
+                if (s / kPer != lane) continue;
+                const int c = clamp_count(own_cnt[le], max_tokens);
 #pragma unroll
-        for (int u = 0; u < kPer; ++u) {  // whatever recv_count holds for the own segments is stale
-            const int s = lane * kPer + u;
-            if (s < num_segments && s % num_ranks == own_rank)
-                seg_table.cnt[u] = clamp_count(own_cnt[s / num_ranks], max_tokens);
+                for (int u = 0; u < kPer; ++u)
+                    if (s % kPer == u) seg_table.cnt[u] = c;
+            }
+        } else {
+#pragma unroll
+            for (int u = 0; u < kPer; ++u) {
+                const int s = lane * kPer + u;
+                if (s < num_segments && s % num_ranks == own_rank)
+                    seg_table.cnt[u] = clamp_count(own_cnt[s / num_ranks], max_tokens);
+            }
         }
     }
 
@@ -502,7 +554,7 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
         int v_begin, v_end;
         row_part_range(num_vec, parts, part, v_begin, v_end);
         DEEPEP_PHASE(2);
-        wave_copy_vec16(src, a.packed_x + out_row * data_bytes, v_begin, v_end, lane);
+        wave_copy_vec16<4>(src, a.packed_x + out_row * data_bytes, v_begin, v_end, lane);
         DEEPEP_PHASE(3);
         if (part != parts - 1) continue;  // the last part is the shortest: it also carries scales and source index
         if (a.packed_scales != nullptr && scale_bytes > 0) {
@@ -583,6 +635,14 @@ static int send_split_override() {
     return v;
 }
 
+static int send_waves_override() {
+    static const int v = [] {
+        const char* s = getenv("DEEPEP_SEND_WAVES");
+        return s != nullptr ? atoi(s) : 0;
+    }();
+    return v;
+}
+
 static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_t* src_ranks, int num_src,
                             int num_tokens, int hidden, int num_topk, int num_experts, int num_ranks, int rank,
                             int max_tokens, int row_format, void* recv_staging, int32_t* recv_count,
@@ -609,12 +669,19 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     // A small batch cannot fill 1024 SIMDs with one wave per row piece: give a share of the
     // K stores of each piece to a second wave.
     int split_log2 = int64_t(num_src) * num_tokens * pieces < 4096 && num_topk > 1 ? 1 : 0;
+    // In the single launch the receive workgroups share the chip: whole tokens per workgroup, and
+    // workgroups small enough that two fit a compute unit.
+    if (fused_recv != nullptr) split_log2 = 0;
     if (send_split_override() == 1) split_log2 = 0;
     if (send_split_override() == 2) split_log2 = 1;
     if (send_split_override() == 4) split_log2 = 2;
     const int items = pieces << split_log2;  // waves per token
-    const int waves = items < kSendMaxWaves ? items : kSendMaxWaves;
+    int max_waves = kSendMaxWaves;
+    if (send_waves_override() >= 1 && send_waves_override() <= kSendMaxWaves) max_waves = send_waves_override();
+    if (fused_recv != nullptr && max_waves > 8) max_waves = 8;
+    int waves = items < max_waves ? items : max_waves;
     const int blocks_per_token = (items + waves - 1) / waves;
+    if (fused_recv != nullptr && waves < 4) waves = 4;  // the receive workgroups want a few waves each
     EP_HOST_ASSERT(num_tokens < 65535 && num_src <= 65535);
     // floor(e / E_l) == umulhi(e, ceil(2^32 / E_l)) for every e below 2^16.
     const uint32_t experts_per_rank = uint32_t(num_experts / num_ranks);
