@@ -266,23 +266,33 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             dst_rank = a.rank_of_expert_magic != 0 ? int(__umulhi(uint32_t(my_expert), a.rank_of_expert_magic))
                                                    : my_expert;
             local = my_expert - dst_rank * (num_experts / a.num_ranks);
-            if (direct.packed_x != nullptr && dst_rank == a.rank) {
-                // rows of the ranks below come first in the expert's packed range
-                for (int s0 = 0; s0 < a.rank; s0 += 8) {  // eight loads in flight
-                    int c[8];
-#pragma unroll
-                    for (int u = 0; u < 8; ++u)
-                        c[u] = s0 + u < a.rank ? a.recv_count[local * a.num_ranks + s0 + u] : 0;
-#pragma unroll
-                    for (int u = 0; u < 8; ++u) direct_begin += c[u] < 0 ? 0 : (c[u] > a.max_tokens ? a.max_tokens : c[u]);
+        }
+    }
+    if (direct.packed_x != nullptr && tid < kWave) {
+        // Rows for this rank's own experts go straight to the packed tensors, behind the rows of all
+        // the peers: for each such selection wave 0 adds up the peers' counts of that expert.
+        uint64_t to_own = __ballot(my_expert >= 0 && dst_rank == a.rank);
+        while (to_own != 0) {
+            const int k = __builtin_ctzll(to_own);
+            to_own &= to_own - 1;
+            const int le = __builtin_amdgcn_readlane(local, k);
+            int part = 0;
+            for (int s = lane; s < a.num_ranks; s += kWave)
+                if (s != a.rank) {
+                    const int c = a.recv_count[le * a.num_ranks + s];
+                    part += c < 0 ? 0 : (c > a.max_tokens ? a.max_tokens : c);
                 }
-            }
+            const int sum = __builtin_amdgcn_readlane(wave_inclusive_sum(part), kWave - 1);
+            if (lane == k) direct_begin = sum;
         }
     }
     DEEPEP_PHASE(1);
+    u32x4 payload = lo;  // quantised below, while the workgroup's bookkeeping is in flight
+    uint32_t scale_bits = 0;
     if (a.num_chunks > 1) {  // slots were ranked by ll_route_slots_kernel
         if (tid < num_topk && my_expert >= 0)
             my_slot = reinterpret_cast<const int32_t*>(a.scratch_base + int64_t(b) * a.scratch_stride)[entry0 + tid];
+        if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
     } else {
         // Small batch: rank here.  Each thread takes every blockDim-th entry before this token (four of
         // them fetched up front, so their latency overlaps the loads above); each wave counts, per
@@ -320,6 +330,7 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             }
         }
         if (lane < num_topk) lds.wave_count[lane][w] = my_count;
+        if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
         lds_barrier();
         DEEPEP_PHASE(3);
         if (tid < kWave) {  // wave 0: lane k finishes selection k
@@ -374,10 +385,7 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
     DEEPEP_PHASE(4);
     if (!wave_live) return;
 
-    // ---- quantise, then one store per selection ---------------------------
-    u32x4 payload = lo;
-    uint32_t scale_bits = 0;
-    if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
+    // ---- one store per selection ----------------------------------------
     const int64_t lane_off = int64_t(piece) * 1024 + lane * 16;
     DEEPEP_PHASE(5);
     // lane k reads selection k's destinations once; the loop takes them back as wave-uniform values
@@ -448,8 +456,13 @@ __device__ __forceinline__ int clamp_count(int c, int max_tokens) {
 }
 
 // Workgroups [0, num_copy_blocks) copy rows; workgroup num_copy_blocks writes layout_range,
-// packed_count and stats and copies nothing, so the copying waves never wait for a barrier:
-// each builds the segment prefix in its own registers (WaveSegments) from the E counts.
+// packed_count and stats and copies nothing.  A copying wave builds the segment prefix in its own
+// registers (WaveSegments) from the E counts: no LDS, no barrier.
+//
+// With own_topk (single-launch dispatch) this rank's own rows are not in the staging area: the
+// send workgroups of the same launch put them straight into the packed tensors, behind the rows
+// of all the peers.  The copying waves then see the peers' segments only and need nothing from
+// the own routing; the metadata workgroup recounts the own rows from own_topk for layout_range.
 // lds: [num_segments + 1 + num_local_experts] ints; wave_totals: 16 ints.
 template <int kPer>
 __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int num_copy_blocks,
@@ -459,7 +472,43 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
     const int threads = blockDim.x, waves = threads >> 6;
     const int num_ranks = a.num_ranks, max_tokens = a.max_tokens;
     const int num_segments = a.num_local_experts * num_ranks;
-    const bool recount_own = own_topk != nullptr;
+    const bool own_last = own_topk != nullptr;
+
+    if (block == num_copy_blocks) {  // the metadata workgroup
+        int32_t* own_cnt = lds + num_segments + 1;
+        if (own_last) {
+            for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
+            lds_barrier();
+            const int64_t first = int64_t(own_rank) * a.num_local_experts;
+            for (int i = tid; i < own_entries; i += threads) {
+                const int64_t v = own_topk[i] - first;
+                if (v >= 0 && v < a.num_local_experts) atomicAdd(&own_cnt[int(v)], 1);
+            }
+        }
+        for (int s = tid; s < num_segments; s += threads) {
+            const bool own = own_last && s % num_ranks == own_rank;
+            lds[s] = own ? 0 : clamp_count(a.recv_count[s], max_tokens);
+        }
+        lds_barrier();
+        block_exclusive_scan(lds, num_segments, wave_totals);
+        for (int s = tid; s < num_segments; s += threads) {
+            const int le = s / num_ranks;
+            int64_t cnt = lds[s + 1] - lds[s];
+            int64_t begin = lds[s] - lds[le * num_ranks];
+            if (own_last && s - le * num_ranks == own_rank) {
+                cnt = clamp_count(own_cnt[le], max_tokens);
+                begin = lds[(le + 1) * num_ranks] - lds[le * num_ranks];  // behind all the peers
+            }
+            a.layout_range[s] = cnt > 0 ? ((begin << 32) | cnt) : 0;
+        }
+        for (int le = tid; le < a.num_local_experts; le += threads) {
+            int c = lds[(le + 1) * num_ranks] - lds[le * num_ranks];
+            if (own_last) c += clamp_count(own_cnt[le], max_tokens);
+            a.packed_count[le] = c;
+            if (a.stats != nullptr) a.stats[le] += c;
+        }
+        return;
+    }
 
     WaveSegments<kPer> seg_table;
     DEEPEP_PHASE(0);
@@ -469,69 +518,17 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
         seg_table.aux[u] = 0;
         seg_table.cnt[u] = clamp_count(seg_table.cnt[u], max_tokens);
     }
-    int32_t* own_cnt = lds + num_segments + 1;
-    if (recount_own) {  // rows from this rank itself: recount them from its own indices
-        const int64_t first = int64_t(own_rank) * a.num_local_experts;
-        constexpr int kAhead = 4;  // four loads in flight per thread: 2048 entries at 512 threads
-        int64_t ahead[kAhead];
+    if (own_last) {  // whatever recv_count holds for the own segments (le * R + own_rank) is stale
+        int source = (lane * kPer) % num_ranks;  // source rank of this lane's first segment
 #pragma unroll
-        for (int r = 0; r < kAhead; ++r) {
-            const int i = tid + r * threads;
-            ahead[r] = i < own_entries ? own_topk[i] - first : -1;
-        }
-        for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
-        lds_barrier();
-#pragma unroll
-        for (int r = 0; r < kAhead; ++r)
-            if (ahead[r] >= 0 && ahead[r] < a.num_local_experts) atomicAdd(&own_cnt[int(ahead[r])], 1);
-        for (int i = tid + kAhead * threads; i < own_entries; i += threads) {
-            const int64_t v = own_topk[i] - first;
-            if (v >= 0 && v < a.num_local_experts) atomicAdd(&own_cnt[int(v)], 1);
-        }
-        lds_barrier();
-        // whatever recv_count holds for the own segments (le * R + own_rank) is stale
-        if (a.num_local_experts <= 64) {  // few own segments: visit them, no division per table entry
-            for (int le = 0; le < a.num_local_experts; ++le) {
-                const int s = le * num_ranks + own_rank;
-                if (s / kPer != lane) continue;
-                const int c = clamp_count(own_cnt[le], max_tokens);
-#pragma unroll
-                for (int u = 0; u < kPer; ++u)
-                    if (s % kPer == u) seg_table.cnt[u] = c;
-            }
-        } else {
-#pragma unroll
-            for (int u = 0; u < kPer; ++u) {
-                const int s = lane * kPer + u;
-                if (s < num_segments && s % num_ranks == own_rank)
-                    seg_table.cnt[u] = clamp_count(own_cnt[s / num_ranks], max_tokens);
-            }
+        for (int u = 0; u < kPer; ++u) {
+            if (source == own_rank) seg_table.cnt[u] = 0;
+            source = source + 1 == num_ranks ? 0 : source + 1;
         }
     }
-
-    if (block == num_copy_blocks) {  // the metadata workgroup
-        for (int s = tid; s < num_segments; s += threads) {
-            const bool own = recount_own && s % num_ranks == own_rank;
-            lds[s] = clamp_count(own ? own_cnt[s / num_ranks] : a.recv_count[s], max_tokens);
-        }
-        lds_barrier();
-        block_exclusive_scan(lds, num_segments, wave_totals);
-        for (int s = tid; s < num_segments; s += threads) {
-            const int le = s / num_ranks;
-            const int64_t cnt = lds[s + 1] - lds[s];
-            const int64_t begin = lds[s] - lds[le * num_ranks];
-            a.layout_range[s] = cnt > 0 ? ((begin << 32) | cnt) : 0;
-        }
-        for (int le = tid; le < a.num_local_experts; le += threads) {
-            const int c = lds[(le + 1) * num_ranks] - lds[le * num_ranks];
-            a.packed_count[le] = c;
-            if (a.stats != nullptr) a.stats[le] += c;
-        }
-        return;
-    }
-
     wave_segments_finish(seg_table);
     DEEPEP_PHASE(1);
+
     const int64_t data_bytes = row_data_bytes(a.hidden, a.fmt);
     const int64_t data_pad = align16(data_bytes);
     const int64_t scale_bytes = row_scale_bytes(a.hidden, a.fmt);
@@ -546,7 +543,6 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
         int seg_first, unused;
         const int seg = wave_segments_find(seg_table, row, seg_first, unused);
         const int le = seg / num_ranks;
-        if (recount_own && seg - le * num_ranks == own_rank) continue;  // placed by the send workgroups
         const int j = row - seg_first;
         const int slot = row - wave_segments_prefix(seg_table, le * num_ranks);
         const uint8_t* src = a.recv_staging + (int64_t(seg) * max_tokens + j) * stride;
@@ -586,9 +582,12 @@ __global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a) {
 // workgroups, the counting workgroup and the receive workgroups of the two
 // kernels above in one grid.  No workgroup waits on another: the receive
 // workgroups copy only the peers' rows (already in the staging area when the
-// launch starts) and recount the own segments from topk_idx; the send
-// workgroups place the rank's rows for its own experts at their final packed
-// position, which they find from the peers' counts.
+// launch starts); the send workgroups place the rank's rows for its own
+// experts at their final packed position, behind the rows of all the peers,
+// which they find from the peers' counts.  Inside an expert's packed range
+// the order of the source ranks is therefore "peers ascending, then this
+// rank"; layout_range says so (the reference assigns the ranges in arrival
+// order, csrc/kernels/efa_kernels.cu:1017-1052 being its deterministic variant).
 // (The reference's dispatch is one kernel with a send and a receive phase as
 // well: csrc/kernels/coop_dispatch_send.cuh:304, coop_dispatch_recv.cuh:42.)
 // ---------------------------------------------------------------------

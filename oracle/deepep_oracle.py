@@ -219,8 +219,14 @@ def route(topk_idx: torch.Tensor, num_experts: int, max_tokens: int):
     return send_count, pair_slot.view(t, k)
 
 
-def ll_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_tokens: int, fmt: int = ROW_FP8):
+def ll_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_tokens: int, fmt: int = ROW_FP8,
+                own_last: bool = False):
     """What rank `rank` receives when every rank of the world dispatches.
+
+    own_last: inside each expert's packed range the source ranks come in ascending order with
+    `rank`'s own segment moved behind all the others (the order of the single-launch dispatch);
+    otherwise plain ascending order.  The reference fixes no order across source ranks (its live
+    kernel claims ranges with atomics); layout_range carries whichever is used.
 
     all_x: list of R tensors [T_s, H] bf16; all_topk_idx: list of R tensors [T_s, K] int64.
     Follows deep_ep/buffer.py:1816-1887,2266-2457 (nccl-fallback branch) with
@@ -247,9 +253,10 @@ def ll_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_tokens: in
         _, pair_slot = route(all_topk_idx[s], num_experts, max_tokens)
         data, scales = quantise_rows(all_x[s], fmt)
         per_src.append((pair_slot, data, scales))
+    order = [s for s in range(r) if s != rank] + [rank] if own_last else list(range(r))
     for le in range(epr):
         e = rank * epr + le
-        for s in range(r):
+        for s in order:
             pair_slot, data, scales = per_src[s]
             sel = (all_topk_idx[s] == e) & (pair_slot >= 0)
             tok, kk = torch.nonzero(sel, as_tuple=True)

@@ -55,6 +55,12 @@ def make_world(r, t, h, k, e, seed, drop=10, recipe="randn"):
 ONE_CALL = pytest.mark.parametrize("one_call", [False, True], ids=["two_calls", "one_call"])
 
 
+def own_last(one_call, t, k, e, m):
+    """The one-call dispatch runs as a single launch for small batches and then places this rank's own
+    rows behind the peers' inside each expert's range; otherwise source ranks come in ascending order."""
+    return one_call and t * k <= 2048 and e * m <= (1 << 18)
+
+
 def poison_outputs(st):
     """Fresh tensors may reuse memory that an earlier test left holding the right answer."""
     st.packed_recv_x.view(torch.uint8).fill_(0xEE)
@@ -130,7 +136,7 @@ def check_dispatch(st, want, fmt):
 def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
     x_all, topk_all, _ = make_world(r, t, h, k, e, seed=r * 100 + t, drop=min(5, t))
     st, _ = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt, one_call=one_call)
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt, own_last=own_last(one_call, t, k, e, t))
     check_dispatch(st, want, fmt)
     send_count, pair_slot = O.route(topk_all[rank], e, t)
     assert torch.equal(st.send_count.cpu(), send_count)
@@ -243,7 +249,7 @@ def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e, one_ca
     # oracle: which row does each of this rank's pairs get back?
     topk, w = topk_all[rank], w_all[rank]
     _, pair_slot = O.route(topk, e, t)
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8, own_last=own_last(one_call, t, k, e, t))
     keys_local, keys_remote = [], []
     pair_rows = torch.zeros((t, k, h), dtype=torch.bfloat16)
     live = pair_slot >= 0
@@ -296,7 +302,7 @@ def test_ll_config_full_size(rt, one_call):
     assert torch.equal(world.topk_idx_all.cpu(), topk_all)
     x_all = O.synth_bf16_rows(np.arange(r * t, dtype=np.uint32), h, 2024).view(r, t, h)
     assert torch.equal(world.x_all.cpu().view(torch.int16), x_all.view(torch.int16))
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8, own_last=own_last(one_call, t, k, e, t))
     check_dispatch(st, want, O.ROW_FP8)
     assert int(st.packed_recv_count.sum()) == int(((topk_all // (e // r)) == rank).sum())
 
@@ -315,7 +321,7 @@ def test_skewed_routing_roundtrip(rt, one_call):
     x_all = O.synth_bf16_rows(np.arange(r * t, dtype=np.uint32), h, 99, outlier_period=100).view(r, t, h)
     assert torch.equal(world.topk_idx_all.cpu(), topk_all)
     assert torch.equal(world.x_all.cpu().view(torch.int16), x_all.view(torch.int16))
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8, own_last=own_last(one_call, t, k, e, t))
     check_dispatch(st, want, O.ROW_FP8)
     assert int(st.packed_recv_count[0]) > r * t // 2, "the hottest expert should fill over half its slots"
     # round trip with identity experts: combined == x * sum(w) within FP8 error
@@ -364,6 +370,6 @@ def test_empty_batch(rt, one_call):
     run_dispatch(st, world, x_all[rank, :0].cuda(), topk_all[rank, :0].cuda(), one_call=one_call)
     xs, tks = list(x_all), list(topk_all)
     xs[rank], tks[rank] = xs[rank][:0], tks[rank][:0]
-    want = O.ll_dispatch(xs, tks, rank, e, t, O.ROW_FP8)
+    want = O.ll_dispatch(xs, tks, rank, e, t, O.ROW_FP8, own_last=own_last(one_call, 0, k, e, t))
     check_dispatch(st, want, O.ROW_FP8)
     assert (st.send_count == 0).all()

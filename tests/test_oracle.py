@@ -221,6 +221,31 @@ def test_vectorised_dispatch_equals_serial_restatement(fmt):
             assert torch.equal(a[key], b[key]), (rank, key)
 
 
+def test_own_last_order_is_the_ascending_order_with_one_segment_moved():
+    """own_last only permutes whole segments: every (expert, source) segment keeps its rows and their order,
+    the own segment starts where the peers' rows end, the peers keep ascending order among themselves."""
+    xs, tk = _world(4, 8, 512, 3, 16, seed=5, drop=4)
+    for rank in range(4):
+        a = O.ll_dispatch(xs, tk, rank, 16, 8, O.ROW_FP8)
+        b = O.ll_dispatch(xs, tk, rank, 16, 8, O.ROW_FP8, own_last=True)
+        assert torch.equal(a["packed_recv_count"], b["packed_recv_count"])
+        for le in range(4):
+            la, lb = a["packed_recv_layout_range"][le], b["packed_recv_layout_range"][le]
+            assert torch.equal(la & 0xFFFFFFFF, lb & 0xFFFFFFFF)
+            cursor = 0
+            for s in [x for x in range(4) if x != rank] + [rank]:
+                cnt = int(lb[s] & 0xFFFFFFFF)
+                if cnt == 0:
+                    assert int(lb[s]) == 0
+                    continue
+                assert int(lb[s] >> 32) == cursor
+                ba = int(la[s] >> 32)
+                for key in ("packed_recv_x", "packed_recv_scales", "packed_recv_src_info"):
+                    assert torch.equal(a[key][le, ba:ba + cnt], b[key][le, cursor:cursor + cnt]), (rank, le, s, key)
+                cursor += cnt
+            assert cursor == int(b["packed_recv_count"][le])
+
+
 def test_dispatch_invariants_of_reference_test():
     # tests/test_low_latency.py:59-60,119-147: x = rank-128 with the token index in the last 128 columns.
     r, t, h, k, e = 4, 16, 256, 4, 16
