@@ -254,7 +254,7 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
 /* deepep_ll_dispatch_send followed by deepep_ll_dispatch_recv, for a caller
  * whose peers' rows and counts are already in recv_staging / recv_count when
  * the call is made (the reference's dispatch is one call too:
- * Buffer::low_latency_dispatch, csrc/deep_ep.cpp:1622-1799; its kernel has a
+ * Buffer::low_latency_dispatch, csrc/deep_ep.cpp:1658-1796; its kernel has a
  * send and a receive phase, csrc/kernels/coop_dispatch_send.cuh:304,
  * coop_dispatch_recv.cuh:42).  Arguments are those of the two calls; outputs
  * are identical, with one difference: for small batches
@@ -280,7 +280,7 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx,
 /* deepep_ll_combine_send followed by deepep_ll_combine_recv, for a caller
  * whose remote experts' answers are already in combine_staging when the call
  * is made (the reference: Buffer::low_latency_combine,
- * csrc/deep_ep.cpp:1801-1939; kernel phases csrc/kernels/coop_combine_send.cuh:37,
+ * csrc/deep_ep.cpp:1798-1920; kernel phases csrc/kernels/coop_combine_send.cuh:37,
  * coop_combine_recv.cuh:72).  `out` is identical to the two calls'.  For
  * num_experts * M <= 2^18 both phases run as one kernel launch, and then the
  * answers of this rank's own experts are read from x directly — the own
