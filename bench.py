@@ -142,6 +142,32 @@ def bench_pack(torch, _capi, lib, loopback, args):
     def cast():
         _capi.check(lib.deepep_per_token_cast_to_fp8(_capi.ptr(x), t, h, 1, _capi.ptr(q), _capi.ptr(sc), stream))
 
+    # the steps either side of the pack: top-k remap of the send rows, source metadata of the rows
+    # received (here: as many as were sent), and the per-token reduce of the rows that come back
+    # (here: the packed rows themselves, i.e. every rank returns what it was sent)
+    weights = torch.rand((t, k), device="cuda")
+    remap_e = torch.empty((s, k), dtype=torch.int64, device="cuda")
+    remap_w = torch.empty((s, k), dtype=torch.float32, device="cuda")
+    meta = torch.empty((s, 8), dtype=torch.uint8, device="cuda")
+    comb_x = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    comb_w = torch.empty((t, k), dtype=torch.float32, device="cuda")
+    ws3 = torch.empty(max(256, lib.deepep_combine_reduce_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
+    pack_bf16()
+
+    def remap():
+        _capi.check(lib.deepep_topk_remap(_capi.ptr(topk), _capi.ptr(weights), _capi.ptr(ids), _capi.ptr(cumsum), t, k, r,
+                                          e // r, s, _capi.ptr(remap_e), _capi.ptr(remap_w), stream))
+
+    def src_meta():
+        _capi.check(lib.deepep_build_recv_src_meta(_capi.ptr(cumsum), r, 8, s, _capi.ptr(meta), stream))
+
+    remap()
+
+    def reduce():
+        _capi.check(lib.deepep_combine_reduce(_capi.ptr(out16), _capi.ptr(remap_w), _capi.ptr(ids), _capi.ptr(cumsum),
+                                              _capi.ptr(is_in), None, None, t, h, k, r, s, _capi.ptr(comb_x),
+                                              _capi.ptr(comb_w), _capi.ptr(ws3), ws3.numel(), stream))
+
     n = max(10, args.steps // 4)
     res = {"workload": "4096 tokens x 7168 bf16, top-8 of 256 experts, 8 ranks x 32 experts", "rows_packed": s}
     for name, fn, nbytes in (("layout", layout, t * k * 8 + t * r + 4 * (r + e)),
@@ -149,7 +175,10 @@ def bench_pack(torch, _capi, lib, loopback, args):
                              ("channel_prefix", prefix, t * r + r * 10 * 4),
                              ("cast_fp8", cast, t * 2 * h + t * h + t * (h // 32)),
                              ("pack_bf16", pack_bf16, s * 2 * h * 2 + s * 8),
-                             ("pack_fp8", pack_fp8, s * (h + h // 32) * 2 + s * 8)):
+                             ("pack_fp8", pack_fp8, s * (h + h // 32) * 2 + s * 8),
+                             ("topk_remap", remap, s * 8 + s * k * 12 * 2),
+                             ("recv_src_meta", src_meta, s * 8),
+                             ("combine_reduce", reduce, s * 2 * h + s * k * 4 + s * 12 + t * r + t * 2 * h + t * k * 4)):
         us = time_calls(torch, fn, n)
         res[name] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
                      "frac_of_8TBps": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}

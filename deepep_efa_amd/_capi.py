@@ -37,6 +37,10 @@ PROTOTYPES = {
                                 _VP, _I64, _VP, _SZ, _VP, _SZ, _VP]),
     "deepep_ll_combine": (_I, [_VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _I64, _VP, _SZ,
                                _VP]),
+    "deepep_topk_remap": (_I, [_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP]),
+    "deepep_build_recv_src_meta": (_I, [_VP, _I, _I, _I64, _VP, _VP]),
+    "deepep_combine_reduce_workspace_bytes": (_SZ, [_I, _I]),
+    "deepep_combine_reduce": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP, _SZ, _VP]),
     "deepep_synth_topk_idx": (_I, [_VP, _VP, _I, _I, _I, _I, _U32, _VP, _VP]),
     "deepep_synth_bf16_rows": (_I, [_VP, _I64, _I, _I64, _VP, _U32, _U32, _I, _VP]),
     "deepep_loopback_dispatch_from_peers": (_I, [_VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _SZ,

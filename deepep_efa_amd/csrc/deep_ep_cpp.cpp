@@ -674,6 +674,85 @@ static torch::Tensor channel_prefix_matrix(const torch::Tensor& is_token_in_rank
     return cpm;
 }
 
+// reference: csrc/kernels/efa_kernels.cu:1653-1691 (same arguments, same outputs)
+static std::tuple<torch::Tensor, torch::Tensor> topk_remap(const torch::Tensor& topk_idx, const torch::Tensor& topk_weights,
+                                                           const torch::Tensor& sorted_token_ids,
+                                                           const torch::Tensor& send_cumsum, int64_t total_send,
+                                                           int num_ranks, int num_local_experts) {
+    EP_HOST_ASSERT(topk_idx.dim() == 2);
+    EP_HOST_ASSERT(topk_idx.is_contiguous() && topk_idx.is_cuda());
+    EP_HOST_ASSERT(topk_weights.dim() == 2);
+    EP_HOST_ASSERT(topk_weights.is_contiguous() && topk_weights.is_cuda());
+    EP_HOST_ASSERT(topk_idx.scalar_type() == torch::kInt64 and topk_weights.scalar_type() == torch::kFloat32);
+    EP_HOST_ASSERT(topk_weights.size(0) == topk_idx.size(0) and topk_weights.size(1) == topk_idx.size(1));
+    EP_HOST_ASSERT(sorted_token_ids.scalar_type() == torch::kInt64 and sorted_token_ids.is_contiguous());
+    EP_HOST_ASSERT(send_cumsum.scalar_type() == torch::kInt64 and send_cumsum.is_contiguous());
+    EP_HOST_ASSERT(send_cumsum.numel() == num_ranks + 1);
+    EP_HOST_ASSERT(total_send >= 0 and total_send <= sorted_token_ids.numel());
+    const int num_topk = static_cast<int>(topk_idx.size(1));
+    auto remapped_topk = torch::empty({total_send, num_topk}, topk_idx.options());
+    auto remapped_weights = torch::empty({total_send, num_topk}, topk_weights.options());
+    abi_check(deepep_topk_remap(topk_idx.data_ptr<int64_t>(), topk_weights.data_ptr<float>(),
+                                sorted_token_ids.data_ptr<int64_t>(), send_cumsum.data_ptr<int64_t>(),
+                                static_cast<int>(topk_idx.size(0)), num_topk, num_ranks, num_local_experts, total_send,
+                                remapped_topk.data_ptr<int64_t>(), remapped_weights.data_ptr<float>(), current_stream()));
+    return {remapped_topk, remapped_weights};
+}
+
+// reference: csrc/kernels/efa_kernels.cu:1726-1749 (recv_counts is accepted and not needed: the prefix has it)
+static torch::Tensor build_recv_src_meta(const torch::Tensor& recv_counts, const torch::Tensor& recv_cumsum,
+                                         int64_t num_recv_tokens, int num_ranks, int num_local_ranks) {
+    EP_HOST_ASSERT(recv_counts.is_cuda() and recv_cumsum.is_cuda());
+    EP_HOST_ASSERT(recv_cumsum.scalar_type() == torch::kInt64 and recv_cumsum.is_contiguous());
+    EP_HOST_ASSERT(recv_cumsum.numel() == num_ranks + 1 and num_recv_tokens >= 0);
+    auto meta = torch::empty({num_recv_tokens, 8}, torch::dtype(torch::kUInt8).device(recv_cumsum.device()));
+    abi_check(deepep_build_recv_src_meta(recv_cumsum.data_ptr<int64_t>(), num_ranks, num_local_ranks, num_recv_tokens,
+                                         meta.data_ptr<uint8_t>(), current_stream()));
+    return meta;
+}
+
+// reference: deep_ep/buffer.py:1542-1557 — zero_() + index_add_ over the returned rows, then the biases
+static std::tuple<torch::Tensor, std::optional<torch::Tensor>> combine_reduce(
+    const torch::Tensor& recv_x, const std::optional<torch::Tensor>& recv_topk_weights,
+    const torch::Tensor& sorted_token_ids, const torch::Tensor& send_cumsum, const torch::Tensor& is_token_in_rank,
+    const std::optional<torch::Tensor>& bias_0, const std::optional<torch::Tensor>& bias_1) {
+    EP_HOST_ASSERT(recv_x.dim() == 2 and recv_x.is_contiguous() and recv_x.is_cuda());
+    EP_HOST_ASSERT(recv_x.scalar_type() == torch::kBFloat16);
+    EP_HOST_ASSERT(is_token_in_rank.dim() == 2 and is_token_in_rank.is_contiguous());
+    EP_HOST_ASSERT(is_token_in_rank.scalar_type() == torch::kBool);
+    EP_HOST_ASSERT(sorted_token_ids.scalar_type() == torch::kInt64 and sorted_token_ids.is_contiguous());
+    EP_HOST_ASSERT(send_cumsum.scalar_type() == torch::kInt64 and send_cumsum.is_contiguous());
+    const int num_tokens = static_cast<int>(is_token_in_rank.size(0)), num_ranks = static_cast<int>(is_token_in_rank.size(1));
+    const int hidden = static_cast<int>(recv_x.size(1));
+    EP_HOST_ASSERT(send_cumsum.numel() == num_ranks + 1);
+    const int64_t max_rows = std::min<int64_t>(recv_x.size(0), sorted_token_ids.numel());
+    int num_topk = 0;
+    if (recv_topk_weights.has_value()) {
+        EP_HOST_ASSERT(recv_topk_weights->dim() == 2 and recv_topk_weights->is_contiguous());
+        EP_HOST_ASSERT(recv_topk_weights->scalar_type() == torch::kFloat32 and recv_topk_weights->size(0) >= max_rows);
+        num_topk = static_cast<int>(recv_topk_weights->size(1));
+    }
+    for (const auto* b : {&bias_0, &bias_1})
+        if (b->has_value()) {
+            EP_HOST_ASSERT((*b)->dim() == 2 and (*b)->is_contiguous() and (*b)->scalar_type() == torch::kBFloat16);
+            EP_HOST_ASSERT((*b)->size(0) == num_tokens and (*b)->size(1) == hidden);
+        }
+    auto combined_x = torch::empty({num_tokens, hidden}, recv_x.options());
+    std::optional<torch::Tensor> combined_w;
+    if (recv_topk_weights.has_value()) combined_w = torch::empty({num_tokens, num_topk}, recv_topk_weights->options());
+    auto ws = torch::empty({std::max<int64_t>(256, int64_t(deepep_combine_reduce_workspace_bytes(num_tokens, num_ranks)))},
+                           torch::dtype(torch::kUInt8).device(recv_x.device()));
+    abi_check(deepep_combine_reduce(
+        recv_x.data_ptr(), recv_topk_weights.has_value() ? recv_topk_weights->data_ptr<float>() : nullptr,
+        sorted_token_ids.data_ptr<int64_t>(), send_cumsum.data_ptr<int64_t>(),
+        reinterpret_cast<const uint8_t*>(is_token_in_rank.data_ptr<bool>()),
+        bias_0.has_value() ? bias_0->data_ptr() : nullptr, bias_1.has_value() ? bias_1->data_ptr() : nullptr, num_tokens,
+        hidden, num_topk, num_ranks, max_rows, combined_x.data_ptr(),
+        combined_w.has_value() ? combined_w->data_ptr<float>() : nullptr, ws.data_ptr(), size_t(ws.numel()),
+        current_stream()));
+    return {combined_x, combined_w};
+}
+
 // reference: deep_ep/buffer.py:877,917 — send_x = x[sorted_ids], send_scales = scales[sorted_ids]
 static std::tuple<torch::Tensor, std::optional<torch::Tensor>> pack_rows(const torch::Tensor& x,
                                                                          const std::optional<torch::Tensor>& x_scales,
@@ -766,4 +845,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("moe_routing_sort", &deep_ep::moe_routing_sort, "Token ids grouped by destination rank");
     m.def("channel_prefix_matrix", &deep_ep::channel_prefix_matrix, "Per-rank prefix of token counts over channels");
     m.def("pack_rows", &deep_ep::pack_rows, "Gather rows into per-rank contiguous send buffers");
+    m.def("topk_remap", &deep_ep::topk_remap, "Top-k of the send rows in the destination rank's expert numbering");
+    m.def("build_recv_src_meta", &deep_ep::build_recv_src_meta, "Source-rank metadata of the received rows");
+    m.def("combine_reduce", &deep_ep::combine_reduce, "Per-token sum of the rows that came back (normal-mode combine)");
 }

@@ -128,6 +128,56 @@ int deepep_pack_rows(const void* src, const void* scale_src, const int64_t* sort
                      int row_bytes, int scale_row_bytes,
                      void* dst, void* scale_dst, void* stream);
 
+/* Top-k of the rows being sent, in the destination rank's expert numbering:
+ * for send row i (destination rank d, send_cumsum[d] <= i < send_cumsum[d+1])
+ * and selection k, (e - d*E_l, w) if the token's expert e is one of rank d's,
+ * else (-1, 0).  Rows i < min(send_cumsum[R], max_send) are written.
+ *   topk_idx [T, K] int64       topk_weights [T, K] float32
+ *   sorted_token_ids [>= S] int64, send_cumsum [R + 1] int64 (from deepep_moe_routing_sort)
+ *   remapped_topk [max_send, K] int64 (out), remapped_weights [max_send, K] float32 (out)
+ * Replaces topk_remap (csrc/kernels/efa_kernels.cu:339-387,1653-1691; call site
+ * deep_ep/buffer.py:727); the row count stays on the device. */
+int deepep_topk_remap(const int64_t* topk_idx, const float* topk_weights,
+                      const int64_t* sorted_token_ids, const int64_t* send_cumsum,
+                      int num_tokens, int num_topk, int num_ranks, int num_local_experts,
+                      int64_t max_send, int64_t* remapped_topk, float* remapped_weights,
+                      void* stream);
+
+/* Source metadata of the rows received: row i came from rank s with
+ * recv_cumsum[s] <= i < recv_cumsum[s+1]; its 8 bytes are the int32 pair
+ * {s / num_local_ranks, 1 << (s % num_local_ranks)}.  Rows
+ * i < min(recv_cumsum[R], max_recv_tokens) are written.
+ *   recv_cumsum [R + 1] int64     recv_src_meta [max_recv_tokens, 8] bytes (out)
+ * Replaces build_recv_src_meta (csrc/kernels/efa_kernels.cu:448-482,1726-1749;
+ * call site deep_ep/buffer.py:792). */
+int deepep_build_recv_src_meta(const int64_t* recv_cumsum, int num_ranks, int num_local_ranks,
+                               int64_t max_recv_tokens, uint8_t* recv_src_meta, void* stream);
+
+/* Bytes of scratch `deepep_combine_reduce` needs. */
+size_t deepep_combine_reduce_workspace_bytes(int num_tokens, int num_ranks);
+
+/* Normal-mode combine, receive side: the rows that came back, in the order of
+ * the send list (row j of rank r's segment answers token sorted_token_ids[j]),
+ * are added per token:
+ *   combined_x[t,:] = bf16( sum_{r: is_token_in_rank[t,r]} f32(recv_x[row(t,r),:])
+ *                           + bias_0[t,:] + bias_1[t,:] )
+ * in float32, ranks ascending, one rounding; the weights likewise in float32.
+ * Tokens sent nowhere give the biases (or zeros).
+ *   recv_x [>= S, H] bf16          recv_topk_weights [>= S, K] float32 or NULL
+ *   sorted_token_ids, send_cumsum  as used for the dispatch pack
+ *   is_token_in_rank [T, R] bool bytes
+ *   bias_0, bias_1 [T, H] bf16 or NULL
+ *   combined_x [T, H] bf16 (out)   combined_topk_weights [T, K] float32 (out) or NULL
+ *   max_rows bounds the rows of recv_x that may be read.
+ * Replaces the zero_() + index_add_ + bias adds of deep_ep/buffer.py:1542-1557
+ * (which accumulate in bf16 through atomics, in arrival order). */
+int deepep_combine_reduce(const void* recv_x, const float* recv_topk_weights,
+                          const int64_t* sorted_token_ids, const int64_t* send_cumsum,
+                          const uint8_t* is_token_in_rank, const void* bias_0, const void* bias_1,
+                          int num_tokens, int hidden, int num_topk, int num_ranks, int64_t max_rows,
+                          void* combined_x, float* combined_topk_weights,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------ */
 /* FP8 cast                                                           */
 /* ------------------------------------------------------------------ */

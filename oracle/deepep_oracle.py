@@ -28,6 +28,11 @@ generative on CUDA RNG streams that cannot be replayed here):
   kernels (``_serial_dispatch``) compared against the vectorised form.
 * combine — the closed form ``x * sum(w)`` of ``tests/test_low_latency.py:181``
   and a float64 sum.
+* ``topk_remap``, ``build_recv_src_meta`` — the torch expressions the reference's kernels
+  replaced (named in their headers, ``csrc/kernels/efa_kernels.cu:321-337,438-446``), pinned
+  by literal Python loops over the kernels' own per-element rule.
+* ``combine_reduce`` — ``zero_() + index_add_`` (``deep_ep/buffer.py:1542-1557``) in float64,
+  the identity "one rank per token returns the row itself", and a float32 chain in rank order.
 * ``get_low_latency_rdma_size_hint`` — hand-computed values.
 * ``round_scale`` scales: **parity unpinned at ulp boundaries** — the reference
   computes ``exp2(ceil(log2(s)))`` in float32 (``deep_ep/buffer.py:1601``,
@@ -127,6 +132,73 @@ def channel_prefix_matrix(is_token_in_rank: torch.Tensor, num_channels: int) -> 
         e = min(b + per, t)
         out[:, c] = is_token_in_rank[b:e].sum(0).to(torch.int32)
     return torch.cumsum(out, 1).to(torch.int32)
+
+
+# ----------------------------------------------------------------------------
+# Normal mode: the steps either side of the per-rank pack
+# ----------------------------------------------------------------------------
+def topk_remap(topk_idx: torch.Tensor, topk_weights: torch.Tensor, sorted_token_ids: torch.Tensor,
+               send_cumsum: torch.Tensor, num_local_experts: int):
+    """csrc/kernels/efa_kernels.cu:339-387, written as the torch expression that kernel replaced
+    (repeat_interleave + broadcast compare + where, :323): per send row, the token's top-k in the
+    destination rank's expert numbering; entries naming other ranks' experts become (-1, 0.0)."""
+    r = send_cumsum.numel() - 1
+    counts = (send_cumsum[1:] - send_cumsum[:-1]).to(torch.int64)
+    total = int(send_cumsum[r])
+    dst = torch.repeat_interleave(torch.arange(r, dtype=torch.int64), counts)
+    ids = sorted_token_ids[:total].to(torch.int64)
+    e = topk_idx[ids]
+    w = topk_weights[ids]
+    first = (dst * num_local_experts).view(-1, 1)
+    ok = (e >= first) & (e < first + num_local_experts)
+    return torch.where(ok, e - first, torch.full_like(e, -1)), torch.where(ok, w, torch.zeros_like(w))
+
+
+def build_recv_src_meta(recv_cumsum: torch.Tensor, num_local_ranks: int) -> torch.Tensor:
+    """csrc/kernels/efa_kernels.cu:448-482 as the expression it replaced (repeat_interleave +
+    division + shift, :440): [N, 8] uint8 holding the int32 pair (src // L, 1 << (src % L))."""
+    r = recv_cumsum.numel() - 1
+    counts = (recv_cumsum[1:] - recv_cumsum[:-1]).to(torch.int64)
+    src = torch.repeat_interleave(torch.arange(r, dtype=torch.int64), counts)
+    meta = torch.stack([src // num_local_ranks, torch.ones_like(src) << (src % num_local_ranks)], dim=1)
+    return meta.to(torch.int32).contiguous().view(torch.uint8).view(-1, 8)
+
+
+def combine_reduce(recv_x: torch.Tensor, recv_w, sorted_token_ids: torch.Tensor, num_tokens: int,
+                   bias_0=None, bias_1=None):
+    """deep_ep/buffer.py:1542-1557 in float64: zeros, index_add_ of the returned rows at their token
+    ids, then the biases.  Returns (x float64 [T, H], w float64 [T, K] or None)."""
+    total = sorted_token_ids.numel()
+    out = torch.zeros((num_tokens, recv_x.shape[1]), dtype=torch.float64)
+    out.index_add_(0, sorted_token_ids.to(torch.int64), recv_x[:total].double())
+    for b in (bias_0, bias_1):
+        if b is not None:
+            out += b.double()
+    w = None
+    if recv_w is not None:
+        w = torch.zeros((num_tokens, recv_w.shape[1]), dtype=torch.float64)
+        w.index_add_(0, sorted_token_ids.to(torch.int64), recv_w[:total].double())
+    return out, w
+
+
+def combine_reduce_f32_chain(recv_x: torch.Tensor, recv_w, sorted_token_ids: torch.Tensor,
+                             send_cumsum: torch.Tensor, num_tokens: int, bias_0=None, bias_1=None):
+    """The bit-level definition the kernel implements: float32 adds in ascending rank order (a token
+    occurs at most once per rank segment, so a per-segment indexed add is that order exactly), the
+    biases last, one rounding to bf16; weights the same way without the rounding."""
+    r = send_cumsum.numel() - 1
+    acc = torch.zeros((num_tokens, recv_x.shape[1]), dtype=torch.float32)
+    wacc = None if recv_w is None else torch.zeros((num_tokens, recv_w.shape[1]), dtype=torch.float32)
+    for rank in range(r):
+        lo, hi = int(send_cumsum[rank]), int(send_cumsum[rank + 1])
+        ids = sorted_token_ids[lo:hi].to(torch.int64)
+        acc[ids] = acc[ids] + recv_x[lo:hi].float()
+        if wacc is not None:
+            wacc[ids] = wacc[ids] + recv_w[lo:hi]
+    for b in (bias_0, bias_1):
+        if b is not None:
+            acc = acc + b.float()
+    return acc.to(torch.bfloat16), wacc
 
 
 # ----------------------------------------------------------------------------

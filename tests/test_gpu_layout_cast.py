@@ -196,3 +196,106 @@ def test_cast_argument_errors(capi):
     assert rc != 0 and "num_cols % 128 == 0" in lib.deepep_last_error().decode()
     with pytest.raises(capi.DeepEPError):
         capi.check(lib.deepep_per_token_cast_to_fp8(capi.ptr(x), 2, 128, 3, capi.ptr(x), capi.ptr(x), stream()))
+
+
+# ---- the steps either side of the normal-mode pack ------------------------------------------------
+def _normal_world(t, k, e, r, seed, drop=3):
+    topk = _topk(t, k, e, seed, drop)
+    if t > 2:
+        topk[0, :] = -1   # sent nowhere
+        topk[1, 1:] = -1  # held by exactly one rank
+    g = torch.Generator().manual_seed(seed + 1)
+    w = torch.rand((t, k), generator=g)
+    _, _, _, is_in = O.get_dispatch_layout(topk, e, r)
+    ids, counts, cumsum, total = O.moe_routing_sort(is_in)
+    return topk, w, is_in, ids, counts, cumsum, total
+
+
+@pytest.mark.parametrize("t,k,e,r", [(4096, 8, 256, 8), (333, 6, 64, 16), (5, 2, 8, 4), (1200, 8, 288, 72)])
+def test_topk_remap(capi, t, k, e, r):
+    lib = capi.load()
+    topk, w, _, ids, _, cumsum, total = _normal_world(t, k, e, r, seed=t + r)
+    want_e, want_w = O.topk_remap(topk, w, ids, cumsum, e // r)
+    cap = total + 7  # rows past the device-side total must stay untouched
+    out_e = torch.full((cap, k), -99, dtype=torch.int64, device="cuda")
+    out_w = torch.full((cap, k), -99.0, dtype=torch.float32, device="cuda")
+    ids_dev = torch.cat([ids, torch.zeros(7, dtype=torch.int64)]).cuda()
+    topk_dev, w_dev, cumsum_dev = topk.cuda(), w.cuda(), cumsum.cuda()  # named: they must outlive the launch
+    capi.check(lib.deepep_topk_remap(capi.ptr(topk_dev), capi.ptr(w_dev), capi.ptr(ids_dev), capi.ptr(cumsum_dev), t, k,
+                                     r, e // r, cap, capi.ptr(out_e), capi.ptr(out_w), stream()))
+    torch.cuda.synchronize()
+    assert torch.equal(out_e[:total].cpu(), want_e)
+    assert torch.equal(out_w[:total].cpu(), want_w)
+    assert (out_e[total:] == -99).all() and (out_w[total:] == -99.0).all()
+
+
+@pytest.mark.parametrize("r,local", [(8, 8), (32, 8), (17, 4), (1, 1)])
+def test_build_recv_src_meta(capi, r, local):
+    lib = capi.load()
+    g = torch.Generator().manual_seed(r)
+    counts = torch.randint(0, 50, (r,), generator=g)
+    counts[r // 2] = 0
+    cumsum = torch.zeros(r + 1, dtype=torch.int64)
+    cumsum[1:] = torch.cumsum(counts, 0)
+    total = int(cumsum[r])
+    want = O.build_recv_src_meta(cumsum, local)
+    meta = torch.full((total + 3, 8), 0xEE, dtype=torch.uint8, device="cuda")
+    cumsum_dev = cumsum.cuda()
+    capi.check(lib.deepep_build_recv_src_meta(capi.ptr(cumsum_dev), r, local, total + 3, capi.ptr(meta), stream()))
+    torch.cuda.synchronize()
+    assert torch.equal(meta[:total].cpu(), want)
+    assert (meta[total:] == 0xEE).all()
+
+
+@pytest.mark.parametrize("t,k,e,r,h,with_bias", [(4096, 8, 256, 8, 7168, False), (333, 6, 64, 16, 512, True),
+                                                 (5, 2, 8, 4, 128, True), (700, 8, 288, 72, 1024, False)])
+def test_combine_reduce(capi, t, k, e, r, h, with_bias):
+    """The per-token sum of the rows that came back: bit-exact against the float32 chain in rank order,
+    within 1e-2 relative of the float64 index_add_ of deep_ep/buffer.py:1542-1557."""
+    lib = capi.load()
+    topk, w, is_in, ids, counts, cumsum, total = _normal_world(t, k, e, r, seed=t + h)
+    g = torch.Generator().manual_seed(5)
+    rows = torch.randn((total, h), generator=g).to(torch.bfloat16)
+    rw = torch.rand((total, k), generator=g)
+    b0 = torch.randn((t, h), generator=g).to(torch.bfloat16) if with_bias else None
+    b1 = torch.randn((t, h), generator=g).to(torch.bfloat16) if with_bias else None
+    out_x = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    out_x.view(torch.int16).fill_(0x7FC0)
+    out_w = torch.full((t, k), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.full((max(256, lib.deepep_combine_reduce_workspace_bytes(t, r)),), 0x7F, dtype=torch.uint8, device="cuda")
+    dev = [None if v is None else v.cuda() for v in (rows, rw, ids, cumsum, is_in, b0, b1)]  # outlive the launch
+    capi.check(lib.deepep_combine_reduce(*[capi.ptr(v) for v in dev], t, h, k, r, total, capi.ptr(out_x),
+                                         capi.ptr(out_w), capi.ptr(ws), ws.numel(), stream()))
+    torch.cuda.synchronize()
+    chain_x, chain_w = O.combine_reduce_f32_chain(rows, rw, ids, cumsum, t, b0, b1)
+    assert torch.equal(out_x.cpu().view(torch.int16), chain_x.view(torch.int16))
+    assert torch.equal(out_w.cpu(), chain_w)
+    ref_x, ref_w = O.combine_reduce(rows, rw, ids, t, b0, b1)
+    err = (out_x.cpu().double() - ref_x).abs()
+    assert (err <= 1e-2 * ref_x.abs() + 1e-2 * ref_x.abs().mean()).all()
+    assert torch.allclose(out_w.cpu().double(), ref_w, rtol=1e-5, atol=1e-6)
+
+
+def test_normal_mode_steps_through_the_host_module():
+    """topk_remap / build_recv_src_meta / combine_reduce with the reference's Python-visible signatures."""
+    from deepep_efa_amd import normal
+    t, k, e, r, h = 257, 4, 32, 8, 256
+    topk, w, is_in, ids, counts, cumsum, total = _normal_world(t, k, e, r, seed=12)
+    ids_d, counts_d, cumsum_d, total_d = normal.moe_routing_sort(is_in.cuda())
+    assert total_d == total and torch.equal(ids_d.cpu(), ids)
+    re, rw = normal.topk_remap(topk.cuda(), w.cuda(), ids_d, cumsum_d, total_d, r, e // r)
+    want_e, want_w = O.topk_remap(topk, w, ids, cumsum, e // r)
+    assert torch.equal(re.cpu(), want_e) and torch.equal(rw.cpu(), want_w)
+    meta = normal.build_recv_src_meta(counts_d, cumsum_d, total_d, r, 8)
+    assert torch.equal(meta.cpu(), O.build_recv_src_meta(cumsum, 8))
+    # the exchange is the identity here: every rank returns the row it was sent
+    x = torch.randn((t, h), generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
+    send_x, _ = normal.pack_rows(x.cuda(), None, ids_d, cumsum_d)
+    cx, cw = normal.combine_reduce(send_x, rw, ids_d, cumsum_d, is_in.cuda())
+    # remapped weights are zero outside the destination's experts, so their sum is the original weight row
+    want_cw = torch.where(topk >= 0, w, torch.zeros_like(w))
+    assert torch.allclose(cw.cpu(), want_cw, rtol=1e-6, atol=1e-7)
+    chain_x, _ = O.combine_reduce_f32_chain(x[ids], None, ids, cumsum, t)
+    assert torch.equal(cx.cpu().view(torch.int16), chain_x.view(torch.int16))
+    with pytest.raises(RuntimeError, match="Assertion"):
+        normal.topk_remap(topk.cuda(), w.cuda(), ids_d, cumsum_d, total_d + 10 ** 6, r, e // r)

@@ -376,3 +376,83 @@ def test_seeded_topk_numpy_equals_c(oracle_c, cdf_name):
     assert (srt[..., 1:] != srt[..., :-1]).all() and a.min() >= 0 and a.max() < e
     if cdf_name == "zipf":
         assert (a == 0).any(-1).float().mean() > 0.5  # the hottest expert is in most tokens
+
+
+# ---- normal mode: top-k remap, source metadata, combine reduce -------------------------------------
+def _normal_world(t, k, e, r, seed):
+    g = torch.Generator().manual_seed(seed)
+    topk = torch.argsort(torch.rand((t, e), generator=g), dim=1)[:, :k].contiguous()
+    topk[t // 2, 0] = -1
+    topk[0, :] = -1     # a token sent nowhere
+    topk[1, 1:] = -1    # a token held by exactly one rank
+    w = torch.rand((t, k), generator=g)
+    _, _, _, is_in = O.get_dispatch_layout(topk, e, r)
+    ids, counts, cumsum, _ = O.moe_routing_sort(is_in)
+    return topk, w, is_in, ids, counts, cumsum
+
+
+def test_topk_remap_against_the_kernels_per_element_rule():
+    # csrc/kernels/efa_kernels.cu:352-386, one (row, k) at a time
+    t, k, e, r = 37, 4, 24, 6
+    topk, w, _, ids, _, cumsum = _normal_world(t, k, e, r, seed=3)
+    got_e, got_w = O.topk_remap(topk, w, ids, cumsum, e // r)
+    total = int(cumsum[r])
+    assert got_e.shape == (total, k)
+    for row in range(total):
+        dst = max(d for d in range(r) if int(cumsum[d]) <= row and int(cumsum[d + 1]) > row)
+        tok = int(ids[row])
+        for kk in range(k):
+            ex = int(topk[tok, kk])
+            lo, hi = dst * (e // r), (dst + 1) * (e // r)
+            if lo <= ex < hi and ex >= 0:
+                assert int(got_e[row, kk]) == ex - lo and float(got_w[row, kk]) == float(w[tok, kk])
+            else:
+                assert int(got_e[row, kk]) == -1 and float(got_w[row, kk]) == 0.0
+    # every send row keeps at least one selection: that is why the token was sent to that rank
+    assert ((got_e >= 0).sum(1) >= 1).all()
+
+
+def test_build_recv_src_meta_against_the_kernels_per_element_rule():
+    # csrc/kernels/efa_kernels.cu:456-481
+    cumsum = torch.tensor([0, 3, 3, 4, 9, 9, 11, 11, 12, 15, 15, 15, 16, 20, 20, 21, 30, 31], dtype=torch.int64)
+    r, local = cumsum.numel() - 1, 8
+    meta = O.build_recv_src_meta(cumsum, local).view(torch.int32).view(-1, 2)
+    assert meta.shape[0] == int(cumsum[r])
+    for i in range(meta.shape[0]):
+        src = max(s for s in range(r) if int(cumsum[s]) <= i < int(cumsum[s + 1]))
+        assert meta[i].tolist() == [src // local, 1 << (src % local)]
+
+
+def test_combine_reduce_definitions_agree():
+    t, k, e, r, h = 29, 3, 16, 4, 256
+    topk, w, is_in, ids, counts, cumsum = _normal_world(t, k, e, r, seed=8)
+    g = torch.Generator().manual_seed(1)
+    total = int(cumsum[r])
+    rows = torch.randn((total, h), generator=g).to(torch.bfloat16)
+    rw = torch.rand((total, k), generator=g)
+    b0 = torch.randn((t, h), generator=g).to(torch.bfloat16)
+    ref_x, ref_w = O.combine_reduce(rows, rw, ids, t, b0, None)
+    # the same sum written as a loop over (token, rank) pairs
+    want = b0.double().clone()
+    pos = 0
+    for rank in range(r):
+        for tok in range(t):
+            if is_in[tok, rank]:
+                want[tok] += rows[pos].double()
+                pos += 1
+    assert pos == total and torch.equal(ref_x, want)
+    chain_x, chain_w = O.combine_reduce_f32_chain(rows, rw, ids, cumsum, t, b0, None)
+    err = (chain_x.double() - ref_x).abs()
+    assert (err <= 2.0 ** -8 * ref_x.abs() + 1e-6).all()  # one bf16 rounding of a float32 sum of <= 5 terms
+    assert torch.allclose(chain_w.double(), ref_w, rtol=1e-6, atol=1e-7)
+    # a token held by exactly one rank gets its row back bit for bit (no bias)
+    chain_nb, _ = O.combine_reduce_f32_chain(rows, None, ids, cumsum, t)
+    single = torch.nonzero(is_in.sum(1) == 1).flatten()
+    assert single.numel() > 0
+    for tok in single.tolist():
+        j = int(torch.nonzero(ids == tok).flatten()[0])
+        assert torch.equal(chain_nb[tok].view(torch.int16), rows[j].view(torch.int16))
+    # a token sent nowhere gives zeros
+    none = torch.nonzero(is_in.sum(1) == 0).flatten()
+    for tok in none.tolist():
+        assert (chain_nb[tok] == 0).all()
