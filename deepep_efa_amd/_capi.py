@@ -32,10 +32,10 @@ PROTOTYPES = {
     "deepep_ll_segment_workspace_bytes": (_SZ, [_I, _I]),
     "deepep_ll_dispatch_recv": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _SZ, _VP]),
     "deepep_ll_combine_send": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I64, _VP, _SZ, _VP]),
-    "deepep_ll_combine_recv": (_I, [_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP, _VP]),
+    "deepep_ll_combine_recv": (_I, [_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP]),
     "deepep_ll_dispatch": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                 _VP, _I64, _VP, _SZ, _VP, _SZ, _VP]),
-    "deepep_ll_combine": (_I, [_VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _I64, _VP, _SZ,
+    "deepep_ll_combine": (_I, [_VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _I64, _VP, _SZ,
                                _VP]),
     "deepep_topk_remap": (_I, [_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP]),
     "deepep_build_recv_src_meta": (_I, [_VP, _I, _I, _I64, _VP, _VP]),

@@ -564,7 +564,7 @@ struct Buffer {
         abi_check(deepep_ll_combine(src.data_ptr(), layout_range.data_ptr<int64_t>(), topk_idx.data_ptr<int64_t>(),
                                     topk_weights.data_ptr<float>(), c.pair_slot.data_ptr<int>(), num_combined_tokens,
                                     hidden, num_topk, num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,
-                                    c.combine_staging.data_ptr(), c.combine_send_slots.data_ptr(),
+                                    /*accumulate=*/0, c.combine_staging.data_ptr(), c.combine_send_slots.data_ptr(),
                                     combined_x.data_ptr(), int64_t(num_max_dispatch_tokens_per_rank) * num_topk,
                                     c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
                                     c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));

@@ -106,6 +106,7 @@ struct CombineRecvArgs {
     const float* topk_weights;
     const int32_t* pair_slot;
     int num_tokens, hidden, num_topk, num_experts, max_tokens, pieces_per_row;
+    int accumulate;  // non-zero: the sum starts from what `out` already holds
     uint8_t* out;
 };
 
@@ -150,6 +151,11 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    if (a.accumulate != 0 && lane_live) {  // reference: csrc/kernels/coop_combine_recv.cuh:174-179
+        const u32x4 prev = load_global_u32x4(a.out + int64_t(t) * row_bytes + off);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[2 * i] = bf16_lo(prev[i]), acc[2 * i + 1] = bf16_hi(prev[i]);
+    }
 
     for (int k0 = 0; k0 < num_topk; k0 += 8) {
         u32x4 v[8];
@@ -234,12 +240,14 @@ static CombineSendArgs make_combine_send_args(const void* x, const int64_t* layo
 
 static CombineRecvArgs make_combine_recv_args(const void* combine_staging, const int64_t* topk_idx,
                                               const float* topk_weights, const int32_t* pair_slot, int num_tokens,
-                                              int hidden, int num_topk, int num_experts, int max_tokens, void* out) {
+                                              int hidden, int num_topk, int num_experts, int max_tokens, int accumulate,
+                                              void* out) {
     CombineRecvArgs ra;
     ra.combine_staging = reinterpret_cast<const uint8_t*>(combine_staging);
     ra.topk_idx = topk_idx, ra.topk_weights = topk_weights, ra.pair_slot = pair_slot;
     ra.num_tokens = num_tokens, ra.hidden = hidden, ra.num_topk = num_topk, ra.num_experts = num_experts;
     ra.max_tokens = max_tokens, ra.pieces_per_row = (hidden * 2 + 1023) / 1024;
+    ra.accumulate = accumulate;
     ra.out = reinterpret_cast<uint8_t*>(out);
     return ra;
 }
@@ -326,7 +334,7 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
 
 int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx, const float* topk_weights,
                            const int32_t* pair_slot, int num_tokens, int hidden, int num_topk, int num_experts,
-                           int num_max_dispatch_tokens_per_rank, void* out, void* stream) {
+                           int num_max_dispatch_tokens_per_rank, int accumulate, void* out, void* stream) {
     clear_error();
     if (int rc = check_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden,
                                          num_topk, num_experts, num_max_dispatch_tokens_per_rank, out))
@@ -334,7 +342,7 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
     if (num_tokens == 0) return 0;
     const CombineRecvArgs ra = make_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens,
                                                       hidden, num_topk, num_experts,
-                                                      num_max_dispatch_tokens_per_rank, out);
+                                                      num_max_dispatch_tokens_per_rank, accumulate, out);
     const int64_t blocks = (int64_t(num_tokens) * ra.pieces_per_row + 3) / 4;
     ll_combine_recv_kernel<<<dim3(unsigned(blocks)), 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(ra);
     EP_LAUNCH_CHECK();
@@ -343,9 +351,9 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
 
 int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t* topk_idx, const float* topk_weights,
                       const int32_t* pair_slot, int num_tokens, int hidden, int num_topk, int num_experts,
-                      int num_ranks, int rank, int num_max_dispatch_tokens_per_rank, void* combine_staging,
-                      void* combine_send_slots, void* out, int64_t expected_rows, void* workspace,
-                      size_t workspace_bytes, void* stream) {
+                      int num_ranks, int rank, int num_max_dispatch_tokens_per_rank, int accumulate,
+                      void* combine_staging, void* combine_send_slots, void* out, int64_t expected_rows,
+                      void* workspace, size_t workspace_bytes, void* stream) {
     clear_error();
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     if (max_rows > kLargeBatchRows) {  // the two phases back to back
@@ -354,7 +362,7 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
                                             expected_rows, workspace, workspace_bytes, stream))
             return rc;
         return deepep_ll_combine_recv(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden, num_topk,
-                                      num_experts, num_max_dispatch_tokens_per_rank, out, stream);
+                                      num_experts, num_max_dispatch_tokens_per_rank, accumulate, out, stream);
     }
     if (int rc = check_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
                                          num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots))
@@ -367,7 +375,7 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
                                                       combine_send_slots);
     const CombineRecvArgs ra = make_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens,
                                                       hidden, num_topk, num_experts,
-                                                      num_max_dispatch_tokens_per_rank, out);
+                                                      num_max_dispatch_tokens_per_rank, accumulate, out);
     const int64_t recv_blocks = (int64_t(num_tokens) * ra.pieces_per_row + 3) / 4;
     int64_t rows = expected_rows > 0 ? expected_rows : int64_t(num_max_dispatch_tokens_per_rank) * num_topk;
     rows += rows / 8 + 16;

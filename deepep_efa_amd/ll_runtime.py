@@ -137,15 +137,17 @@ class LowLatencyState:
             _capi.ptr(self.segment_workspace),
             0 if self.segment_workspace is None else self.segment_workspace.numel(), current_stream_ptr()))
 
-    def combine_recv(self, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor) -> None:
+    def combine_recv(self, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor,
+                     accumulate: bool = False) -> None:
         s = self.shape
         t = topk_idx.shape[0]
         _capi.check(self.lib.deepep_ll_combine_recv(
             _capi.ptr(self.combine_staging), _capi.ptr(topk_idx), _capi.ptr(topk_weights), _capi.ptr(self.pair_slot),
-            t, s.hidden, s.num_topk, s.num_experts, s.max_tokens, _capi.ptr(out), current_stream_ptr()))
+            t, s.hidden, s.num_topk, s.num_experts, s.max_tokens, int(accumulate), _capi.ptr(out),
+            current_stream_ptr()))
 
     def combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor,
-                layout_range: torch.Tensor = None) -> None:
+                layout_range: torch.Tensor = None, accumulate: bool = False) -> None:
         """Row return + weighted reduce in one call; the remote experts' answers must already be staged."""
         s = self.shape
         t = topk_idx.shape[0]
@@ -153,6 +155,6 @@ class LowLatencyState:
         sw = self.segment_workspace
         _capi.check(self.lib.deepep_ll_combine(
             _capi.ptr(x), _capi.ptr(lr), _capi.ptr(topk_idx), _capi.ptr(topk_weights), _capi.ptr(self.pair_slot),
-            t, s.hidden, s.num_topk, s.num_experts, s.num_ranks, s.rank, s.max_tokens,
+            t, s.hidden, s.num_topk, s.num_experts, s.num_ranks, s.rank, s.max_tokens, int(accumulate),
             _capi.ptr(self.combine_staging), _capi.ptr(self.combine_send_slots), _capi.ptr(out),
             self.expected_rows, _capi.ptr(sw), 0 if sw is None else sw.numel(), current_stream_ptr()))

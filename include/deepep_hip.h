@@ -289,13 +289,14 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range,
  * selection give zeros.
  *   combine_staging [E, M, H] bf16     topk_idx [T, K] int64
  *   topk_weights    [T, K] float32     pair_slot [T, K] int32 from the dispatch
- *   out             [T, H] bf16 (out)
+ *   out             [T, H] bf16 (out; in/out when accumulate != 0: the sum then starts from
+ *                   f32(out[t,:]) instead of zero, csrc/kernels/coop_combine_recv.cuh:174-179)
  * Replaces ll_combine_weighted_reduce_v2 (csrc/kernels/efa_kernels.cu:1413-1486,1982-2031)
  * and a2a_combine_recv (csrc/deep_ep.cpp:3850, csrc/kernels/coop_combine_recv.cuh:69-283). */
 int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
                            const float* topk_weights, const int32_t* pair_slot,
                            int num_tokens, int hidden, int num_topk, int num_experts,
-                           int num_max_dispatch_tokens_per_rank, void* out, void* stream);
+                           int num_max_dispatch_tokens_per_rank, int accumulate, void* out, void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Whole dispatch / whole combine in one call                          */
@@ -340,7 +341,7 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range,
                       const int64_t* topk_idx, const float* topk_weights,
                       const int32_t* pair_slot,
                       int num_tokens, int hidden, int num_topk, int num_experts,
-                      int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                      int num_ranks, int rank, int num_max_dispatch_tokens_per_rank, int accumulate,
                       void* combine_staging, void* combine_send_slots, void* out,
                       int64_t expected_rows, void* workspace, size_t workspace_bytes,
                       void* stream);

@@ -437,8 +437,11 @@ def ll_combine(pair_rows: torch.Tensor, topk_idx: torch.Tensor, topk_weights: to
     return (pair_rows.double() * w.unsqueeze(-1)).sum(1)
 
 
-def ll_combine_f32_chain(pair_rows: torch.Tensor, topk_weights: torch.Tensor, pair_live: torch.Tensor):
+def ll_combine_f32_chain(pair_rows: torch.Tensor, topk_weights: torch.Tensor, pair_live: torch.Tensor,
+                         initial: torch.Tensor = None):
     """Bit-level definition: acc = 0; for k: acc = fma(f32(row_k), w_k, acc); bf16_rne(acc).
+    `initial` [T, H] bf16: the accumulate variant (csrc/kernels/coop_combine_recv.cuh:174-179),
+    acc starts as f32(initial) instead of zero.
 
     float32 FMA emulated exactly: the product of two float32 is exact in float64;
     the float64 sum with a float32 addend is rounded once to float64 and once more
@@ -447,7 +450,7 @@ def ll_combine_f32_chain(pair_rows: torch.Tensor, topk_weights: torch.Tensor, pa
     (oracle_kernels.c, fmaf) covers; this torch form is used for speed.
     """
     t, k, h = pair_rows.shape
-    acc = torch.zeros((t, h), dtype=torch.float32)
+    acc = torch.zeros((t, h), dtype=torch.float32) if initial is None else initial.float().clone()
     for j in range(k):
         prod = pair_rows[:, j].double() * topk_weights[:, j].double().unsqueeze(1)
         nxt = (prod + acc.double()).float()

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in include/deepep_hip.h but not exported"
         assert name in _capi.PROTOTYPES, f"{name} has no ctypes prototype"
     assert sorted(_capi.PROTOTYPES) == declared
-    assert lib.deepep_abi_version() == 3
+    assert lib.deepep_abi_version() == 4
 
 
 @pytest.mark.parametrize("hidden", [128, 512, 2048, 7168])
@@ -55,7 +55,7 @@ def test_host_argument_checks_without_a_gpu():
     assert rc != 0
     assert lib.deepep_last_error().decode() == "Failed: Assertion error cast.hip:%d 'num_rows >= 0 && num_cols > 0 && num_cols %% 128 == 0'" % \
         int(re.search(r"cast\.hip:(\d+)", lib.deepep_last_error().decode()).group(1))
-    rc = lib.deepep_ll_combine_recv(None, None, None, None, 4, 7168, 0, 256, 128, None, None)
+    rc = lib.deepep_ll_combine_recv(None, None, None, None, 4, 7168, 0, 256, 128, 0, None, None)
     assert rc != 0 and "num_topk > 0" in lib.deepep_last_error().decode()
     rc = lib.deepep_moe_routing_sort(None, -1, 8, None, None, None, None, 0, None)
     assert rc != 0 and lib.deepep_last_error().decode().startswith("Failed: Assertion error layout.hip:")

@@ -281,6 +281,16 @@ def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e, one_ca
                                   h, ctypes.c_void_p(chain.data_ptr()))
     got = out.cpu()
     assert torch.equal(got.view(torch.int16), chain), "combine differs from the float32 FMA chain"
+    # accumulate: the sum starts from what `out` holds (csrc/kernels/coop_combine_recv.cuh:174-179)
+    prev = torch.randn((t, h), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    out2 = prev.cuda()
+    if one_call:
+        st.combine(y, topk_all[rank].cuda(), w_all[rank].cuda(), out2, accumulate=True)
+    else:
+        st.combine_recv(topk_all[rank].cuda(), w_all[rank].cuda(), out2, accumulate=True)
+    torch.cuda.synchronize()
+    want2 = O.ll_combine_f32_chain(pair_rows, w, live, initial=prev)
+    assert torch.equal(out2.cpu().view(torch.int16), want2.view(torch.int16)), "accumulating combine"
     ref = O.ll_combine(pair_rows, topk, w, live)
     err = (got.double() - ref).abs()
     assert (err <= 1e-2 * ref.abs() + 1e-2 * ref.abs().mean()).all()
