@@ -131,6 +131,8 @@ def check_dispatch(st, want, fmt):
     (2, 1, 600, 512, 8, 16),   # T*K > 2048: chunked route + cross-chunk scan
     (4, 3, 300, 512, 11, 32),  # both
     (8, 5, 4200, 512, 4, 64),  # E*M > 2^18: receive runs as index kernel + flat row copy
+    (8, 2, 20, 512, 4, 512),   # more than 256 segments: 16 counts per lane in the register segment table
+    (16, 9, 12, 512, 6, 1024),  # the most experts the path takes
 ])
 @ONE_CALL
 def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
@@ -231,7 +233,9 @@ def test_reference_recipe_roundtrip(rt, use_fp8, one_call):
 
 
 @pytest.mark.parametrize("r,rank,t,h,k,e", [(32, 5, 128, 7168, 8, 256), (4, 0, 16, 512, 3, 8),
-                                            (8, 3, 4200, 512, 4, 64)])  # the last: large-batch combine-send path
+                                            (8, 3, 4200, 512, 4, 64),   # large-batch combine-send path
+                                            (4, 2, 40, 512, 11, 64),    # more than eight selections per token
+                                            (8, 6, 20, 512, 4, 512)])   # more than 256 segments
 @ONE_CALL
 def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e, one_call):
     """Seeded expert outputs along the dispatch routing; combine vs the float32 chain and the float64 sum."""
