@@ -6,6 +6,8 @@
 //   combine_staging     [E][M][H] bf16 — slot j of expert e holds the output
 //                       for this rank's pair whose dispatch slot was j
 //   combine_send_slots  [E_l][R][M][H] bf16 — rows owed to other ranks
+#include <cstdlib>
+
 #include "common.hpp"
 #include "segments.hpp"
 #include "../../include/deepep_hip.h"
@@ -194,8 +196,8 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
     }
 }
 
-__global__ __launch_bounds__(256) void ll_combine_recv_kernel(CombineRecvArgs a) {
-    combine_recv_piece(a, int64_t(blockIdx.x) * 4 + wave_in_block(), nullptr, nullptr, 0, 0, 0);
+__global__ __launch_bounds__(1024) void ll_combine_recv_kernel(CombineRecvArgs a) {
+    combine_recv_piece(a, int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(), nullptr, nullptr, 0, 0, 0);
 }
 
 // ---------------------------------------------------------------------
@@ -343,8 +345,9 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
     const CombineRecvArgs ra = make_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens,
                                                       hidden, num_topk, num_experts,
                                                       num_max_dispatch_tokens_per_rank, accumulate, out);
-    const int64_t blocks = (int64_t(num_tokens) * ra.pieces_per_row + 3) / 4;
-    ll_combine_recv_kernel<<<dim3(unsigned(blocks)), 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(ra);
+    const int waves = 4;  // block shape makes no measurable difference (1..16 waves: within 5 %)
+    const int64_t blocks = (int64_t(num_tokens) * ra.pieces_per_row + waves - 1) / waves;
+    ll_combine_recv_kernel<<<dim3(unsigned(blocks)), waves * kWave, 0, reinterpret_cast<hipStream_t>(stream)>>>(ra);
     EP_LAUNCH_CHECK();
     return 0;
 }

@@ -89,18 +89,39 @@ __global__ __launch_bounds__(kRouteChunk) void ll_route_slots_kernel(
     }
     __syncthreads();
 
-    // base: histogram of every earlier chunk, eight independent loads per thread per step
-    const int before = c * kRouteChunk;
-    for (int i0 = tid; i0 < before; i0 += kRouteChunk * 8) {
-        int64_t v[8];
+    // base: histogram of every earlier chunk.  Two entries per 16-byte load, sixteen loads in flight
+    // per thread: one round of memory latency covers 32 chunks.
+    const int before = c * kRouteChunk;  // a multiple of 1024, so pairs never straddle it
+    if ((reinterpret_cast<uintptr_t>(my_topk) & 15) == 0) {
+        const u32x4* pairs = reinterpret_cast<const u32x4*>(my_topk);
+        const int num_pairs = before >> 1;
+        for (int p0 = tid; p0 < num_pairs; p0 += kRouteChunk * 16) {
+            u32x4 v[16];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const int j = i0 + u * kRouteChunk;
-            v[u] = j < before ? my_topk[j] : -1;
+            for (int u = 0; u < 16; ++u) {
+                const int p = p0 + u * kRouteChunk;
+                if (p < num_pairs) v[u] = pairs[p];
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                if (p0 + u * kRouteChunk >= num_pairs) continue;
+                // an int64 entry is valid when its high word is zero and its low word is below E
+                if (v[u][1] == 0 && v[u][0] < uint32_t(num_experts)) atomicAdd(&base_hist[v[u][0]], 1);
+                if (v[u][3] == 0 && v[u][2] < uint32_t(num_experts)) atomicAdd(&base_hist[v[u][2]], 1);
+            }
         }
+    } else {
+        for (int i0 = tid; i0 < before; i0 += kRouteChunk * 8) {
+            int64_t v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u)
-            if (v[u] >= 0 && v[u] < num_experts) atomicAdd(&base_hist[int(v[u])], 1);
+            for (int u = 0; u < 8; ++u) {
+                const int j = i0 + u * kRouteChunk;
+                v[u] = j < before ? my_topk[j] : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (v[u] >= 0 && v[u] < num_experts) atomicAdd(&base_hist[int(v[u])], 1);
+        }
     }
 
     // rank inside the wave
