@@ -285,3 +285,48 @@ def test_normal_mode_layout_and_pack(deep_ep):
     assert torch.equal(pq.cpu().view(torch.uint8), wq.view(torch.uint8)[w_ids])
     assert torch.equal(psc.cpu(), ws[w_ids])
     buffer.destroy()
+
+
+def test_dispatch_and_combine_replay_in_a_hip_graph(deep_ep):
+    """Decode loops capture the dispatch + combine pair once and replay it.  The captured calls must
+    allocate nothing and record no memset; every replay, with eager work and synchronisations in
+    between, must give the eager result."""
+    num_ranks, rank, t, h, k, e = 16, 4, 64, 2048, 6, 64
+    buffer = deep_ep.Buffer(None, low_latency_mode=True, explicitly_destroy=True, sim_num_ranks=num_ranks,
+                            sim_rank=rank, sim_seed=21)
+    x, topk_idx = buffer.loopback_synthesise(t, h, k, e)
+    w = torch.softmax(torch.randn((t, k), generator=torch.Generator().manual_seed(4)), dim=-1).cuda()
+
+    def step():
+        (rx, rs), cnt, handle, _, _ = buffer.low_latency_dispatch(x, topk_idx, t, e)
+        y = (rx.float().view(rx.shape[0], rx.shape[1], h // 128, 128) * rs.unsqueeze(-1)).view(rx.shape).to(torch.bfloat16)
+        out, _, _ = buffer.low_latency_combine(y, topk_idx, w, handle)
+        return rx, rs, cnt, handle, out
+
+    rx, rs, cnt, handle, out = step()  # eager: also fills the per-shape caches
+    torch.cuda.synchronize()
+    want = [v.clone() for v in (rx.view(torch.uint8), rs, cnt, handle[0], handle[1], out)]
+    live = torch.arange(rx.shape[1], device="cuda").view(1, -1) < cnt.view(-1, 1)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        grx, grs, gcnt, ghandle, gout = step()
+    for replay in range(4):
+        for v in (grx.view(torch.uint8), grs, gout):  # eager work between replays: scribble over the outputs
+            v.fill_(0)
+        gcnt.fill_(-1)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = (grx.view(torch.uint8), grs, gcnt, ghandle[0], ghandle[1], gout)
+        assert torch.equal(got[2], want[2]) and torch.equal(got[4], want[4]), f"replay {replay}: counts / layout"
+        assert torch.equal(got[0][live], want[0][live]), f"replay {replay}: payload"
+        assert torch.equal(got[1][live], want[1][live]), f"replay {replay}: scales"
+        assert torch.equal(got[3][live], want[3][live]), f"replay {replay}: src_info"
+        assert torch.equal(got[5].view(torch.int16), want[5].view(torch.int16)), f"replay {replay}: combined"
+    buffer.destroy()
