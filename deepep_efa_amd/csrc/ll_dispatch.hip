@@ -1,5 +1,6 @@
-// Low-latency dispatch: route ranking, fused quantise + pack (send side) and
-// segment compaction (receive side).
+// Low-latency dispatch: route ranking, fused quantise + pack (send side),
+// segment compaction (receive side), and the single launch that runs both
+// for decode-sized batches.
 //
 // Data layout in HBM (row stride S = row_stride_bytes(H, format)):
 //   recv_staging  [E_l][R][M] rows — slot j of segment (e_l, s) is the j-th
@@ -167,17 +168,19 @@ __global__ __launch_bounds__(kRouteChunk) void ll_route_slots_kernel(
 // (reference idea: csrc/kernels/coop_dispatch_send.cuh:572-607).
 //
 // Per-selection bookkeeping (slot, destination row address, row tail,
-// pair_slot) is done once per token by the first K threads and handed to the
-// waves through LDS, so a wave's own work is: two loads, the DPP quantise,
-// and per selection one 8-byte LDS read and two stores.
+// pair_slot) is done once per token by lanes 0..K-1 of wave 0 and handed to the
+// other waves through LDS; each wave reads all K destinations with one LDS
+// access and takes them back per selection with readlane.  Quantisation runs
+// while wave 0 does that.  Barriers fence LDS only, so the row loads stay in
+// flight across them.
 //
 // A small batch (T*K <= 2048) needs no route kernel: while the row loads are
-// in flight the workgroup's threads sweep the (token,k) entries before the
-// token, one entry per thread per step, and bump an LDS counter for every entry
-// that names one of the token's experts (integer adds — order does not matter);
-// the per-expert totals come from one extra row of workgroups (blockIdx.y == T),
-// an LDS histogram per source.  Larger batches read the slots ranked by
-// ll_route_slots_kernel.
+// in flight every thread fetches up to four (token,k) entries that precede the
+// token (more in a loop for workgroups under 512 threads); each wave counts, per
+// selection, its entries naming that selection's expert with a ballot and a
+// popcount, and wave 0 adds the waves' counts.  The per-expert totals come from
+// one extra workgroup per source, an LDS histogram.  Larger batches read the
+// slots ranked by ll_route_slots_kernel.
 // ---------------------------------------------------------------------
 constexpr int kMaxTopk = 64;
 constexpr int kFusedMaxEntries = 2048;

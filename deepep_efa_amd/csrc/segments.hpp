@@ -1,6 +1,8 @@
 // Helpers for kernels that walk a list of variable-length row segments with
-// one wavefront per row: a workgroup-wide exclusive scan in LDS, the row ->
-// segment search, and the 16-byte-per-lane row copy.
+// one wavefront per row (part): the segment prefix held in a wave's registers
+// with its row -> segment lookup, a workgroup-wide exclusive scan in LDS for the
+// metadata pass, the 16-byte-per-lane row copy, and the index + flat-copy pair
+// of kernels for large batches.
 #pragma once
 
 #include <cstdlib>
@@ -42,16 +44,6 @@ __device__ __forceinline__ void block_exclusive_scan(int32_t* data, int n, int32
         }
     if (tid == 0) data[n] = total;
     lds_barrier();
-}
-
-// Largest seg with flat[seg] <= row, for flat[] non-decreasing, flat[0] = 0.
-__device__ __forceinline__ int find_segment(const int32_t* flat, int num_segments, int row) {
-    int lo = 0, hi = num_segments;  // invariant: flat[lo] <= row < flat[hi]
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (flat[mid] <= row) lo = mid; else hi = mid;
-    }
-    return lo;
 }
 
 // ---------------------------------------------------------------------
