@@ -359,9 +359,9 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
                       void* workspace, size_t workspace_bytes, void* stream) {
     clear_error();
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
-    // one launch pays while the batch is latency-bound; past ~256 tokens x top-8 the two kernels, each
-    // shaped for its own access pattern, are faster back to back (measured crossover: 300-400 tokens)
-    if (max_rows > kLargeBatchRows || int64_t(num_tokens) * num_topk > 2048) {
+    // measured as whole calls the single launch wins up to this bound (512 tokens: 36 us against 40 for
+    // the phases back to back), although each phase timed alone on cache-warm data suggests otherwise
+    if (max_rows > kLargeBatchRows) {  // the two phases back to back
         if (int rc = deepep_ll_combine_send(x, layout_range, hidden, num_experts, num_ranks, rank,
                                             num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots,
                                             expected_rows, workspace, workspace_bytes, stream))

@@ -174,7 +174,7 @@ __global__ __launch_bounds__(kRouteChunk) void ll_route_slots_kernel(
 // while wave 0 does that.  Barriers fence LDS only, so the row loads stay in
 // flight across them.
 //
-// A small batch (T*K <= 2048) needs no route kernel: while the row loads are
+// A batch of up to 8192 (token,k) entries needs no route kernel: while the row loads are
 // in flight every thread fetches up to four (token,k) entries that precede the
 // token (more in a loop for workgroups under 512 threads); each wave counts, per
 // selection, its entries naming that selection's expert with a ballot and a
@@ -183,7 +183,8 @@ __global__ __launch_bounds__(kRouteChunk) void ll_route_slots_kernel(
 // slots ranked by ll_route_slots_kernel.
 // ---------------------------------------------------------------------
 constexpr int kMaxTopk = 64;
-constexpr int kFusedMaxEntries = 2048;
+constexpr int kFusedMaxEntries = 2048;     // send + receive in one launch up to here
+constexpr int kSelfRankMaxEntries = 8192;  // the send kernel ranks its own slots up to here
 constexpr int kSendMaxWaves = 16;
 
 struct SendArgs {
@@ -345,11 +346,19 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             for (int r = 0; r < kSweepAhead; ++r) count += __popcll(__ballot(ahead[r] == e));
             if (lane == k) my_count = count;
         }
-        for (int base = kSweepAhead * int(blockDim.x); base < entry0; base += blockDim.x) {
-            const int64_t v = base + tid < entry0 ? my_topk[base + tid] : -1;
-            const int e32 = v >= 0 && v < num_experts ? int(v) : -1;
+        for (int base = kSweepAhead * int(blockDim.x); base < entry0; base += kSweepAhead * int(blockDim.x)) {
+            int more[kSweepAhead];  // the same again, four loads in flight per thread
+#pragma unroll
+            for (int r = 0; r < kSweepAhead; ++r) {
+                const int i = base + tid + r * int(blockDim.x);
+                const int64_t v = i < entry0 ? my_topk[i] : -1;
+                more[r] = v >= 0 && v < num_experts ? int(v) : -1;
+            }
             for (int k = 0; k < num_topk; ++k) {
-                const int count = __popcll(__ballot(e32 == __builtin_amdgcn_readlane(sel, k)));
+                const int e = __builtin_amdgcn_readlane(sel, k);
+                int count = 0;
+#pragma unroll
+                for (int r = 0; r < kSweepAhead; ++r) count += __popcll(__ballot(more[r] == e));
                 if (lane == k) my_count += count;
             }
         }
@@ -658,6 +667,14 @@ static int send_split_override() {
     return v;
 }
 
+static int self_rank_max_override() {
+    static const int v = [] {
+        const char* s = getenv("DEEPEP_SELF_RANK_MAX");
+        return s != nullptr ? atoi(s) : 0;
+    }();
+    return v;
+}
+
 static int send_waves_override() {
     static const int v = [] {
         const char* s = getenv("DEEPEP_SEND_WAVES");
@@ -677,7 +694,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
     const int n = num_tokens * num_topk;
     uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
-    const bool single_chunk = n <= kFusedMaxEntries;  // up to two nominal chunks are swept as one
+    const bool single_chunk = n <= (self_rank_max_override() > 0 ? self_rank_max_override() : kSelfRankMaxEntries);
     if (single_chunk) rs.num_chunks = 1;
 
     if (!single_chunk) {

@@ -332,9 +332,8 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx,
  * whose remote experts' answers are already in combine_staging when the call
  * is made (the reference: Buffer::low_latency_combine,
  * csrc/deep_ep.cpp:1798-1920; kernel phases csrc/kernels/coop_combine_send.cuh:37,
- * coop_combine_recv.cuh:72).  `out` is identical to the two calls'.  For small
- * batches (num_tokens * num_topk <= 2048 and num_experts * M <= 2^18) both
- * phases run as one kernel launch, and then the
+ * coop_combine_recv.cuh:72).  `out` is identical to the two calls'.  For
+ * num_experts * M <= 2^18 both phases run as one kernel launch, and then the
  * answers of this rank's own experts are read from x directly — the own
  * experts' part of combine_staging is neither written nor read.  Larger
  * batches launch the phases back to back. */
