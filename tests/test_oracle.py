@@ -333,7 +333,9 @@ def test_combine_closed_form_and_chain(oracle_c):
 
 
 def test_size_hint_hand_values():
-    # SURVEY hand computation for (128, 7168, 32, 256)
+    # by hand for (128, 7168, 32, 256): dmsg = 16 + max(14336, 7168 + 224) = 14352, cmsg = 224 + 14336 = 14560;
+    # send = recv = max(128 * 14352, 256 * 128 * 14560) = 477102080; sig = 1024;
+    # total = 4 * 477102080 + 2048 = 1908410368 -> (total + 128) // 128 * 128
     assert O.get_low_latency_rdma_size_hint(128, 7168, 32, 256) == 1908410496
     # tiny case by hand: M=1,H=128,E=2: dmsg=16+256=272, cmsg=4+256=260; send=max(272,520)=520; recv=max(544,520)=544
     # sig=128 -> total = 1040+1088+256 = 2384 -> (2384+128)//128*128 = 2432
