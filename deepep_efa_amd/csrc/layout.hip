@@ -138,15 +138,21 @@ __global__ __launch_bounds__(kSortChunk) void routing_sort_pass_kernel(
             chunk_table[int64_t(c) * num_ranks + r] = sum;
         }
     } else {
+        // one thread per rank turns the 16 per-wave counts into the waves' first positions
+        for (int r = tid; r < num_ranks; r += kSortChunk) {
+            int run = chunk_table[int64_t(c) * num_ranks + r];
+#pragma unroll
+            for (int w2 = 0; w2 < kSortChunk / kWave; ++w2) {
+                const int cnt = wave_cnt[w2 * num_ranks + r];
+                wave_cnt[w2 * num_ranks + r] = run;
+                run += cnt;
+            }
+        }
+        __syncthreads();
         for (int r = 0; r < num_ranks; ++r) {
             const bool in = t < num_tokens && row[r] != 0;
             const uint64_t votes = __ballot(in);
-            if (in) {
-                int pos = chunk_table[int64_t(c) * num_ranks + r];
-                for (int w2 = 0; w2 < w; ++w2) pos += wave_cnt[w2 * num_ranks + r];
-                pos += __popcll(votes & lanes_below(lane));
-                sorted_token_ids[pos] = t;
-            }
+            if (in) sorted_token_ids[wave_cnt[w * num_ranks + r] + __popcll(votes & lanes_below(lane))] = t;
         }
     }
 }
