@@ -134,6 +134,9 @@ def check_dispatch(st, want, fmt):
     (8, 5, 4200, 512, 4, 64),  # E*M > 2^18: receive runs as index kernel + flat row copy
     (8, 2, 20, 512, 4, 512),   # more than 256 segments: 16 counts per lane in the register segment table
     (16, 9, 12, 512, 6, 1024),  # the most experts the path takes
+    (1, 0, 16, 512, 2, 4),     # a world of one rank: every row is the rank's own
+    (4, 1, 12, 512, 2, 4),     # one expert per rank
+    (2, 1, 9, 512, 64, 128),   # the most selections per token
 ])
 @ONE_CALL
 def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
