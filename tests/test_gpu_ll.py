@@ -391,3 +391,31 @@ def test_empty_batch(rt, one_call):
     want = O.ll_dispatch(xs, tks, rank, e, t, O.ROW_FP8, own_last=own_last(one_call, 0, k, e, t))
     check_dispatch(st, want, O.ROW_FP8)
     assert (st.send_count == 0).all()
+
+
+def test_large_batch_without_the_segment_workspace(rt, oracle_c):
+    """E*M > 2^18 slots but no workspace for the row index: receive and row return fall back to the
+    kernels of the small-batch path and must give the same answers."""
+    r, rank, t, h, k, e = 8, 5, 4200, 512, 4, 64
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=77, drop=10)
+    shape = rt.ll.LLShape(num_ranks=r, rank=rank, num_experts=e, max_tokens=t, hidden=h, num_topk=k, fmt=O.ROW_FP8)
+    st = rt.ll.LowLatencyState(shape)
+    assert st.segment_workspace is not None
+    st.segment_workspace = None
+    world = rt.lb.LoopbackWorld(r, rank, seed=0)
+    world.set_inputs(x_all.cuda(), topk_all.cuda())
+    x, topk = world.own_inputs()
+    run_dispatch(st, world, x, topk)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
+    check_dispatch(st, want, O.ROW_FP8)
+    # identity experts: the round trip returns x * sum(w) within the FP8 error
+    count = st.packed_recv_count.cpu()
+    y = torch.zeros((e // r, r * t, h), dtype=torch.bfloat16)
+    for le in range(e // r):
+        n = int(count[le])
+        y[le, :n] = O.per_token_cast_back(st.packed_recv_x[le, :n].cpu(), st.packed_recv_scales[le, :n].cpu())
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    w = torch.softmax(w_all[rank], dim=-1)
+    run_combine(st, world, y.cuda(), topk, w.cuda(), out, mode=0)
+    wsum = w.masked_fill(topk_all[rank] == -1, 0).sum(1, keepdim=True)
+    assert O.calc_diff(x_all[rank].float() * wsum, out.cpu()) < 9e-4
