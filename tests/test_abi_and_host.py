@@ -85,3 +85,16 @@ def test_buffer_needs_a_world():
     import deep_ep
     with pytest.raises(ValueError, match="Either 'group' or 'comm' must be provided"):
         deep_ep.Buffer(None)
+
+
+def test_c_abi_library_needs_no_torch():
+    """The boundary is plain C over device pointers: the library links the HIP runtime and the C/C++
+    runtime, nothing from PyTorch, and exports no C++-mangled entry point a caller would have to use."""
+    import subprocess
+    so = os.path.join(ROOT, "deepep_efa_amd", "libdeepep_hip.so")
+    needed = subprocess.run(["readelf", "-d", so], capture_output=True, text=True, check=True).stdout
+    libs = re.findall(r"Shared library: \[([^\]]+)\]", needed)
+    assert any(lib.startswith("libamdhip64") for lib in libs)
+    assert not [lib for lib in libs if "torch" in lib or "c10" in lib or "python" in lib], libs
+    header = open(os.path.join(ROOT, "include", "deepep_hip.h")).read()
+    assert 'extern "C"' in header and "torch" not in header and "at::" not in header
