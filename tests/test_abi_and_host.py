@@ -97,4 +97,5 @@ def test_c_abi_library_needs_no_torch():
     assert any(lib.startswith("libamdhip64") for lib in libs)
     assert not [lib for lib in libs if "torch" in lib or "c10" in lib or "python" in lib], libs
     header = open(os.path.join(ROOT, "include", "deepep_hip.h")).read()
-    assert 'extern "C"' in header and "torch" not in header and "at::" not in header
+    code = re.sub(r"/\*.*?\*/", "", header, flags=re.S)  # declarations only, comments cite the reference
+    assert 'extern "C"' in code and "torch" not in code and "at::" not in code and "#include <hip" not in code
