@@ -137,6 +137,8 @@ def check_dispatch(st, want, fmt):
     (1, 0, 16, 512, 2, 4),     # a world of one rank: every row is the rank's own
     (4, 1, 12, 512, 2, 4),     # one expert per rank
     (2, 1, 9, 512, 64, 128),   # the most selections per token
+    (4, 2, 24, 1536, 4, 16),   # hidden not a multiple of 1024: the last row piece is partly empty
+    (8, 3, 17, 5120, 8, 64),
 ])
 @ONE_CALL
 def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
@@ -239,7 +241,8 @@ def test_reference_recipe_roundtrip(rt, use_fp8, one_call):
 @pytest.mark.parametrize("r,rank,t,h,k,e", [(32, 5, 128, 7168, 8, 256), (4, 0, 16, 512, 3, 8),
                                             (8, 3, 4200, 512, 4, 64),   # large-batch combine-send path
                                             (4, 2, 40, 512, 11, 64),    # more than eight selections per token
-                                            (8, 6, 20, 512, 4, 512)])   # more than 256 segments
+                                            (8, 6, 20, 512, 4, 512),    # more than 256 segments
+                                            (4, 1, 33, 1536, 5, 32)])   # hidden not a multiple of 512
 @ONE_CALL
 def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e, one_call):
     """Seeded expert outputs along the dispatch routing; combine vs the float32 chain and the float64 sum."""
