@@ -422,3 +422,83 @@ def test_large_batch_without_the_segment_workspace(rt, oracle_c):
     run_combine(st, world, y.cuda(), topk, w.cuda(), out, mode=0)
     wsum = w.masked_fill(topk_all[rank] == -1, 0).sum(1, keepdim=True)
     assert O.calc_diff(x_all[rank].float() * wsum, out.cpu()) < 9e-4
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
+def test_every_rank_on_one_gpu_with_a_real_exchange(rt, fmt):
+    """All R ranks run on the one GPU, each with its own buffers, and the exchange between them is a
+    plain copy of what the send sides produced (send_slots -> the peer's recv_staging, then
+    combine_send_slots -> the peer's combine_staging).  Nothing is synthesised "in a peer's name":
+    this is the data flow of a multi-GPU run with the transport replaced by device copies."""
+    r, t, h, k, e = 4, 12, 512, 3, 16
+    epr = e // r
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=123, drop=4)
+    states = []
+    for rank in range(r):
+        st = rt.ll.LowLatencyState(rt.ll.LLShape(r, rank, e, t, h, k, fmt))
+        st.recv_count.zero_()
+        st.dispatch_send(x_all[rank].cuda(), topk_all[rank].cuda())
+        states.append(st)
+    torch.cuda.synchronize()
+    # the dispatch exchange: rank s's rows for expert e travel to the rank that owns e
+    for s in range(r):
+        src = states[s]
+        slots = src.send_slots.view(e, t, src.stride)
+        counts = src.send_count.cpu()
+        for ex in range(e):
+            dst_rank, le = ex // epr, ex % epr
+            if dst_rank == s:
+                continue
+            cnt = int(counts[ex])
+            dst = states[dst_rank]
+            dst.recv_staging.view(epr, r, t, dst.stride)[le, s, :cnt] = slots[ex, :cnt]
+            dst.recv_count.view(epr, r)[le, s] = cnt
+    outs = []
+    for rank in range(r):
+        st = states[rank]
+        poison_outputs_keep_pair_slot(st)
+        st.dispatch_recv()
+        torch.cuda.synchronize()
+        want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
+        check_dispatch(st, want, fmt)
+        # identity experts
+        if fmt == O.ROW_BF16:
+            y = st.packed_recv_x.clone()
+        else:
+            q = st.packed_recv_x.float().view(epr, r * t, h // 128, 128)
+            y = (q * st.packed_recv_scales.unsqueeze(-1)).view(epr, r * t, h).to(torch.bfloat16)
+        y = torch.nan_to_num(y, nan=0.0, posinf=0.0, neginf=0.0)  # rows past the counts hold poison
+        st.combine_send(y)
+        outs.append(y)
+    torch.cuda.synchronize()
+    # the combine exchange: what rank q returns for rank s's pairs goes to s's staging for q's experts
+    for q in range(r):
+        src = states[q]
+        back = src.combine_send_slots  # [E_l, R, M, H]
+        lr = src.packed_recv_layout_range.cpu()
+        for le in range(epr):
+            for s in range(r):
+                if s == q:
+                    continue
+                cnt = int(lr[le, s] & 0xFFFFFFFF)
+                states[s].combine_staging[q * epr + le, :cnt] = back[le, s, :cnt]
+    for rank in range(r):
+        st = states[rank]
+        out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+        out.view(torch.int16).fill_(0x7FC0)
+        topk, w = topk_all[rank].cuda(), w_all[rank].cuda()
+        st.combine_recv(topk, w, out)
+        torch.cuda.synchronize()
+        wsum = w_all[rank].masked_fill(topk_all[rank] == -1, 0).sum(1, keepdim=True)
+        diff = O.calc_diff(x_all[rank].float() * wsum, out.cpu())
+        assert not torch.isnan(out.float()).any()
+        assert diff < (9e-4 if fmt != O.ROW_BF16 else 1e-5), (rank, diff)
+
+
+def poison_outputs_keep_pair_slot(st):
+    st.packed_recv_x.view(torch.uint8).fill_(0xEE)
+    if st.packed_recv_scales is not None:
+        st.packed_recv_scales.view(torch.uint8).fill_(0xEE)
+    st.packed_recv_src_info.fill_(-7)
+    st.packed_recv_count.fill_(-7)
+    st.packed_recv_layout_range.fill_(-7)
