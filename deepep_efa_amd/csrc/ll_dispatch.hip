@@ -22,23 +22,47 @@
 
 namespace deepep {
 
-constexpr int kRouteChunk = 1024;  // (token,k) entries ranked by one workgroup
-
 __host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
 
-struct RouteScratch {
-    int num_chunks;  // 1024-entry chunks of the (token,k) list
-    int64_t bytes;   // per source: slot of every (token,k) entry, int32 [T*K]
-};
+constexpr int kSweepChunkEntries = 2048;  // a token sweeps at most this many earlier entries itself
 
-static RouteScratch route_scratch(int num_tokens, int num_topk, int num_experts) {
-    (void)num_experts;
-    RouteScratch s;
-    const int64_t n = int64_t(num_tokens) * num_topk;
-    s.num_chunks = int((n + kRouteChunk - 1) / kRouteChunk);
-    if (s.num_chunks < 1) s.num_chunks = 1;
-    s.bytes = align256(n * 4 + 4);
-    return s;
+// Tokens per sweep chunk: whole tokens, about kSweepChunkEntries entries.
+inline int sweep_chunk_tokens(int num_topk) {
+    const int t = kSweepChunkEntries / num_topk;
+    return t < 1 ? 1 : t;
+}
+
+// Per source: the chunk histograms, int32 [chunks][E].
+static int64_t route_scratch_bytes(int num_tokens, int num_topk, int num_experts) {
+    const int tpc = sweep_chunk_tokens(num_topk);
+    const int64_t chunks = (num_tokens + tpc - 1) / tpc;
+    return align256((chunks < 1 ? 1 : chunks) * num_experts * 4);
+}
+
+// ---------------------------------------------------------------------
+// Per-chunk expert histograms for medium and large batches: workgroup c counts the
+// entries of tokens [c * tpc, (c + 1) * tpc) per expert.  The send kernel then
+// ranks a pair as (entries of earlier chunks naming its expert, summed from these
+// rows) + (earlier entries of its own chunk, which it sweeps itself).
+// ---------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void ll_chunk_hist_kernel(const int64_t* __restrict__ topk_idx, int n,
+                                                             int entries_per_chunk, int num_experts,
+                                                             int64_t scratch_stride,
+                                                             uint8_t* __restrict__ scratch_base) {
+    extern __shared__ int32_t hist_lds[];  // [E]
+    const int c = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int64_t* my_topk = topk_idx + int64_t(b) * n;
+    int32_t* out = reinterpret_cast<int32_t*>(scratch_base + int64_t(b) * scratch_stride) + int64_t(c) * num_experts;
+    for (int e = tid; e < num_experts; e += blockDim.x) hist_lds[e] = 0;
+    lds_barrier();
+    const int begin = c * entries_per_chunk;
+    const int end = begin + entries_per_chunk < n ? begin + entries_per_chunk : n;
+    for (int i = begin + tid; i < end; i += blockDim.x) {
+        const int64_t v = my_topk[i];
+        if (v >= 0 && v < num_experts) atomicAdd(&hist_lds[int(v)], 1);
+    }
+    lds_barrier();
+    for (int e = tid; e < num_experts; e += blockDim.x) out[e] = hist_lds[e];
 }
 
 // Writes the per-expert totals where the receivers look for them.
@@ -49,113 +73,6 @@ __device__ __forceinline__ void emit_expert_count(int e, int total, int num_expe
     const int experts_per_rank = num_experts / num_ranks;
     if (send_count != nullptr) send_count[e] = cnt;
     if (e / experts_per_rank == rank) recv_count[(e % experts_per_rank) * num_ranks + src_rank] = cnt;
-}
-
-// ---------------------------------------------------------------------
-// Slot ranking for batches of more than one chunk, in one launch.  Entry
-// i = t*K + k lives in chunk i / 1024; workgroup c owns chunk c and writes the
-// final slot of each of its entries:
-//   base  — entries of earlier chunks naming the same expert: the workgroup
-//           re-reads them (L2-resident, at most T*K*8 bytes) into an LDS
-//           histogram, so no workgroup waits on another;
-//   rank  — earlier entries of the same chunk: in-wave by 64-lane ballots (one
-//           ballot per distinct expert present in the wave), across the 16 waves
-//           by a 16 x E table in LDS.
-// The last chunk's workgroup also publishes the per-expert totals.
-// Deterministic: integer adds and ballots only.
-// Reference semantics: the serial (token,k) scan of
-// csrc/kernels/efa_kernels.cu:617-637 and token_offset / expert_offsets of
-// csrc/kernels/coop_dispatch_send.cuh:360-420.
-// ---------------------------------------------------------------------
-constexpr int kRouteWaves = kRouteChunk / kWave;
-
-__global__ __launch_bounds__(kRouteChunk) void ll_route_slots_kernel(
-    const int64_t* __restrict__ topk_idx, int n, int num_experts, int num_ranks, int rank,
-    const int32_t* __restrict__ src_ranks, int max_tokens, int64_t scratch_stride,
-    uint8_t* __restrict__ scratch_base, int32_t* __restrict__ recv_count, int32_t* __restrict__ send_count) {
-    extern __shared__ int32_t route_lds[];
-    int32_t* base_hist = route_lds;               // [E] entries of earlier chunks
-    int32_t* wave_hist = route_lds + num_experts;  // [kRouteWaves][E]
-    const int b = blockIdx.y, c = blockIdx.x;
-    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
-    const int64_t* my_topk = topk_idx + int64_t(b) * n;
-    int32_t* slots = reinterpret_cast<int32_t*>(scratch_base + int64_t(b) * scratch_stride);
-
-    for (int j = tid; j < (kRouteWaves + 1) * num_experts; j += kRouteChunk) route_lds[j] = 0;
-    const int i = c * kRouteChunk + tid;
-    int e = -1;
-    if (i < n) {
-        const int64_t v = my_topk[i];
-        if (v >= 0 && v < num_experts) e = int(v);
-    }
-    __syncthreads();
-
-    // base: histogram of every earlier chunk.  Two entries per 16-byte load, sixteen loads in flight
-    // per thread: one round of memory latency covers 32 chunks.
-    const int before = c * kRouteChunk;  // a multiple of 1024, so pairs never straddle it
-    if ((reinterpret_cast<uintptr_t>(my_topk) & 15) == 0) {
-        const u32x4* pairs = reinterpret_cast<const u32x4*>(my_topk);
-        const int num_pairs = before >> 1;
-        for (int p0 = tid; p0 < num_pairs; p0 += kRouteChunk * 16) {
-            u32x4 v[16];
-#pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                const int p = p0 + u * kRouteChunk;
-                if (p < num_pairs) v[u] = pairs[p];
-            }
-#pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                if (p0 + u * kRouteChunk >= num_pairs) continue;
-                // an int64 entry is valid when its high word is zero and its low word is below E
-                if (v[u][1] == 0 && v[u][0] < uint32_t(num_experts)) atomicAdd(&base_hist[v[u][0]], 1);
-                if (v[u][3] == 0 && v[u][2] < uint32_t(num_experts)) atomicAdd(&base_hist[v[u][2]], 1);
-            }
-        }
-    } else {
-        for (int i0 = tid; i0 < before; i0 += kRouteChunk * 8) {
-            int64_t v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int j = i0 + u * kRouteChunk;
-                v[u] = j < before ? my_topk[j] : -1;
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (v[u] >= 0 && v[u] < num_experts) atomicAdd(&base_hist[int(v[u])], 1);
-        }
-    }
-
-    // rank inside the wave
-    uint64_t pending = __ballot(e >= 0);
-    int my_rank = 0, my_count = 0;
-    while (pending != 0) {
-        const int leader = __builtin_ctzll(pending);
-        const int e0 = __builtin_amdgcn_readlane(e, leader);
-        const uint64_t same = __ballot(e == e0);
-        if (e == e0) {
-            my_rank = __popcll(same & lanes_below(lane));
-            my_count = __popcll(same);
-        }
-        pending &= ~same;
-    }
-    if (e >= 0 && my_rank == 0) wave_hist[w * num_experts + e] = my_count;
-    __syncthreads();
-    // exclusive scan over the 16 waves, one thread per expert
-    const bool last_chunk = c == int(gridDim.x) - 1;
-    const int src_rank = src_ranks != nullptr ? src_ranks[b] : rank;
-    for (int x = tid; x < num_experts; x += kRouteChunk) {
-        int run = base_hist[x];
-#pragma unroll
-        for (int w2 = 0; w2 < kRouteWaves; ++w2) {
-            const int cnt = wave_hist[w2 * num_experts + x];
-            wave_hist[w2 * num_experts + x] = run;
-            run += cnt;
-        }
-        if (last_chunk)
-            emit_expert_count(x, run, num_experts, num_ranks, rank, src_rank, max_tokens, recv_count, send_count);
-    }
-    __syncthreads();
-    if (i < n) slots[i] = e >= 0 ? wave_hist[w * num_experts + e] + my_rank : -1;
 }
 
 // ---------------------------------------------------------------------
@@ -174,17 +91,21 @@ __global__ __launch_bounds__(kRouteChunk) void ll_route_slots_kernel(
 // while wave 0 does that.  Barriers fence LDS only, so the row loads stay in
 // flight across them.
 //
-// A batch of up to 8192 (token,k) entries needs no route kernel: while the row loads are
-// in flight every thread fetches up to four (token,k) entries that precede the
-// token (more in a loop for workgroups under 512 threads); each wave counts, per
-// selection, its entries naming that selection's expert with a ballot and a
-// popcount, and wave 0 adds the waves' counts.  The per-expert totals come from
-// one extra workgroup per source, an LDS histogram.  Larger batches read the
-// slots ranked by ll_route_slots_kernel.
+// The slot of a selection is the number of earlier (token,k) entries naming its
+// expert (reference: the serial scan of csrc/kernels/efa_kernels.cu:617-637 and
+// token_offset / expert_offsets of csrc/kernels/coop_dispatch_send.cuh:360-420).
+// The workgroup counts them itself: while the row loads are in flight every
+// thread fetches up to four entries that precede the token (more in a loop);
+// each wave counts, per selection, its entries naming that selection's expert
+// with a ballot and a popcount, and wave 0 adds the waves' counts.  Up to 8192
+// entries the sweep covers every earlier entry; beyond, it covers the token's
+// own chunk of about 2048 entries and the chunks before it come from the
+// histograms of ll_chunk_hist_kernel.  The per-expert totals come from one extra
+// workgroup per source.  Deterministic: integer adds and ballots only.
 // ---------------------------------------------------------------------
 constexpr int kMaxTopk = 64;
 constexpr int kFusedMaxEntries = 2048;     // send + receive in one launch up to here
-constexpr int kSelfRankMaxEntries = 8192;  // the send kernel ranks its own slots up to here
+constexpr int kSelfRankMaxEntries = 8192;  // the send kernel ranks its own slots, unaided, up to here
 constexpr int kSendMaxWaves = 16;
 
 struct SendArgs {
@@ -194,7 +115,7 @@ struct SendArgs {
     int num_tokens, hidden, num_topk, num_experts, num_ranks, rank, max_tokens;
     int pieces_per_row, split_log2;
     uint32_t rank_of_expert_magic;
-    int num_chunks;
+    int tokens_per_chunk;  // > 0: scratch holds the per-chunk expert histograms of ll_chunk_hist_kernel
     int64_t scratch_stride;
     const uint8_t* scratch_base;
     uint8_t* recv_staging;
@@ -219,12 +140,23 @@ struct alignas(16) SendLds {
     uint64_t sel_scale[kMaxTopk];                 // where its scales go
 };
 
-// The per-source counting workgroup of a single-chunk batch.
+// The per-source counting workgroup.
 __device__ __forceinline__ void send_count_block(const SendArgs& a, int b, int32_t* lds_hist) {
     const int tid = threadIdx.x;
     const int n = a.num_tokens * a.num_topk;
     const int src_rank = a.src_ranks != nullptr ? a.src_ranks[b] : a.rank;
     const int64_t* my_topk = a.topk_idx + int64_t(b) * n;
+    if (a.tokens_per_chunk > 0) {  // the totals are the column sums of the chunk histograms
+        const int32_t* hist = reinterpret_cast<const int32_t*>(a.scratch_base + int64_t(b) * a.scratch_stride);
+        const int chunks = (a.num_tokens + a.tokens_per_chunk - 1) / a.tokens_per_chunk;
+        for (int e = tid; e < a.num_experts; e += blockDim.x) {
+            int total = 0;
+            for (int c = 0; c < chunks; ++c) total += hist[int64_t(c) * a.num_experts + e];
+            emit_expert_count(e, total, a.num_experts, a.num_ranks, a.rank, src_rank, a.max_tokens, a.recv_count,
+                              a.send_count);
+        }
+        return;
+    }
     for (int j = tid; j < a.num_experts; j += blockDim.x) lds_hist[j] = 0;
     lds_barrier();
     for (int i = tid; i < n; i += blockDim.x) {
@@ -311,78 +243,89 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             if (lane == k) direct_begin = sum;
         }
     }
+    // Medium and large batches: the token sweeps only the earlier entries of its own chunk; what the
+    // chunks before it hold of each selection's expert comes from their histograms.
+    const int chunk = a.tokens_per_chunk > 0 ? t / a.tokens_per_chunk : 0;
+    const int sweep_begin = chunk * a.tokens_per_chunk * num_topk;
+    int chunk_base = 0;
+    if (chunk > 0 && tid < num_topk && my_expert >= 0) {
+        const int32_t* hist = reinterpret_cast<const int32_t*>(a.scratch_base + int64_t(b) * a.scratch_stride);
+        for (int c0 = 0; c0 < chunk; c0 += 8) {  // eight loads in flight
+            int c[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) c[u] = c0 + u < chunk ? hist[int64_t(c0 + u) * num_experts + my_expert] : 0;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) chunk_base += c[u];
+        }
+    }
     DEEPEP_PHASE(1);
     u32x4 payload = lo;  // quantised below, while the workgroup's bookkeeping is in flight
     uint32_t scale_bits = 0;
-    if (a.num_chunks > 1) {  // slots were ranked by ll_route_slots_kernel
-        if (tid < num_topk && my_expert >= 0)
-            my_slot = reinterpret_cast<const int32_t*>(a.scratch_base + int64_t(b) * a.scratch_stride)[entry0 + tid];
-        if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
-    } else {
-        // Small batch: rank here.  Each thread takes every blockDim-th entry before this token (four of
-        // them fetched up front, so their latency overlaps the loads above); each wave counts, per
-        // selection, how many of its entries name that selection's expert (a ballot and a popcount,
-        // against the token's own entries read as wave-uniform values) and leaves the counts in LDS.
-        constexpr int kSweepAhead = 4;
-        int ahead[kSweepAhead];  // -1: no entry
+    // Rank the selections.  Each thread takes every blockDim-th entry between the start of the sweep
+    // and this token (four fetched up front, so their latency overlaps the loads above); each wave
+    // counts, per selection, how many of its entries name that selection's expert (a ballot and a
+    // popcount, against the token's own entries read as wave-uniform values) and leaves the counts
+    // in LDS.
+    constexpr int kSweepAhead = 4;
+    int ahead[kSweepAhead];  // -1: no entry
+#pragma unroll
+    for (int r = 0; r < kSweepAhead; ++r) {
+        const int i = sweep_begin + tid + r * int(blockDim.x);
+        const int64_t v = i < entry0 ? my_topk[i] : -1;
+        ahead[r] = v >= 0 && v < num_experts ? int(v) : -1;
+    }
+    // lane k of every wave holds the token's selection k (-2: none, matches no entry)
+    int sel = -2;
+    if (lane < num_topk) {
+        const int64_t v = my_topk[entry0 + lane];
+        if (v >= 0 && v < num_experts) sel = int(v);
+    }
+    const int w = wave_in_block();
+    int my_count = 0;  // lane k: this wave's entries naming selection k's expert
+    for (int k = 0; k < num_topk; ++k) {
+        const int e = __builtin_amdgcn_readlane(sel, k);
+        int count = 0;
+#pragma unroll
+        for (int r = 0; r < kSweepAhead; ++r) count += __popcll(__ballot(ahead[r] == e));
+        if (lane == k) my_count = count;
+    }
+    for (int base = sweep_begin + kSweepAhead * int(blockDim.x); base < entry0;
+         base += kSweepAhead * int(blockDim.x)) {
+        int more[kSweepAhead];  // the same again, four loads in flight per thread
 #pragma unroll
         for (int r = 0; r < kSweepAhead; ++r) {
-            const int i = tid + r * int(blockDim.x);
+            const int i = base + tid + r * int(blockDim.x);
             const int64_t v = i < entry0 ? my_topk[i] : -1;
-            ahead[r] = v >= 0 && v < num_experts ? int(v) : -1;
+            more[r] = v >= 0 && v < num_experts ? int(v) : -1;
         }
-        // lane k of every wave holds the token's selection k (-2: none, matches no entry)
-        int sel = -2;
-        if (lane < num_topk) {
-            const int64_t v = my_topk[entry0 + lane];
-            if (v >= 0 && v < num_experts) sel = int(v);
-        }
-        const int w = wave_in_block();
-        int my_count = 0;  // lane k: this wave's entries naming selection k's expert
         for (int k = 0; k < num_topk; ++k) {
             const int e = __builtin_amdgcn_readlane(sel, k);
             int count = 0;
 #pragma unroll
-            for (int r = 0; r < kSweepAhead; ++r) count += __popcll(__ballot(ahead[r] == e));
-            if (lane == k) my_count = count;
+            for (int r = 0; r < kSweepAhead; ++r) count += __popcll(__ballot(more[r] == e));
+            if (lane == k) my_count += count;
         }
-        for (int base = kSweepAhead * int(blockDim.x); base < entry0; base += kSweepAhead * int(blockDim.x)) {
-            int more[kSweepAhead];  // the same again, four loads in flight per thread
+    }
+    if (lane < num_topk) lds.wave_count[lane][w] = my_count;
+    if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
+    lds_barrier();
+    DEEPEP_PHASE(3);
+    if (tid < kWave) {  // wave 0: lane k finishes selection k
+        const int waves = int(blockDim.x) >> 6;
+        int total = 0;
+        if (tid < num_topk) {  // one wide read of the row; entries of absent waves are never summed
+            static_assert(kSendMaxWaves == 16, "four 16-byte LDS reads");
+            u32x4 c[4];
 #pragma unroll
-            for (int r = 0; r < kSweepAhead; ++r) {
-                const int i = base + tid + r * int(blockDim.x);
-                const int64_t v = i < entry0 ? my_topk[i] : -1;
-                more[r] = v >= 0 && v < num_experts ? int(v) : -1;
-            }
-            for (int k = 0; k < num_topk; ++k) {
-                const int e = __builtin_amdgcn_readlane(sel, k);
-                int count = 0;
+            for (int q = 0; q < 4; ++q) c[q] = reinterpret_cast<const u32x4*>(lds.wave_count[tid])[q];
 #pragma unroll
-                for (int r = 0; r < kSweepAhead; ++r) count += __popcll(__ballot(more[r] == e));
-                if (lane == k) my_count += count;
-            }
+            for (int w2 = 0; w2 < kSendMaxWaves; ++w2) total += w2 < waves ? int(c[w2 >> 2][w2 & 3]) : 0;
         }
-        if (lane < num_topk) lds.wave_count[lane][w] = my_count;
-        if constexpr (kFmt != kRowBF16) payload = quantise_16<kFmt>(lo, hi, scale_bits);
-        lds_barrier();
-        DEEPEP_PHASE(3);
-        if (tid < kWave) {  // wave 0: lane k finishes selection k
-            const int waves = int(blockDim.x) >> 6;
-            int total = 0;
-            if (tid < num_topk) {  // one wide read of the row; entries of absent waves are never summed
-                static_assert(kSendMaxWaves == 16, "four 16-byte LDS reads");
-                u32x4 c[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) c[q] = reinterpret_cast<const u32x4*>(lds.wave_count[tid])[q];
-#pragma unroll
-                for (int w2 = 0; w2 < kSendMaxWaves; ++w2) total += w2 < waves ? int(c[w2 >> 2][w2 & 3]) : 0;
-            }
-            for (int k2 = 0; k2 < num_topk; ++k2) {  // the same expert named earlier in this token
-                const int other = __builtin_amdgcn_readlane(my_expert, k2);
-                if (k2 < tid && other == my_expert) total += 1;
-            }
-            if (tid < num_topk && my_expert >= 0) my_slot = total;
+        for (int k2 = 0; k2 < num_topk; ++k2) {  // the same expert named earlier in this token
+            const int other = __builtin_amdgcn_readlane(my_expert, k2);
+            if (k2 < tid && other == my_expert) total += 1;
         }
+        if (tid < num_topk && my_expert >= 0) my_slot = total + chunk_base;
     }
     if (tid < num_topk) {
         if (my_slot >= a.max_tokens) my_slot = -1;
@@ -451,7 +394,7 @@ template <int kFmt>
 __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs a) {
     extern __shared__ int32_t lds_hist[];  // [E], counting workgroups only
     __shared__ SendLds lds;
-    if (int(blockIdx.y) == a.num_tokens) {  // the counting row of the grid (single-chunk batches)
+    if (int(blockIdx.y) == a.num_tokens) {  // the counting row of the grid
         if (blockIdx.x == 0) send_count_block(a, blockIdx.z, lds_hist);
         return;
     }
@@ -689,19 +632,19 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
                             void* send_slots, int32_t* send_count, int32_t* pair_slot, void* workspace,
                             size_t workspace_bytes, hipStream_t stream, const RecvArgs* fused_recv = nullptr,
                             int64_t fused_recv_wave_items = 0) {
-    RouteScratch rs = route_scratch(num_tokens, num_topk, num_experts);
-    EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(rs.bytes) * size_t(num_src));
+    const int64_t scratch_bytes = route_scratch_bytes(num_tokens, num_topk, num_experts);
+    EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(scratch_bytes) * size_t(num_src));
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
     const int n = num_tokens * num_topk;
     uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
-    const bool single_chunk = n <= (self_rank_max_override() > 0 ? self_rank_max_override() : kSelfRankMaxEntries);
-    if (single_chunk) rs.num_chunks = 1;
-
-    if (!single_chunk) {
-        const size_t lds = size_t(kRouteWaves + 1) * num_experts * sizeof(int32_t);
-        EP_HOST_ASSERT(lds <= 64 * 1024);
-        ll_route_slots_kernel<<<dim3(rs.num_chunks, num_src), kRouteChunk, lds, stream>>>(
-            topk_idx, n, num_experts, num_ranks, rank, src_ranks, max_tokens, rs.bytes, ws, recv_count, send_count);
+    // How slots get ranked: up to kSelfRankMaxEntries entries the send kernel sweeps every earlier
+    // entry itself; beyond, it sweeps its own chunk on top of the per-chunk histograms.
+    const int self_rank_max = self_rank_max_override() > 0 ? self_rank_max_override() : kSelfRankMaxEntries;
+    const int tpc = n <= self_rank_max ? 0 : sweep_chunk_tokens(num_topk);
+    if (tpc > 0) {
+        const int chunks = (num_tokens + tpc - 1) / tpc;
+        ll_chunk_hist_kernel<<<dim3(chunks, num_src), 1024, size_t(num_experts) * sizeof(int32_t), stream>>>(
+            topk_idx, n, tpc * num_topk, num_experts, scratch_bytes, ws);
         EP_LAUNCH_CHECK();
     }
 
@@ -736,13 +679,14 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     sa.num_ranks = num_ranks, sa.rank = rank, sa.max_tokens = max_tokens;
     sa.pieces_per_row = pieces, sa.split_log2 = split_log2;
     sa.rank_of_expert_magic = magic;
-    sa.num_chunks = rs.num_chunks, sa.scratch_stride = rs.bytes, sa.scratch_base = ws;
+    sa.scratch_stride = scratch_bytes, sa.scratch_base = ws;
+    sa.tokens_per_chunk = tpc;
     sa.recv_staging = reinterpret_cast<uint8_t*>(recv_staging);
     sa.send_slots = reinterpret_cast<uint8_t*>(send_slots);
     sa.pair_slot = pair_slot, sa.recv_count = recv_count, sa.send_count = send_count;
 
     if (fused_recv != nullptr) {  // single launch: send workgroups, the counting workgroup, receive workgroups
-        EP_HOST_ASSERT(single_chunk && num_src == 1 && src_ranks == nullptr);
+        EP_HOST_ASSERT(tpc == 0 && num_src == 1 && src_ranks == nullptr);
         const int num_send_blocks = blocks_per_token * num_tokens;
         int64_t fused_recv_blocks = (fused_recv_wave_items + waves - 1) / waves;
         fused_recv_blocks = fused_recv_blocks < 1 ? 1 : (fused_recv_blocks > 1024 ? 1024 : fused_recv_blocks);
@@ -767,9 +711,8 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
         return 0;
     }
 
-    const dim3 grid(blocks_per_token, num_tokens + (single_chunk ? 1 : 0), num_src);
-    if (grid.y == 0) return 0;
-    const size_t lds = single_chunk ? size_t(num_experts) * sizeof(int32_t) : 0;
+    const dim3 grid(blocks_per_token, num_tokens + 1, num_src);  // + the counting workgroup
+    const size_t lds = size_t(num_experts) * sizeof(int32_t);
 #define DEEPEP_LAUNCH_SEND(FMT) ll_send_kernel<FMT><<<grid, waves * kWave, lds, stream>>>(sa)
     switch (row_format) {
         case kRowBF16: DEEPEP_LAUNCH_SEND(kRowBF16); break;
@@ -797,7 +740,7 @@ size_t deepep_ll_segment_workspace_bytes(int num_experts, int num_max_dispatch_t
 }
 
 size_t deepep_ll_dispatch_workspace_bytes(int num_tokens, int num_topk, int num_experts) {
-    return size_t(route_scratch(num_tokens, num_topk, num_experts).bytes);
+    return size_t(route_scratch_bytes(num_tokens, num_topk, num_experts));
 }
 
 int deepep_ll_dispatch_send(const void* x, const int64_t* topk_idx, int num_tokens, int hidden, int num_topk,

@@ -127,10 +127,10 @@ def check_dispatch(st, want, fmt):
 @pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16, O.ROW_FP8_POW2, O.ROW_FP8_UE8M0])
 @pytest.mark.parametrize("r,rank,t,h,k,e", [
     (4, 1, 8, 512, 3, 16), (8, 7, 33, 1024, 4, 64), (2, 0, 1, 512, 1, 2),
-    (4, 1, 40, 512, 9, 64),    # K > 8: separate route kernel, one chunk
-    (2, 1, 600, 512, 8, 16),   # T*K > 2048: two launches, the send kernel still ranks its own slots
+    (4, 1, 40, 512, 9, 64),    # K > 8
+    (2, 1, 600, 512, 8, 16),   # T*K > 2048: two launches, the send kernel sweeps every earlier entry
     (4, 3, 300, 512, 11, 32),  # both
-    (2, 0, 1100, 512, 8, 16),  # T*K > 8192: slots ranked by the route kernel, small receive path
+    (2, 0, 1100, 512, 8, 16),  # T*K > 8192: chunk histograms under the send kernel's sweep, small receive path
     (8, 5, 4200, 512, 4, 64),  # E*M > 2^18: receive runs as index kernel + flat row copy
     (8, 2, 20, 512, 4, 512),   # more than 256 segments: 16 counts per lane in the register segment table
     (16, 9, 12, 512, 6, 1024),  # the most experts the path takes
