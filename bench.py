@@ -338,6 +338,32 @@ def main():
         torch.cuda.synchronize()
         return ev0.elapsed_time(ev1) * 1e3 / reps, per_graph
 
+    def time_cold(fn, reps=40):
+        """One call at a time, each after 512 MiB of fresh writes have pushed the step's data out of
+        the 256 MB last-level cache; the call is a one-step HIP graph (so that its launches are queued
+        while the flush still runs) between its own pair of events.  Median over `reps`."""
+        flush = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+        launch = fn
+        if not args.no_graph:
+            try:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    fn()
+                launch = g.replay
+            except Exception:
+                launch = fn
+        samples = []
+        for i in range(reps + 3):
+            flush.fill_(i & 0xFF)
+            ev0.record()
+            launch()
+            ev1.record()
+            torch.cuda.synchronize()
+            if i >= 3:
+                samples.append(ev0.elapsed_time(ev1) * 1e3)
+        samples.sort()
+        return samples[len(samples) // 2]
+
     eager_us, host_wall_us = time_eager(step, args.warmup, args.steps)
     eager_phase_us, _ = time_eager(step_by_phase, 10, args.steps)
     graph_us = graph_phase_us = per_graph = None
@@ -357,6 +383,9 @@ def main():
         # the same call `steps` times back to back between two events
         for name, fn in calls.items():
             per_call[name], _ = time_eager(fn, 10, args.steps)
+    cold_us = time_cold(step)
+    tiny = torch.zeros(64, dtype=torch.int32, device="cuda")
+    cold_floor_us = time_cold(lambda: (tiny.add_(1), tiny.add_(1)))  # two trivial launches, timed the same way
     us_per_step = graph_us if graph_us is not None else eager_us
     us_per_phase_step = graph_phase_us if graph_phase_us is not None else eager_phase_us
 
@@ -388,6 +417,8 @@ def main():
         "timing": timing,
         "eager_us_per_step": round(eager_us, 2),  # launched call by call from Python: host-bound
         "eager_host_wall_us_per_step": round(host_wall_us, 2),
+        "cold_cache_us_per_step": round(cold_us, 2),  # every step after a 512 MiB flush of the last-level cache
+        "cold_cache_two_trivial_launches_us": round(cold_floor_us, 2),  # what that way of timing costs by itself
         "kernels": kernels,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
