@@ -338,11 +338,15 @@ def main():
         torch.cuda.synchronize()
         return ev0.elapsed_time(ev1) * 1e3 / reps, per_graph
 
-    def time_cold(fn, reps=40):
-        """One call at a time, each after 512 MiB of fresh writes have pushed the step's data out of
+    flush = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
+
+    def time_cold(fn, reps=40, by_reads=False):
+        """One call at a time, each after 512 MiB of other traffic has pushed the step's data out of
         the 256 MB last-level cache; the call is a one-step HIP graph (so that its launches are queued
-        while the flush still runs) between its own pair of events.  Median over `reps`."""
-        flush = torch.empty(512 << 20, dtype=torch.uint8, device="cuda")
+        while the flush still runs) between its own pair of events.  Median over `reps`.
+        The flush writes the 512 MiB (what the reference's bench does before each timed call: the
+        caches are then full of lines that must be written back first) or, `by_reads`, reads them
+        (the caches are left full of clean lines, as after a GEMM over expert weights)."""
         launch = fn
         if not args.no_graph:
             try:
@@ -354,7 +358,10 @@ def main():
                 launch = fn
         samples = []
         for i in range(reps + 3):
-            flush.fill_(i & 0xFF)
+            if by_reads:
+                flush.max()
+            else:
+                flush.fill_(i)
             ev0.record()
             launch()
             ev1.record()
@@ -386,6 +393,8 @@ def main():
     cold_us = time_cold(step)
     tiny = torch.zeros(64, dtype=torch.int32, device="cuda")
     cold_floor_us = time_cold(lambda: (tiny.add_(1), tiny.add_(1)))  # two trivial launches, timed the same way
+    cold_reads_us = time_cold(step, by_reads=True)
+    cold_reads_floor_us = time_cold(lambda: (tiny.add_(1), tiny.add_(1)), by_reads=True)
     us_per_step = graph_us if graph_us is not None else eager_us
     us_per_phase_step = graph_phase_us if graph_phase_us is not None else eager_phase_us
 
@@ -419,6 +428,8 @@ def main():
         "eager_host_wall_us_per_step": round(host_wall_us, 2),
         "cold_cache_us_per_step": round(cold_us, 2),  # every step after a 512 MiB flush of the last-level cache
         "cold_cache_two_trivial_launches_us": round(cold_floor_us, 2),  # what that way of timing costs by itself
+        "cold_cache_read_flush_us_per_step": round(cold_reads_us, 2),  # the same after 512 MiB of reads
+        "cold_cache_read_flush_two_trivial_launches_us": round(cold_reads_floor_us, 2),
         "kernels": kernels,
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
