@@ -151,6 +151,55 @@ def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
     assert torch.equal(st.pair_slot[:t].cpu(), pair_slot)
 
 
+def _random_shape(seed):
+    g = np.random.default_rng(seed)
+    r = int(g.choice([1, 2, 3, 4, 5, 6, 8, 12, 16, 24]))
+    epr = int(g.choice([1, 2, 3, 5, 8, 16]))
+    e = r * epr
+    k = int(g.integers(1, min(e, 12) + 1))
+    t = int(g.choice([1, 2, 7, 31, 64, 100, 129, 257, 300, 1100]))
+    m = t + int(g.choice([0, 0, 1, 13, 64]))  # room for more tokens than the batch holds
+    h = int(g.choice([128, 256, 384, 640, 1024, 2048, 2176]))
+    fmt = int(g.choice([O.ROW_FP8, O.ROW_BF16, O.ROW_FP8_POW2]))
+    return r, int(g.integers(0, r)), t, m, h, k, e, fmt, int(g.integers(0, min(40, t * k) + 1))
+
+
+@pytest.mark.parametrize("seed", range(24))
+@ONE_CALL
+def test_dispatch_and_combine_seeded_random_shapes(rt, seed, one_call):
+    """Shapes nobody picked by hand: odd world sizes, hidden sizes with a ragged last piece, more slots
+    than tokens, many or no dropped selections.  Dispatch bit-exact, combine against the float32 chain."""
+    r, rank, t, m, h, k, e, fmt, drop = _random_shape(seed)
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=1000 + seed, drop=drop)
+    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, m, fmt, one_call=one_call)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, fmt, own_last=own_last(one_call, t, k, e, m))
+    check_dispatch(st, want, fmt)
+    send_count, pair_slot = O.route(topk_all[rank], e, m)
+    assert torch.equal(st.send_count.cpu(), send_count)
+    assert torch.equal(st.pair_slot[:t].cpu(), pair_slot)
+    # combine with the identity expert: every pair returns the row it was sent, so out = x * sum of weights
+    epr = e // r
+    y = torch.zeros((epr, r * m, h), dtype=torch.bfloat16)
+    count = st.packed_recv_count.cpu()
+    for le in range(epr):
+        n = int(count[le])
+        if fmt == O.ROW_BF16:
+            y[le, :n] = st.packed_recv_x[le, :n].cpu()
+        else:
+            y[le, :n] = O.per_token_cast_back(st.packed_recv_x[le, :n].cpu(), st.packed_recv_scales[le, :n].cpu())
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    run_combine(st, world, y.cuda(), topk_all[rank].cuda(), w_all[rank].cuda(), out, mode=0, one_call=one_call)
+    wsum = w_all[rank].masked_fill(topk_all[rank] == -1, 0).sum(1).view(-1, 1)
+    expect = x_all[rank].float() * wsum
+    got = out.cpu().float()
+    assert torch.isnan(got).sum().item() == 0
+    live = wsum.view(-1) > 0
+    assert (got[~live] == 0).all()  # a token with no valid selection combines to zero
+    if live.any():
+        diff = O.calc_diff(expect[live], got[live])
+        assert diff < (2e-3 if fmt != O.ROW_BF16 else 1e-4), (diff, (r, rank, t, m, h, k, e, fmt))
+
+
 def test_dispatch_send_staging_and_send_slots(rt):
     """The send side alone: own rows for own experts land in recv_staging, the rest in send_slots."""
     r, rank, t, h, k, e, m = 4, 2, 20, 512, 4, 32, 24
