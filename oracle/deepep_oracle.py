@@ -28,6 +28,8 @@ generative on CUDA RNG streams that cannot be replayed here):
   kernels (``_serial_dispatch``) compared against the vectorised form.
 * combine — the closed form ``x * sum(w)`` of ``tests/test_low_latency.py:181``
   and a float64 sum.
+* layout, route slots, dispatch outputs (both segment orders) and the combine — also a
+  two-rank world worked out on paper, ``tests/golden/ll_tiny_world.json``.
 * ``topk_remap``, ``build_recv_src_meta`` — the torch expressions the reference's kernels
   replaced (named in their headers, ``csrc/kernels/efa_kernels.cu:321-337,438-446``), pinned
   by literal Python loops over the kernels' own per-element rule.

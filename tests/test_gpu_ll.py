@@ -13,6 +13,7 @@ import pytest
 import torch
 
 from oracle import deepep_oracle as O
+from tiny_world import load_tiny_world, tiny_world_expected
 
 pytestmark = pytest.mark.gpu
 
@@ -149,6 +150,38 @@ def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
     send_count, pair_slot = O.route(topk_all[rank], e, t)
     assert torch.equal(st.send_count.cpu(), send_count)
     assert torch.equal(st.pair_slot[:t].cpu(), pair_slot)
+
+
+@pytest.mark.parametrize("key,rank,one_call", [("rank0_ascending", 0, False), ("rank0_own_last", 0, True),
+                                               ("rank1_ascending", 1, False)])
+@pytest.mark.parametrize("fmt", [O.ROW_BF16, O.ROW_FP8])
+def test_hand_derived_world(rt, key, rank, one_call, fmt):
+    """The HIP path against values worked out on paper (tests/golden/ll_tiny_world.json): no oracle involved."""
+    g, x_all, topk_all = load_tiny_world()
+    e, m, h, t, k = g["num_experts"], g["max_tokens"], g["hidden"], g["num_tokens"], g["num_topk"]
+    st, world = dispatch_on_gpu(rt, torch.stack(x_all), torch.stack(topk_all), rank, e, m, fmt, one_call=one_call)
+    want, layout = tiny_world_expected(g, key)
+    assert st.packed_recv_count.cpu().tolist() == want["count"]
+    assert torch.equal(st.packed_recv_layout_range.cpu(), layout)
+    for le, n in enumerate(want["count"]):
+        assert st.packed_recv_src_info[le, :n].cpu().tolist() == want["src_info"][le]
+        values = torch.tensor(want["row_value"][le], dtype=torch.float32)
+        if fmt == O.ROW_BF16:
+            assert torch.equal(st.packed_recv_x[le, :n].cpu().float(), values.view(-1, 1).expand(-1, h))
+        else:
+            assert (st.packed_recv_x[le, :n].view(torch.uint8).cpu() == g["fp8"]["payload_byte"]).all()
+            assert torch.equal(st.packed_recv_scales[le, :n].cpu().view(-1), values / torch.tensor(448.0))
+    if rank != 0:
+        return
+    assert st.send_count.cpu().tolist() == g["route_rank0"]["send_count"]
+    assert st.pair_slot[:t].cpu().tolist() == g["route_rank0"]["pair_slot"]
+    if fmt == O.ROW_BF16:  # identity experts: what comes back is what was sent
+        y = st.packed_recv_x.clone()
+        out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+        w = torch.tensor(g["topk_weights_rank0"], dtype=torch.float32, device="cuda")
+        run_combine(st, world, y, topk_all[0].cuda(), w, out, mode=0, one_call=one_call)
+        expect = torch.tensor(g["combine_rank0_identity_experts"]).view(-1, 1).expand(-1, h)
+        assert torch.equal(out.cpu().float(), expect)
 
 
 def _random_shape(seed):

@@ -458,3 +458,48 @@ def test_combine_reduce_definitions_agree():
     none = torch.nonzero(is_in.sum(1) == 0).flatten()
     for tok in none.tolist():
         assert (chain_nb[tok] == 0).all()
+
+
+# ---------------------------------------------------------------------------
+# the hand-derived two-rank world of tests/golden/ll_tiny_world.json
+# ---------------------------------------------------------------------------
+from tiny_world import load_tiny_world, tiny_world_expected  # noqa: E402
+
+
+@pytest.mark.parametrize("key,rank,own_last", [("rank0_ascending", 0, False), ("rank0_own_last", 0, True),
+                                               ("rank1_ascending", 1, False)])
+@pytest.mark.parametrize("fmt", [O.ROW_BF16, O.ROW_FP8])
+def test_oracle_against_the_hand_derived_world(key, rank, own_last, fmt):
+    g, x_all, topk_all = load_tiny_world()
+    e, m, h = g["num_experts"], g["max_tokens"], g["hidden"]
+    got = O.ll_dispatch(x_all, topk_all, rank, e, m, fmt, own_last=own_last)
+    want, layout = tiny_world_expected(g, key)
+    assert got["packed_recv_count"].tolist() == want["count"]
+    assert torch.equal(got["packed_recv_layout_range"], layout)
+    for le, n in enumerate(want["count"]):
+        assert got["packed_recv_src_info"][le, :n].tolist() == want["src_info"][le]
+        values = torch.tensor(want["row_value"][le], dtype=torch.float32)
+        if fmt == O.ROW_BF16:
+            rows = got["packed_recv_x"][le, :n].contiguous().view(torch.bfloat16).float()
+            assert torch.equal(rows, values.view(-1, 1).expand(-1, h))
+        else:
+            assert (got["packed_recv_x"][le, :n] == g["fp8"]["payload_byte"]).all()
+            scales = got["packed_recv_scales"][le, :n].contiguous().view(torch.float32).view(-1)
+            assert torch.equal(scales, values / torch.tensor(448.0))  # one group per row
+    if rank == 0:
+        send_count, pair_slot = O.route(topk_all[0], e, m)
+        assert send_count.tolist() == g["route_rank0"]["send_count"]
+        assert pair_slot.tolist() == g["route_rank0"]["pair_slot"]
+        pr, pn, pe, is_in = O.get_dispatch_layout(topk_all[0], e, g["num_ranks"])
+        assert pe.tolist() == g["layout_rank0"]["num_tokens_per_expert"]
+        assert pr.tolist() == g["layout_rank0"]["num_tokens_per_rank"] and pn is None
+        assert is_in.tolist() == g["layout_rank0"]["is_token_in_rank"]
+
+
+def test_oracle_combine_against_the_hand_derived_world():
+    g, x_all, topk_all = load_tiny_world()
+    w = torch.tensor(g["topk_weights_rank0"], dtype=torch.float32)
+    pair_rows = x_all[0].unsqueeze(1).expand(-1, g["num_topk"], -1)  # identity experts
+    want = torch.tensor(g["combine_rank0_identity_experts"]).view(-1, 1).expand(-1, g["hidden"])
+    assert torch.equal(O.ll_combine(pair_rows, topk_all[0], w).float(), want)
+    assert torch.equal(O.ll_combine_f32_chain(pair_rows, w, topk_all[0] >= 0).float(), want)
