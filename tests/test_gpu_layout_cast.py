@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from oracle import deepep_oracle as O
+from tiny_world import load_tiny_world
 
 pytestmark = pytest.mark.gpu
 
@@ -69,6 +70,34 @@ def test_get_dispatch_layout(capi, t, k, e, r, drop):
         assert torch.equal(got[1], want[1])
     assert torch.equal(got[2], want[2])
     assert torch.equal(got[3], want[3])
+
+
+def test_hand_derived_world_layout_sort_and_prefix(capi):
+    """Layout, routing sort and channel prefix against values worked out on paper
+    (tests/golden/ll_tiny_world.json): no oracle involved."""
+    g, _, topk_all = load_tiny_world()
+    lib = capi.load()
+    r, e, t = g["num_ranks"], g["num_experts"], g["num_tokens"]
+    per_rank, per_rdma, per_expert, is_in = run_layout(capi, topk_all[0], e, r)
+    assert per_rank.tolist() == g["layout_rank0"]["num_tokens_per_rank"] and per_rdma is None
+    assert per_expert.tolist() == g["layout_rank0"]["num_tokens_per_expert"]
+    assert is_in.tolist() == g["layout_rank0"]["is_token_in_rank"]
+    want = g["normal_mode_rank0"]
+    dev = is_in.cuda()
+    ids = torch.full((t * r,), -1, dtype=torch.int64, device="cuda")
+    counts = torch.full((r,), -1, dtype=torch.int32, device="cuda")
+    cumsum = torch.full((r + 1,), -1, dtype=torch.int64, device="cuda")
+    ws = torch.empty(max(16, lib.deepep_routing_sort_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
+    capi.check(lib.deepep_moe_routing_sort(capi.ptr(dev), t, r, capi.ptr(ids), capi.ptr(counts), capi.ptr(cumsum),
+                                           capi.ptr(ws), ws.numel(), stream()))
+    torch.cuda.synchronize()
+    assert counts.cpu().tolist() == want["send_counts"] and cumsum.cpu().tolist() == want["send_cumsum"]
+    assert ids[:4].cpu().tolist() == want["sorted_token_ids"]
+    for c in (2, 3):
+        cpm = torch.full((r, c), -1, dtype=torch.int32, device="cuda")
+        capi.check(lib.deepep_channel_prefix_matrix(capi.ptr(dev), t, r, c, capi.ptr(cpm), stream()))
+        torch.cuda.synchronize()
+        assert cpm.cpu().tolist() == want[f"channel_prefix_matrix_{c}_channels"]
 
 
 def test_layout_rejects_bad_shapes(capi):

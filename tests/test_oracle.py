@@ -503,3 +503,14 @@ def test_oracle_combine_against_the_hand_derived_world():
     want = torch.tensor(g["combine_rank0_identity_experts"]).view(-1, 1).expand(-1, g["hidden"])
     assert torch.equal(O.ll_combine(pair_rows, topk_all[0], w).float(), want)
     assert torch.equal(O.ll_combine_f32_chain(pair_rows, w, topk_all[0] >= 0).float(), want)
+
+
+def test_oracle_normal_mode_against_the_hand_derived_world():
+    g, _, _ = load_tiny_world()
+    want = g["normal_mode_rank0"]
+    is_in = torch.tensor(g["layout_rank0"]["is_token_in_rank"])
+    ids, counts, cumsum, total = O.moe_routing_sort(is_in)
+    assert ids.tolist() == want["sorted_token_ids"] and counts.tolist() == want["send_counts"]
+    assert cumsum.tolist() == want["send_cumsum"] and total == 4
+    assert O.channel_prefix_matrix(is_in, 2).tolist() == want["channel_prefix_matrix_2_channels"]
+    assert O.channel_prefix_matrix(is_in, 3).tolist() == want["channel_prefix_matrix_3_channels"]
