@@ -711,6 +711,34 @@ static torch::Tensor build_recv_src_meta(const torch::Tensor& recv_counts, const
     return meta;
 }
 
+// reference: csrc/transport/ll_pipeline.cpp:1204-1269,1277-1361 — the bookkeeping between the gather of the
+// route counts and the exchange, on the stream instead of on the host.  Returns (send_counts [R] i32,
+// recv_counts [R] i32, totals [3] i32 = sent / received / corrupt, combine_remote_recv_offset [R] i64,
+// records [4, row_capacity] i32 = source_rank / source_offset / padded_index / combine_send_offset,
+// num_recv_tokens [2] i32, tokens_per_expert [E_l] i32).
+static std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor, torch::Tensor>
+ll_exchange_metadata(const torch::Tensor& all_num_routed, int rank, int num_max_dispatch_tokens_per_rank,
+                     int64_t row_capacity) {
+    EP_HOST_ASSERT(all_num_routed.dim() == 2 and all_num_routed.is_contiguous() and all_num_routed.is_cuda());
+    EP_HOST_ASSERT(all_num_routed.scalar_type() == torch::kInt32);
+    EP_HOST_ASSERT(row_capacity >= 0);
+    const int num_ranks = static_cast<int>(all_num_routed.size(0)), num_experts = static_cast<int>(all_num_routed.size(1));
+    EP_HOST_ASSERT(num_ranks > 0 and num_experts % num_ranks == 0);
+    const auto i32 = torch::dtype(torch::kInt32).device(all_num_routed.device());
+    auto send_counts = torch::empty({num_ranks}, i32), recv_counts = torch::empty({num_ranks}, i32);
+    auto totals = torch::empty({3}, i32), num_recv_tokens = torch::empty({2}, i32);
+    auto remote = torch::empty({num_ranks}, i32.dtype(torch::kInt64));
+    auto records = torch::empty({4, row_capacity}, i32);
+    auto tokens_per_expert = torch::empty({num_experts / num_ranks}, i32);
+    auto rec = [&](int i) { return reinterpret_cast<uint32_t*>(records.data_ptr<int>()) + int64_t(i) * row_capacity; };
+    abi_check(deepep_ll_exchange_metadata(
+        all_num_routed.data_ptr<int>(), num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank, row_capacity,
+        send_counts.data_ptr<int>(), recv_counts.data_ptr<int>(), totals.data_ptr<int>(), remote.data_ptr<int64_t>(),
+        rec(0), rec(1), rec(2), rec(3), reinterpret_cast<uint32_t*>(num_recv_tokens.data_ptr<int>()),
+        reinterpret_cast<uint32_t*>(tokens_per_expert.data_ptr<int>()), current_stream()));
+    return {send_counts, recv_counts, totals, remote, records, num_recv_tokens, tokens_per_expert};
+}
+
 // reference: deep_ep/buffer.py:1542-1557 — zero_() + index_add_ over the returned rows, then the biases
 static std::tuple<torch::Tensor, std::optional<torch::Tensor>> combine_reduce(
     const torch::Tensor& recv_x, const std::optional<torch::Tensor>& recv_topk_weights,
@@ -847,5 +875,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("pack_rows", &deep_ep::pack_rows, "Gather rows into per-rank contiguous send buffers");
     m.def("topk_remap", &deep_ep::topk_remap, "Top-k of the send rows in the destination rank's expert numbering");
     m.def("build_recv_src_meta", &deep_ep::build_recv_src_meta, "Source-rank metadata of the received rows");
+    m.def("ll_exchange_metadata", &deep_ep::ll_exchange_metadata,
+          "Send/receive counts, combine offsets and per-row records from the gathered route counts");
     m.def("combine_reduce", &deep_ep::combine_reduce, "Per-token sum of the rows that came back (normal-mode combine)");
 }

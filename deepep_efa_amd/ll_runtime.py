@@ -158,3 +158,24 @@ class LowLatencyState:
             t, s.hidden, s.num_topk, s.num_experts, s.num_ranks, s.rank, s.max_tokens, int(accumulate),
             _capi.ptr(self.combine_staging), _capi.ptr(self.combine_send_slots), _capi.ptr(out),
             self.expected_rows, _capi.ptr(sw), 0 if sw is None else sw.numel(), current_stream_ptr()))
+
+
+def exchange_metadata(all_num_routed: torch.Tensor, rank: int, max_tokens: int, row_capacity: int) -> dict:
+    """Send / receive counts, combine offsets and one record per expected row from the gathered
+    per-expert route counts [R, E] int32 (csrc/transport/ll_pipeline.cpp:1204-1361), on the current stream."""
+    lib = _capi.load()
+    r, e = all_num_routed.shape
+    dev = all_num_routed.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    out = dict(send_counts=torch.empty(r, **i32), recv_counts=torch.empty(r, **i32), totals=torch.empty(3, **i32),
+               combine_remote_recv_offset=torch.empty(r, dtype=torch.int64, device=dev),
+               source_rank=torch.empty(row_capacity, **i32), source_offset=torch.empty(row_capacity, **i32),
+               padded_index=torch.empty(row_capacity, **i32), combine_send_offset=torch.empty(row_capacity, **i32),
+               num_recv_tokens=torch.empty(2, **i32), tokens_per_expert=torch.empty(e // r, **i32))
+    _capi.check(lib.deepep_ll_exchange_metadata(
+        _capi.ptr(all_num_routed), e, r, rank, max_tokens, row_capacity, _capi.ptr(out["send_counts"]),
+        _capi.ptr(out["recv_counts"]), _capi.ptr(out["totals"]), _capi.ptr(out["combine_remote_recv_offset"]),
+        _capi.ptr(out["source_rank"]), _capi.ptr(out["source_offset"]), _capi.ptr(out["padded_index"]),
+        _capi.ptr(out["combine_send_offset"]), _capi.ptr(out["num_recv_tokens"]), _capi.ptr(out["tokens_per_expert"]),
+        current_stream_ptr()))
+    return out

@@ -260,6 +260,32 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
                             int64_t expected_rows, void* workspace, size_t workspace_bytes,
                             void* stream);
 
+/* What a rank derives from the gathered per-expert route counts before the
+ * exchange, in one launch instead of the reference's host loops over three
+ * device-to-host copies.
+ *   all_num_routed [R, E] int32: row s = the pairs rank s routed to each expert
+ *                  (this rank's own row is the send_count of its dispatch)
+ *   send_counts [R] int32 (out): rows this rank sends to each rank
+ *   recv_counts [R] int32 (out): rows it receives from each rank
+ *   totals      [3] int32 (out): total sent, total received, 1 if the gather was corrupt
+ *               (any count above M: every count is then reported as zero, as the reference does)
+ *   combine_remote_recv_offset [R] int64 (out): rows peer s sent to the ranks below this one,
+ *               i.e. where this rank's returned rows start in peer s's combine buffer
+ *   source_rank, source_offset, padded_index, combine_send_offset [row_capacity] uint32 (out):
+ *               one record per expected row i, grouped by source rank s in ascending order, the
+ *               j-th row of a source getting (s, s * M + j, i, i)
+ *   num_recv_tokens [2] uint32 (out): rows expected, records written (the smaller of that and row_capacity)
+ *   tokens_per_expert [E_l] uint32 (out): zeroed, as the reference leaves it for the receive kernel
+ * Replaces LLPipelineWorker::compute_send_recv_counts and ::upload_recv_metadata
+ * (csrc/transport/ll_pipeline.cpp:1204-1269, :1277-1361). */
+int deepep_ll_exchange_metadata(const int32_t* all_num_routed, int num_experts, int num_ranks, int rank,
+                                int num_max_dispatch_tokens_per_rank, int64_t row_capacity,
+                                int32_t* send_counts, int32_t* recv_counts, int32_t* totals,
+                                int64_t* combine_remote_recv_offset,
+                                uint32_t* source_rank, uint32_t* source_offset, uint32_t* padded_index,
+                                uint32_t* combine_send_offset, uint32_t* num_recv_tokens,
+                                uint32_t* tokens_per_expert, void* stream);
+
 /* ------------------------------------------------------------------ */
 /* Low-latency combine                                                */
 /* ------------------------------------------------------------------ */

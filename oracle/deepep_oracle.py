@@ -35,6 +35,9 @@ generative on CUDA RNG streams that cannot be replayed here):
   by literal Python loops over the kernels' own per-element rule.
 * ``combine_reduce`` — ``zero_() + index_add_`` (``deep_ep/buffer.py:1542-1557``) in float64,
   the identity "one rank per token returns the row itself", and a float32 chain in rank order.
+* ``ll_exchange_metadata`` — the reference's host loops restated loop for loop; pinned by the
+  hand-derived two-rank world (``tests/golden/ll_tiny_world.json``) and by the identities that tie it to
+  the dispatch (recv_counts = row sums of the receiver's ``recv_count``; records = a running index).
 * ``get_low_latency_rdma_size_hint`` — hand-computed values.
 * ``round_scale`` scales: **parity unpinned at ulp boundaries** — the reference
   computes ``exp2(ceil(log2(s)))`` in float32 (``deep_ep/buffer.py:1601``,
@@ -426,6 +429,64 @@ def staged_rows(x: torch.Tensor, topk_idx: torch.Tensor, src_rank: int, num_expe
 # ----------------------------------------------------------------------------
 # Low-latency combine
 # ----------------------------------------------------------------------------
+def ll_exchange_metadata(all_num_routed: torch.Tensor, rank: int, max_tokens: int):
+    """The host-side bookkeeping between the route-count gather and the exchange, loop for loop.
+
+    all_num_routed [R, E] int: row s = pairs rank s routed to each expert.
+    compute_send_recv_counts (csrc/transport/ll_pipeline.cpp:1204-1269): any count above the
+    per-expert bound (max_tokens, 4096 if that is not positive) zeroes every send and receive count;
+    otherwise send[r] = sum of this rank's row over rank r's experts, recv[r] = sum of rank r's row
+    over this rank's experts.
+    upload_recv_metadata (:1277-1361): combine_remote_recv_offset[j] = what peer j routed to the
+    ranks below this one; per expected row, grouped by source rank: (source_rank, source_offset =
+    r * max_tokens + t, padded_index = running index, combine_send_offset = rows of lower sources + t);
+    a total outside [0, R * max_tokens * 8] receives nothing.
+    Returns a dict of int64 tensors / ints under the reference's names.
+    """
+    num_ranks, num_experts = all_num_routed.shape
+    epr = num_experts // num_ranks
+    routed = all_num_routed.to(torch.int64) & 0xFFFFFFFF  # the reference reads them as uint32
+    bound = max_tokens if max_tokens > 0 else 4096
+    send = [0] * num_ranks
+    recv = [0] * num_ranks
+    corrupt = bool((routed > bound).any())
+    if not corrupt:
+        for e in range(num_experts):
+            send[e // epr] += int(routed[rank, e])
+        for r in range(num_ranks):
+            for e in range(rank * epr, (rank + 1) * epr):
+                recv[r] += int(routed[r, e])
+    total_send, total_recv = sum(send), sum(recv)
+    remote = []
+    for j in range(num_ranks):
+        off = 0
+        for r in range(rank):
+            for e in range(r * epr, (r + 1) * epr):
+                off += int(routed[j, e])
+        remote.append(off)
+    if total_recv < 0 or total_recv > num_ranks * max_tokens * 8:
+        total_recv = 0
+    src_rank, src_off, padded, comb = [], [], [], []
+    group = [0] * num_ranks
+    acc = 0
+    for r in range(num_ranks):
+        group[r] = acc
+        acc += recv[r]
+    idx = 0
+    if total_recv:
+        for r in range(num_ranks):
+            for t in range(recv[r]):
+                src_rank.append(r)
+                src_off.append(r * max_tokens + t)
+                padded.append(idx)
+                comb.append(group[r] + t)
+                idx += 1
+    as_t = lambda v: torch.tensor(v, dtype=torch.int64)
+    return dict(send_counts=as_t(send), recv_counts=as_t(recv), total_send=total_send, total_recv=total_recv,
+                corrupt=corrupt, combine_remote_recv_offset=as_t(remote), source_rank=as_t(src_rank),
+                source_offset=as_t(src_off), padded_index=as_t(padded), combine_send_offset=as_t(comb))
+
+
 def ll_combine(pair_rows: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor,
                pair_live: torch.Tensor | None = None) -> torch.Tensor:
     """out[t] = sum_k [live] w[t,k] * f32(pair_rows[t,k]) in float64, rounded to bf16 by the caller's check.

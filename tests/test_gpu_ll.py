@@ -184,6 +184,75 @@ def test_hand_derived_world(rt, key, rank, one_call, fmt):
         assert torch.equal(out.cpu().float(), expect)
 
 
+def check_exchange_metadata(got, want, capacity):
+    assert got["send_counts"].cpu().tolist() == want["send_counts"].tolist()
+    assert got["recv_counts"].cpu().tolist() == want["recv_counts"].tolist()
+    assert got["totals"].cpu().tolist() == [want["total_send"], want["total_recv"], int(want["corrupt"])]
+    assert got["combine_remote_recv_offset"].cpu().tolist() == want["combine_remote_recv_offset"].tolist()
+    n = min(want["total_recv"], capacity)
+    assert got["num_recv_tokens"].cpu().tolist() == [want["total_recv"], n]
+    for key in ("source_rank", "source_offset", "padded_index", "combine_send_offset"):
+        assert got[key][:n].cpu().tolist() == want[key][:n].tolist(), key
+        assert (got[key][n:] == -7).all(), key  # nothing written past the records
+    assert (got["tokens_per_expert"] == 0).all()
+
+
+@pytest.mark.parametrize("r,e,m,k,rank,capacity", [(2, 4, 3, 2, 1, 16), (6, 24, 40, 5, 4, 400), (32, 256, 128, 8, 5, 4096),
+                                                   (64, 256, 8192, 8, 63, 70000), (8, 64, 300, 6, 0, 100),
+                                                   (1, 4, 9, 2, 0, 32), (160, 160, 20, 3, 77, 64)])
+def test_exchange_metadata(rt, r, e, m, k, rank, capacity):
+    """Counts, combine offsets and row records from the gathered route counts, against the reference's host loops."""
+    g = torch.Generator().manual_seed(r * 7 + e)
+    if r * m <= 4096:
+        topk_all = [torch.stack([torch.randperm(e, generator=g)[:k] for _ in range(m)]) for _ in range(r)]
+        routed = torch.stack([O.route(tk, e, m)[0] for tk in topk_all]).to(torch.int32)
+    else:  # any matrix of plausible counts will do
+        routed = torch.randint(0, min(m, 60) + 1, (r, e), generator=g, dtype=torch.int32)
+    for name, mat in (("clean", routed), ("corrupt", routed.clone())):
+        if name == "corrupt":
+            mat[r // 2, e // 3] = m + 1
+        got = {}
+        out = rt.ll.exchange_metadata(mat.cuda(), rank, m, capacity)
+        torch.cuda.synchronize()
+        want = O.ll_exchange_metadata(mat, rank, m)
+        assert want["corrupt"] == (name == "corrupt")
+        # poison-free check of "nothing written past the records": run again into pre-filled buffers
+        for key in ("source_rank", "source_offset", "padded_index", "combine_send_offset"):
+            got[key] = torch.full((capacity,), -7, dtype=torch.int32, device="cuda")
+        lib, capi = rt.capi.load(), rt.capi
+        for key in ("send_counts", "recv_counts", "totals", "combine_remote_recv_offset", "num_recv_tokens",
+                    "tokens_per_expert"):
+            got[key] = torch.full_like(out[key], -7)
+        capi.check(lib.deepep_ll_exchange_metadata(
+            capi.ptr(mat.cuda()), e, r, rank, m, capacity, capi.ptr(got["send_counts"]), capi.ptr(got["recv_counts"]),
+            capi.ptr(got["totals"]), capi.ptr(got["combine_remote_recv_offset"]), capi.ptr(got["source_rank"]),
+            capi.ptr(got["source_offset"]), capi.ptr(got["padded_index"]), capi.ptr(got["combine_send_offset"]),
+            capi.ptr(got["num_recv_tokens"]), capi.ptr(got["tokens_per_expert"]),
+            torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        check_exchange_metadata(got, want, capacity)
+        for key in got:
+            n = min(want["total_recv"], capacity) if got[key].numel() == capacity else got[key].numel()
+            assert torch.equal(out[key][:n], got[key][:n]), key
+
+
+def test_exchange_metadata_hand_derived_world(rt):
+    g, _, _ = load_tiny_world()
+    routed = torch.tensor(g["all_num_routed"], dtype=torch.int32)
+    for rank in (0, 1):
+        out = rt.ll.exchange_metadata(routed.cuda(), rank, g["max_tokens"], 8)
+        torch.cuda.synchronize()
+        want = g["exchange_metadata"][f"rank{rank}"]
+        n = want["total_recv"]
+        assert out["send_counts"].cpu().tolist() == want["send_counts"]
+        assert out["recv_counts"].cpu().tolist() == want["recv_counts"]
+        assert out["totals"].cpu().tolist() == [want["total_send"], n, 0]
+        assert out["combine_remote_recv_offset"].cpu().tolist() == want["combine_remote_recv_offset"]
+        assert out["num_recv_tokens"].cpu().tolist() == [n, n]
+        for key in ("source_rank", "source_offset", "padded_index", "combine_send_offset"):
+            assert out[key][:n].cpu().tolist() == want[key], key
+
+
 def _random_shape(seed):
     g = np.random.default_rng(seed)
     r = int(g.choice([1, 2, 3, 4, 5, 6, 8, 12, 16, 24]))

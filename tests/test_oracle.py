@@ -514,3 +514,37 @@ def test_oracle_normal_mode_against_the_hand_derived_world():
     assert cumsum.tolist() == want["send_cumsum"] and total == 4
     assert O.channel_prefix_matrix(is_in, 2).tolist() == want["channel_prefix_matrix_2_channels"]
     assert O.channel_prefix_matrix(is_in, 3).tolist() == want["channel_prefix_matrix_3_channels"]
+
+
+@pytest.mark.parametrize("rank", [0, 1])
+def test_oracle_exchange_metadata_against_the_hand_derived_world(rank):
+    g, _, topk_all = load_tiny_world()
+    routed = torch.tensor(g["all_num_routed"], dtype=torch.int32)
+    for s in range(g["num_ranks"]):  # the matrix itself: row s is rank s's per-expert pair count
+        assert routed[s].tolist() == O.route(topk_all[s], g["num_experts"], g["max_tokens"])[0].tolist()
+    got = O.ll_exchange_metadata(routed, rank, g["max_tokens"])
+    want = g["exchange_metadata"][f"rank{rank}"]
+    for key, value in want.items():
+        assert (got[key].tolist() if torch.is_tensor(got[key]) else got[key]) == value, key
+    assert not got["corrupt"]
+
+
+def test_oracle_exchange_metadata_identities_and_corrupt_counts():
+    r, e, m, rank = 6, 24, 40, 4
+    g = torch.Generator().manual_seed(9)
+    topk_all = [torch.stack([torch.randperm(e, generator=g)[:5] for _ in range(m)]) for _ in range(r)]
+    routed = torch.stack([O.route(tk, e, m)[0] for tk in topk_all]).to(torch.int32)
+    got = O.ll_exchange_metadata(routed, rank, m)
+    epr = e // r
+    # what the dispatch itself delivers: rows from source s = its pairs on this rank's experts
+    want = O.ll_dispatch([torch.zeros((m, 128), dtype=torch.bfloat16)] * r, topk_all, rank, e, m, O.ROW_BF16)
+    per_source = (want["packed_recv_layout_range"] & 0xFFFFFFFF).sum(0)
+    assert got["recv_counts"].tolist() == per_source.tolist()
+    assert got["total_recv"] == int(want["packed_recv_count"].sum())
+    assert got["send_counts"].tolist() == routed[rank].view(r, epr).sum(1).tolist()
+    assert got["padded_index"].tolist() == list(range(got["total_recv"])) == got["combine_send_offset"].tolist()
+    assert got["combine_remote_recv_offset"].tolist() == routed[:, :rank * epr].sum(1).tolist()
+    routed[2, 7] = m + 1  # one impossible count: nobody sends or receives this time
+    bad = O.ll_exchange_metadata(routed, rank, m)
+    assert bad["corrupt"] and bad["total_send"] == 0 and bad["total_recv"] == 0
+    assert bad["send_counts"].sum() == 0 and bad["recv_counts"].sum() == 0 and bad["source_rank"].numel() == 0
