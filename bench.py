@@ -43,6 +43,7 @@ def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0):
         "dispatch": (t * 2 * h + t * k * 8 + (p - own) * stride + own * packed + t * k * 4 + e * 4
                      + (rv - own) * (stride + packed) + small),
         "combine": (rv - own) * 2 * h * 2 + (e // r) * r * 8 + p * 2 * h + t * k * 16 + t * 2 * h,
+        "exchange_metadata": r * e * 4 + rv * 16 + r * 24,
     }
 
 
@@ -280,7 +281,17 @@ def main():
     rv = int(st.packed_recv_count.sum())
     own = int((st.packed_recv_layout_range[:, rank] & 0xFFFFFFFF).sum())
 
+    # the gathered route counts of the whole world, as a count all-gather would leave them
+    tk = world.topk_idx_all.view(r, -1)
+    routed = torch.stack([torch.bincount(tk[s][tk[s] >= 0], minlength=e) for s in range(r)]).to(torch.int32)
+    meta_out = ll_runtime.exchange_metadata(routed, rank, t, r * t)  # buffers made once, reused below
+    meta_args = [_capi.ptr(routed), e, r, rank, t, r * t] + [_capi.ptr(meta_out[n]) for n in (
+        "send_counts", "recv_counts", "totals", "combine_remote_recv_offset", "source_rank", "source_offset",
+        "padded_index", "combine_send_offset", "num_recv_tokens", "tokens_per_expert")]
+
     calls = {
+        "exchange_metadata": lambda: _capi.check(lib.deepep_ll_exchange_metadata(
+            *meta_args, torch.cuda.current_stream().cuda_stream)),
         "dispatch": lambda: st.dispatch(x, topk),  # send + receive phase, one launch at this size
         "combine": lambda: st.combine(y, topk, weights, out),  # row return + reduce, one launch at this size
         "dispatch_send": lambda: st.dispatch_send(x, topk),

@@ -12,8 +12,15 @@ namespace deepep {
 constexpr int kExchangeThreads = 1024;
 constexpr int kExchangeMaxRanks = 1024;
 
-// Every workgroup derives the per-rank tables itself (R * E_l reads each, from L2) and then fills
-// its share of the row records; workgroup 0 also writes the per-rank outputs.
+__device__ __forceinline__ int64_t wave_sum_i64(int64_t v) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) v += __shfl_xor(v, d, kWave);
+    return v;
+}
+
+// Every workgroup derives the per-rank tables itself (the R x E counts once, from L2: one wave per
+// source rank, every load of a row in flight together) and then fills its share of the row
+// records; workgroup 0 also writes the per-rank outputs.
 __global__ __launch_bounds__(kExchangeThreads) void ll_exchange_meta_kernel(
     const int32_t* __restrict__ all_num_routed, int num_experts, int num_ranks, int rank, int max_tokens,
     int64_t row_capacity, int32_t* __restrict__ send_counts, int32_t* __restrict__ recv_counts,
@@ -23,34 +30,62 @@ __global__ __launch_bounds__(kExchangeThreads) void ll_exchange_meta_kernel(
     uint32_t* __restrict__ tokens_per_expert) {
     __shared__ int32_t recv_prefix[kExchangeMaxRanks + 1];
     __shared__ int32_t recv_of[kExchangeMaxRanks];
-    __shared__ int corrupt;
-    const int tid = threadIdx.x;
+    __shared__ int32_t send_to[kExchangeMaxRanks];
+    __shared__ int64_t below_of[kExchangeMaxRanks];
+    __shared__ int32_t wave_bad[kExchangeThreads / kWave];
+    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
+    constexpr int kWaves = kExchangeThreads / kWave;
     const int experts_per_rank = num_experts / num_ranks;
     const int first_expert = rank * experts_per_rank;
     // a count above the per-expert bound marks the whole gather as corrupt: nobody sends or
     // receives this time (csrc/transport/ll_pipeline.cpp:1216-1248)
     const uint32_t max_per_expert = max_tokens > 0 ? uint32_t(max_tokens) : 4096u;
-    if (tid == 0) corrupt = 0;
-    lds_barrier();
     bool bad = false;
-    for (int i = tid; i < num_ranks * num_experts; i += kExchangeThreads)
-        bad |= uint32_t(all_num_routed[i]) > max_per_expert;
-    if (bad) corrupt = 1;  // every writer stores the same value
-    lds_barrier();
-    const bool is_corrupt = corrupt != 0;
-
-    for (int r = tid; r < num_ranks; r += kExchangeThreads) {
-        int sum = 0;
-        if (!is_corrupt)
-            for (int e = 0; e < experts_per_rank; ++e) sum += all_num_routed[r * num_experts + first_expert + e];
-        recv_of[r] = sum;
+    for (int r = w; r < num_ranks; r += kWaves) {
+        const int32_t* row = all_num_routed + int64_t(r) * num_experts;
+        int64_t below = 0;  // what rank r routed to the ranks below this one
+        int to_me = 0;      // ... and to this rank's experts
+        for (int e0 = 0; e0 < num_experts; e0 += 4 * kWave) {
+            uint32_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int e = e0 + u * kWave + lane;
+                v[u] = e < num_experts ? uint32_t(row[e]) : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int e = e0 + u * kWave + lane;
+                bad |= v[u] > max_per_expert;
+                if (e < first_expert) below += int64_t(v[u]);
+                else if (e < first_expert + experts_per_rank) to_me += int(v[u]);
+            }
+        }
+        below = wave_sum_i64(below);
+        to_me = __builtin_amdgcn_readlane(wave_inclusive_sum(to_me), kWave - 1);
+        if (lane == 0) below_of[r] = below, recv_of[r] = to_me;
+    }
+    {
+        const bool any = __ballot(bad) != 0;
+        if (lane == 0) wave_bad[w] = any ? 1 : 0;
+    }
+    // this rank's own row, summed per destination rank
+    const int32_t* mine = all_num_routed + int64_t(rank) * num_experts;
+    for (int r = w; r < num_ranks; r += kWaves) {
+        int part = 0;
+        for (int e = lane; e < experts_per_rank; e += kWave) part += mine[r * experts_per_rank + e];
+        part = __builtin_amdgcn_readlane(wave_inclusive_sum(part), kWave - 1);
+        if (lane == 0) send_to[r] = part;
     }
     lds_barrier();
+    bool is_corrupt = false;
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) is_corrupt |= wave_bad[i] != 0;
+
     if (tid < kWave) {  // exclusive prefix over the ranks, one wave
         int carry = 0;
         for (int r0 = 0; r0 < num_ranks; r0 += kWave) {
             const int r = r0 + tid;
-            const int v = r < num_ranks ? recv_of[r] : 0;
+            const int v = r < num_ranks && !is_corrupt ? recv_of[r] : 0;
             const int inc = wave_inclusive_sum(v);
             if (r < num_ranks) recv_prefix[r] = carry + inc - v;
             carry += __builtin_amdgcn_readlane(inc, kWave - 1);
@@ -61,28 +96,21 @@ __global__ __launch_bounds__(kExchangeThreads) void ll_exchange_meta_kernel(
     int total_recv = recv_prefix[num_ranks];
 
     if (blockIdx.x == 0) {
-        const int32_t* mine = all_num_routed + int64_t(rank) * num_experts;
         for (int r = tid; r < num_ranks; r += kExchangeThreads) {
-            int sum = 0;
-            if (!is_corrupt)
-                for (int e = 0; e < experts_per_rank; ++e) sum += mine[r * experts_per_rank + e];
-            send_counts[r] = sum;
-            recv_counts[r] = recv_of[r];
+            send_counts[r] = is_corrupt ? 0 : send_to[r];
+            recv_counts[r] = is_corrupt ? 0 : recv_of[r];
             // where this rank's returned rows start in peer r's combine buffer: behind what peer r
-            // sent to the ranks below this one (csrc/transport/ll_pipeline.cpp:1283-1295; the reference
-            // computes this one even for a corrupt gather)
-            int64_t offset = 0;
-            const int32_t* theirs = all_num_routed + int64_t(r) * num_experts;
-            for (int e = 0; e < first_expert; ++e) offset += int64_t(uint32_t(theirs[e]));
-            combine_remote_recv_offset[r] = offset;
+            // sent to the ranks below this one (csrc/transport/ll_pipeline.cpp:1283-1295, computed
+            // from the raw counts whatever their state)
+            combine_remote_recv_offset[r] = below_of[r];
         }
         for (int e = tid; e < experts_per_rank; e += kExchangeThreads) tokens_per_expert[e] = 0;
-        if (tid < kWave) {
+        if (tid >= kWave && tid < 2 * kWave) {  // wave 1: total sent
             int part = 0;
             if (!is_corrupt)
-                for (int e = tid; e < num_experts; e += kWave) part += mine[e];
+                for (int r = lane; r < num_ranks; r += kWave) part += send_to[r];
             const int total_send = __builtin_amdgcn_readlane(wave_inclusive_sum(part), kWave - 1);
-            if (tid == 0) totals[0] = total_send, totals[1] = total_recv, totals[2] = is_corrupt ? 1 : 0;
+            if (lane == 0) totals[0] = total_send, totals[1] = total_recv, totals[2] = is_corrupt ? 1 : 0;
         }
     }
     // csrc/transport/ll_pipeline.cpp:1306-1312: an impossible total receives nothing
