@@ -189,6 +189,7 @@ def bench_pack(torch, _capi, lib, loopback, args):
 def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args):
     """The same four LL entry points at 4096 tokens (8 ranks x 32 experts), where they are HBM-bound."""
     t, h, k, e, r, rank = 4096, 7168, 8, 256, 8, 3
+    h = int(os.environ.get("DEEPEP_BENCH_LARGE_HIDDEN", h))  # tuning aid
     shape = ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8)
     st = ll_runtime.LowLatencyState(shape)
     world = loopback.LoopbackWorld(r, rank, seed=args.seed + 7)

@@ -83,6 +83,23 @@ __device__ __forceinline__ void store_global(uint8_t* p, uint32_t v) { *(global_
 __device__ __forceinline__ u32x4 load_global_u32x4(const uint8_t* p) { return *(const global_u32x4*)(p); }
 __device__ __forceinline__ void store_global_byte(uint8_t* p, uint8_t v) { *(global_u8*)(p) = v; }
 
+// Streaming variants for kernels whose traffic exceeds what the caches hold: the non-temporal hint
+// keeps lines that will not be touched again from displacing others.  On this GPU a plain device
+// copy of 512 MiB runs at 6.1 TB/s with ordinary accesses and 6.6 TB/s with these; eight gathered
+// loads in flight per lane read at 6.2 against 7.0 TB/s.  kStream == false is the ordinary access.
+template <bool kStream>
+__device__ __forceinline__ u32x4 load_u32x4(const uint8_t* p) {
+    if constexpr (kStream) return __builtin_nontemporal_load((const global_u32x4*)(p));
+    else return *(const global_u32x4*)(p);
+}
+template <bool kStream>
+__device__ __forceinline__ void store_u32x4(uint8_t* p, u32x4 v) {
+    if constexpr (kStream) __builtin_nontemporal_store(v, (global_u32x4*)(p));
+    else *(global_u32x4*)(p) = v;
+}
+// Traffic above which a kernel streams (the memory-side cache holds 256 MB).
+constexpr int64_t kStreamBytes = int64_t(192) << 20;
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load and store of the wave, which stalls kernels that keep row loads in
 // flight across the barrier; use this one where threads exchange data through LDS alone.

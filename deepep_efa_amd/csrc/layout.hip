@@ -222,6 +222,9 @@ __global__ __launch_bounds__(256) void channel_prefix_kernel(const uint8_t* __re
 // should stay in L2 / Infinity Cache.
 // Reference: deep_ep/buffer.py:877,917 (torch advanced-index gathers).
 // ---------------------------------------------------------------------
+// kStream: the packed rows exceed what the caches hold, so they are written with the non-temporal
+// hint; the source rows are read the ordinary way because several destinations re-read them.
+template <bool kStream>
 __global__ __launch_bounds__(1024) void pack_rows_kernel(const uint8_t* __restrict__ src,
                                                          const uint8_t* __restrict__ scale_src,
                                                          const int64_t* __restrict__ ids,
@@ -234,9 +237,10 @@ __global__ __launch_bounds__(1024) void pack_rows_kernel(const uint8_t* __restri
     for (int64_t i = blockIdx.x; i < num_rows; i += gridDim.x) {
         const int64_t id = ids[i];
         if (id < 0 || id >= num_src_rows) continue;
-        const u32x4* s = reinterpret_cast<const u32x4*>(src + id * row_bytes);
-        u32x4* d = reinterpret_cast<u32x4*>(dst + i * row_bytes);
-        for (int v = threadIdx.x; v < num_vec; v += blockDim.x) d[v] = s[v];
+        const uint8_t* s = src + id * row_bytes;
+        uint8_t* d = dst + i * row_bytes;
+        for (int v = threadIdx.x; v < num_vec; v += blockDim.x)
+            store_u32x4<kStream>(d + int64_t(v) * 16, load_u32x4<false>(s + int64_t(v) * 16));
         if (scale_src != nullptr) {
             const uint32_t* ss = reinterpret_cast<const uint32_t*>(scale_src + id * scale_row_bytes);
             uint32_t* sd = reinterpret_cast<uint32_t*>(scale_dst + i * scale_row_bytes);
@@ -348,10 +352,14 @@ int deepep_pack_rows(const void* src, const void* scale_src, const int64_t* sort
     if (threads > 1024) threads = 1024;
     int64_t blocks = max_rows;
     if (blocks > (int64_t(1) << 22)) blocks = int64_t(1) << 22;
-    pack_rows_kernel<<<dim3(unsigned(blocks)), threads, 0, reinterpret_cast<hipStream_t>(stream)>>>(
-        reinterpret_cast<const uint8_t*>(src), reinterpret_cast<const uint8_t*>(scale_src), sorted_token_ids,
-        num_rows_dev, max_rows, num_src_rows, row_bytes, scale_row_bytes, reinterpret_cast<uint8_t*>(dst),
-        reinterpret_cast<uint8_t*>(scale_dst));
+#define DEEPEP_LAUNCH_PACK(STREAM)                                                                              \
+    pack_rows_kernel<STREAM><<<dim3(unsigned(blocks)), threads, 0, reinterpret_cast<hipStream_t>(stream)>>>(      \
+        reinterpret_cast<const uint8_t*>(src), reinterpret_cast<const uint8_t*>(scale_src), sorted_token_ids,      \
+        num_rows_dev, max_rows, num_src_rows, row_bytes, scale_row_bytes, reinterpret_cast<uint8_t*>(dst),         \
+        reinterpret_cast<uint8_t*>(scale_dst))
+    if (max_rows * row_bytes > kStreamBytes) DEEPEP_LAUNCH_PACK(true);
+    else DEEPEP_LAUNCH_PACK(false);
+#undef DEEPEP_LAUNCH_PACK
     EP_LAUNCH_CHECK();
     return 0;
 }

@@ -112,6 +112,7 @@ struct CombineRecvArgs {
     uint8_t* out;
 };
 
+template <bool kStream>
 __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int64_t item, const uint8_t* own_x,
                                                    const int32_t* own_begin, int own_first_expert,
                                                    int num_local_experts, int64_t slots_per_expert) {
@@ -173,7 +174,7 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
                 const uint32_t hi32 = __builtin_amdgcn_readlane(uint32_t(my_row >> 32), k);
                 wgt[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_weight), k));
                 const uint8_t* row = reinterpret_cast<const uint8_t*>((uint64_t(hi32) << 32) | lo32);
-                if (lane_live) v[u] = load_global_u32x4(row + off);
+                if (lane_live) v[u] = load_u32x4<kStream>(row + off);
             }
         }
         DEEPEP_PHASE(1);
@@ -192,12 +193,16 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
         u32x4 o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
-        *reinterpret_cast<u32x4*>(a.out + int64_t(t) * row_bytes + off) = o;
+        store_u32x4<kStream>(a.out + int64_t(t) * row_bytes + off, o);
     }
 }
 
+// kStream: the gathered rows exceed what the caches hold, so they are read (and the result written)
+// with the non-temporal hint.
+template <bool kStream>
 __global__ __launch_bounds__(1024) void ll_combine_recv_kernel(CombineRecvArgs a) {
-    combine_recv_piece(a, int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(), nullptr, nullptr, 0, 0, 0);
+    combine_recv_piece<kStream>(a, int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(), nullptr, nullptr, 0, 0,
+                                0);
 }
 
 // ---------------------------------------------------------------------
@@ -219,7 +224,7 @@ __global__ __launch_bounds__(256) void ll_combine_fused_kernel(CombineSendArgs s
             dyn_lds[le] = (lr & 0xffffffffll) > 0 ? int(lr >> 32) : 0;
         }
         lds_barrier();
-        combine_recv_piece(ra, int64_t(block) * 4 + wave_in_block(), sa.x, dyn_lds, sa.rank * sa.num_local_experts,
+        combine_recv_piece<false>(ra, int64_t(block) * 4 + wave_in_block(), sa.x, dyn_lds, sa.rank * sa.num_local_experts,
                            sa.num_local_experts, int64_t(sa.max_tokens) * sa.num_ranks);
     } else {
         combine_send_rows(sa, block - num_recv_blocks, int(gridDim.x) - num_recv_blocks, true);
@@ -347,7 +352,11 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
                                                       num_max_dispatch_tokens_per_rank, accumulate, out);
     const int waves = 4;  // block shape makes no measurable difference (1..16 waves: within 5 %)
     const int64_t blocks = (int64_t(num_tokens) * ra.pieces_per_row + waves - 1) / waves;
-    ll_combine_recv_kernel<<<dim3(unsigned(blocks)), waves * kWave, 0, reinterpret_cast<hipStream_t>(stream)>>>(ra);
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    if (int64_t(num_tokens) * num_topk * hidden * 2 > kStreamBytes)
+        ll_combine_recv_kernel<true><<<dim3(unsigned(blocks)), waves * kWave, 0, hs>>>(ra);
+    else
+        ll_combine_recv_kernel<false><<<dim3(unsigned(blocks)), waves * kWave, 0, hs>>>(ra);
     EP_LAUNCH_CHECK();
     return 0;
 }

@@ -111,6 +111,7 @@ __global__ __launch_bounds__(kMetaThreads) void combine_positions_kernel(
 // Reference: the zero_() + index_add_ of deep_ep/buffer.py:1542-1557, which
 // accumulates in bf16 through atomics in arrival order.
 // ---------------------------------------------------------------------
+template <bool kStream>  // the returned rows exceed what the caches hold: read them with the non-temporal hint
 __global__ __launch_bounds__(kMetaThreads) void combine_reduce_kernel(
     const uint8_t* __restrict__ recv_x, const float* __restrict__ recv_w,
     const uint8_t* __restrict__ is_token_in_rank, const int32_t* __restrict__ row_of_pair,
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(kMetaThreads) void combine_reduce_kernel(
                     const int src_lane = __builtin_ctzll(present);
                     present &= present - 1;
                     rows[u] = __builtin_amdgcn_readlane(int(my_row), src_lane);
-                    if (lane_live) v[u] = load_global_u32x4(recv_x + int64_t(rows[u]) * row_bytes + off);
+                    if (lane_live) v[u] = load_u32x4<kStream>(recv_x + int64_t(rows[u]) * row_bytes + off);
                     n = u + 1;
                 }
             }
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(kMetaThreads) void combine_reduce_kernel(
         u32x4 o;
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
-        *reinterpret_cast<u32x4*>(out_x + int64_t(t) * row_bytes + off) = o;
+        store_u32x4<kStream>(out_x + int64_t(t) * row_bytes + off, o);
     }
     if (weights_here && lane < num_topk) out_w[int64_t(t) * num_topk + lane] = w_acc;
 }
@@ -269,10 +270,14 @@ int deepep_combine_reduce(const void* recv_x, const float* recv_topk_weights, co
     const int pieces = (hidden * 2 + 1023) / 1024;
     const int64_t blocks = (int64_t(num_tokens) * pieces + (kMetaThreads / kWave) - 1) / (kMetaThreads / kWave);
     EP_HOST_ASSERT(blocks < (int64_t(1) << 31));
-    combine_reduce_kernel<<<dim3(unsigned(blocks)), kMetaThreads, 0, hs>>>(
-        reinterpret_cast<const uint8_t*>(recv_x), recv_topk_weights, is_token_in_rank, row_of_pair,
-        reinterpret_cast<const uint8_t*>(bias_0), reinterpret_cast<const uint8_t*>(bias_1), num_tokens, hidden,
-        num_topk, num_ranks, max_rows, pieces, reinterpret_cast<uint8_t*>(combined_x), combined_topk_weights);
+#define DEEPEP_LAUNCH_REDUCE(STREAM)                                                                          \
+    combine_reduce_kernel<STREAM><<<dim3(unsigned(blocks)), kMetaThreads, 0, hs>>>(                             \
+        reinterpret_cast<const uint8_t*>(recv_x), recv_topk_weights, is_token_in_rank, row_of_pair,               \
+        reinterpret_cast<const uint8_t*>(bias_0), reinterpret_cast<const uint8_t*>(bias_1), num_tokens, hidden,  \
+        num_topk, num_ranks, max_rows, pieces, reinterpret_cast<uint8_t*>(combined_x), combined_topk_weights)
+    if (max_rows * hidden * 2 > kStreamBytes) DEEPEP_LAUNCH_REDUCE(true);
+    else DEEPEP_LAUNCH_REDUCE(false);
+#undef DEEPEP_LAUNCH_REDUCE
     EP_LAUNCH_CHECK();
     return 0;
 }

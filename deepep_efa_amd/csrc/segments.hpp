@@ -278,7 +278,8 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
     }
 }
 
-// One workgroup per described row (looping only if there are more rows than workgroups).
+// One workgroup per described row (looping only if there are more rows than workgroups).  Only
+// batches too large for the caches come here, so the payload streams.
 static __global__ __launch_bounds__(1024) void ll_rows_flat_kernel(
     const int32_t* __restrict__ flat, int num_segments, const RowDesc* __restrict__ desc,
     const uint8_t* __restrict__ src, int64_t src_stride, int num_vec, uint8_t* __restrict__ dst_primary,
@@ -295,14 +296,13 @@ static __global__ __launch_bounds__(1024) void ll_rows_flat_kernel(
         } else {
             o = dst_secondary + int64_t(-(d.dst_row + 1)) * dst_stride;
         }
-        const u32x4* sv = reinterpret_cast<const u32x4*>(s);
-        u32x4* ov = reinterpret_cast<u32x4*>(o);
         // threads [0, data_threads) move the payload; when the launch carries extra threads beyond
         // them, those move scales and the source index in the same pass instead of a second one
         const int data_threads = extra_threads > 0 ? int(blockDim.x) - extra_threads : int(blockDim.x);
         const int tid = threadIdx.x;
         if (tid < data_threads)
-            for (int v = tid; v < num_vec; v += data_threads) ov[v] = sv[v];
+            for (int v = tid; v < num_vec; v += data_threads)
+                store_u32x4<true>(o + int64_t(v) * 16, load_u32x4<true>(s + int64_t(v) * 16));
         if (extra_threads == 0 || tid >= data_threads) {
             const int t2 = extra_threads > 0 ? tid - data_threads : tid;
             const int step = extra_threads > 0 ? extra_threads : int(blockDim.x);
