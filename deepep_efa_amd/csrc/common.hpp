@@ -2,6 +2,7 @@
 // gfx950 only: 64-lane wavefronts, DPP lane exchange, hardware OCP-FP8 and
 // BF16 pack conversions.
 #pragma once
+#include <cstdlib>
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -97,8 +98,15 @@ __device__ __forceinline__ void store_u32x4(uint8_t* p, u32x4 v) {
     if constexpr (kStream) __builtin_nontemporal_store(v, (global_u32x4*)(p));
     else *(global_u32x4*)(p) = v;
 }
-// Traffic above which a kernel streams (the memory-side cache holds 256 MB).
-constexpr int64_t kStreamBytes = int64_t(192) << 20;
+// Traffic above which a kernel streams (the memory-side cache holds 256 MB).  DEEPEP_STREAM_MB
+// overrides the bound, for tuning.
+inline int64_t stream_bytes() {
+    static const int64_t v = [] {
+        const char* s = getenv("DEEPEP_STREAM_MB");
+        return (s != nullptr ? int64_t(atoll(s)) : int64_t(192)) << 20;
+    }();
+    return v;
+}
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load and store of the wave, which stalls kernels that keep row loads in

@@ -357,7 +357,7 @@ int deepep_pack_rows(const void* src, const void* scale_src, const int64_t* sort
         reinterpret_cast<const uint8_t*>(src), reinterpret_cast<const uint8_t*>(scale_src), sorted_token_ids,      \
         num_rows_dev, max_rows, num_src_rows, row_bytes, scale_row_bytes, reinterpret_cast<uint8_t*>(dst),         \
         reinterpret_cast<uint8_t*>(scale_dst))
-    if (max_rows * row_bytes > kStreamBytes) DEEPEP_LAUNCH_PACK(true);
+    if (max_rows * row_bytes > stream_bytes()) DEEPEP_LAUNCH_PACK(true);
     else DEEPEP_LAUNCH_PACK(false);
 #undef DEEPEP_LAUNCH_PACK
     EP_LAUNCH_CHECK();

@@ -353,7 +353,7 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
     const int waves = 4;  // block shape makes no measurable difference (1..16 waves: within 5 %)
     const int64_t blocks = (int64_t(num_tokens) * ra.pieces_per_row + waves - 1) / waves;
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
-    if (int64_t(num_tokens) * num_topk * hidden * 2 > kStreamBytes)
+    if (int64_t(num_tokens) * num_topk * hidden * 2 > stream_bytes())
         ll_combine_recv_kernel<true><<<dim3(unsigned(blocks)), waves * kWave, 0, hs>>>(ra);
     else
         ll_combine_recv_kernel<false><<<dim3(unsigned(blocks)), waves * kWave, 0, hs>>>(ra);

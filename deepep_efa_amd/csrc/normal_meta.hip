@@ -275,7 +275,7 @@ int deepep_combine_reduce(const void* recv_x, const float* recv_topk_weights, co
         reinterpret_cast<const uint8_t*>(recv_x), recv_topk_weights, is_token_in_rank, row_of_pair,               \
         reinterpret_cast<const uint8_t*>(bias_0), reinterpret_cast<const uint8_t*>(bias_1), num_tokens, hidden,  \
         num_topk, num_ranks, max_rows, pieces, reinterpret_cast<uint8_t*>(combined_x), combined_topk_weights)
-    if (max_rows * hidden * 2 > kStreamBytes) DEEPEP_LAUNCH_REDUCE(true);
+    if (max_rows * hidden * 2 > stream_bytes()) DEEPEP_LAUNCH_REDUCE(true);
     else DEEPEP_LAUNCH_REDUCE(false);
 #undef DEEPEP_LAUNCH_REDUCE
     EP_LAUNCH_CHECK();
