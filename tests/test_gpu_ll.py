@@ -653,3 +653,23 @@ def poison_outputs_keep_pair_slot(st):
     st.packed_recv_src_info.fill_(-7)
     st.packed_recv_count.fill_(-7)
     st.packed_recv_layout_range.fill_(-7)
+
+
+def test_exchange_metadata_through_the_host_module(rt):
+    """The pybind11 binding returns the same values as the C-ABI call, and rejects a host tensor."""
+    from deepep_efa_amd import deep_ep_cpp
+    r, e, m, rank, cap = 8, 64, 50, 3, 512
+    g = torch.Generator().manual_seed(77)
+    routed = torch.randint(0, m + 1, (r, e), generator=g, dtype=torch.int32)
+    send, recv, totals, remote, records, num_recv, per_expert = deep_ep_cpp.ll_exchange_metadata(routed.cuda(), rank, m, cap)
+    torch.cuda.synchronize()
+    want = O.ll_exchange_metadata(routed, rank, m)
+    n = min(want["total_recv"], cap)
+    assert send.cpu().tolist() == want["send_counts"].tolist() and recv.cpu().tolist() == want["recv_counts"].tolist()
+    assert totals.cpu().tolist() == [want["total_send"], want["total_recv"], 0]
+    assert remote.cpu().tolist() == want["combine_remote_recv_offset"].tolist()
+    assert num_recv.cpu().tolist() == [want["total_recv"], n] and (per_expert == 0).all()
+    for i, key in enumerate(("source_rank", "source_offset", "padded_index", "combine_send_offset")):
+        assert records[i, :n].cpu().tolist() == want[key][:n].tolist(), key
+    with pytest.raises(RuntimeError, match="Assertion"):
+        deep_ep_cpp.ll_exchange_metadata(routed, rank, m, cap)
