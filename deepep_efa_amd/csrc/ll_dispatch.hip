@@ -104,7 +104,7 @@ __device__ __forceinline__ void emit_expert_count(int e, int total, int num_expe
 // workgroup per source.  Deterministic: integer adds and ballots only.
 // ---------------------------------------------------------------------
 constexpr int kMaxTopk = 64;
-constexpr int kFusedMaxEntries = 2048;     // send + receive in one launch up to here
+constexpr int kFusedMaxEntries = 8192;     // send + receive in one launch up to here
 constexpr int kSelfRankMaxEntries = 8192;  // the send kernel ranks its own slots, unaided, up to here
 constexpr int kSendMaxWaves = 16;
 
@@ -640,7 +640,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     // How slots get ranked: up to kSelfRankMaxEntries entries the send kernel sweeps every earlier
     // entry itself; beyond, it sweeps its own chunk on top of the per-chunk histograms.
     const int self_rank_max = self_rank_max_override() > 0 ? self_rank_max_override() : kSelfRankMaxEntries;
-    const int tpc = n <= self_rank_max ? 0 : sweep_chunk_tokens(num_topk);
+    const int tpc = n <= self_rank_max || fused_recv != nullptr ? 0 : sweep_chunk_tokens(num_topk);
     if (tpc > 0) {
         const int chunks = (num_tokens + tpc - 1) / tpc;
         ll_chunk_hist_kernel<<<dim3(chunks, num_src), 1024, size_t(num_experts) * sizeof(int32_t), stream>>>(
@@ -877,6 +877,14 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
     return 0;
 }
 
+int deepep_ll_dispatch_is_single_launch(int num_tokens, int num_topk, int num_experts,
+                                        int num_max_dispatch_tokens_per_rank) {
+    return int64_t(num_tokens) * num_topk <= kFusedMaxEntries &&
+                   int64_t(num_experts) * num_max_dispatch_tokens_per_rank <= kLargeBatchRows
+               ? 1
+               : 0;
+}
+
 int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, int hidden, int num_topk,
                        int num_experts, int num_ranks, int rank, int num_max_dispatch_tokens_per_rank, int row_format,
                        void* recv_staging, int32_t* recv_count, void* send_slots, int32_t* send_count,
@@ -887,7 +895,8 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, i
                        void* stream) {
     clear_error();
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
-    const bool fused = int64_t(num_tokens) * num_topk <= kFusedMaxEntries && max_rows <= kLargeBatchRows;
+    const bool fused = deepep_ll_dispatch_is_single_launch(num_tokens, num_topk, num_experts,
+                                                           num_max_dispatch_tokens_per_rank) != 0;
     if (!fused) {  // the two phases back to back
         if (int rc = deepep_ll_dispatch_send(x, topk_idx, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
                                              num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count,

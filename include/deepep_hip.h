@@ -335,13 +335,20 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
  * send and a receive phase, csrc/kernels/coop_dispatch_send.cuh:304,
  * coop_dispatch_recv.cuh:42).  Arguments are those of the two calls; outputs
  * are identical, with one difference: for small batches
- * (num_tokens * num_topk <= 2048 and num_experts * M <= 2^18) both phases run
+ * (num_tokens * num_topk <= 8192 and num_experts * M <= 2^18) both phases run
  * as one kernel launch, and then this rank's rows for its own experts go
  * straight to their packed position — the own segment of recv_staging is not
  * written (recv_count, send_count, send_slots, pair_slot are written as by
  * deepep_ll_dispatch_send).  Larger batches launch the phases back to back.
  *   workspace          as for deepep_ll_dispatch_send
  *   segment_workspace  as the workspace of deepep_ll_dispatch_recv */
+/* 1 when deepep_ll_dispatch runs a batch of this shape as one kernel launch (and so places the
+ * rank's own segment behind the peers' inside each expert's range), else 0.  No counterpart in
+ * the reference, whose segment order is whatever its atomics produce; layout_range carries the
+ * order either way. */
+int deepep_ll_dispatch_is_single_launch(int num_tokens, int num_topk, int num_experts,
+                                        int num_max_dispatch_tokens_per_rank);
+
 int deepep_ll_dispatch(const void* x, const int64_t* topk_idx,
                        int num_tokens, int hidden, int num_topk, int num_experts,
                        int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,

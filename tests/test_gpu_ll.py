@@ -59,7 +59,8 @@ ONE_CALL = pytest.mark.parametrize("one_call", [False, True], ids=["two_calls", 
 def own_last(one_call, t, k, e, m):
     """The one-call dispatch runs as a single launch for small batches and then places this rank's own
     rows behind the peers' inside each expert's range; otherwise source ranks come in ascending order."""
-    return one_call and t * k <= 2048 and e * m <= (1 << 18)
+    from deepep_efa_amd import _capi
+    return one_call and _capi.load().deepep_ll_dispatch_is_single_launch(t, k, e, m) == 1
 
 
 def poison_outputs(st):
@@ -129,7 +130,7 @@ def check_dispatch(st, want, fmt):
 @pytest.mark.parametrize("r,rank,t,h,k,e", [
     (4, 1, 8, 512, 3, 16), (8, 7, 33, 1024, 4, 64), (2, 0, 1, 512, 1, 2),
     (4, 1, 40, 512, 9, 64),    # K > 8
-    (2, 1, 600, 512, 8, 16),   # T*K > 2048: two launches, the send kernel sweeps every earlier entry
+    (2, 1, 600, 512, 8, 16),   # a mid-sized batch: the send side sweeps every earlier entry, in the single launch too
     (4, 3, 300, 512, 11, 32),  # both
     (2, 0, 1100, 512, 8, 16),  # T*K > 8192: chunk histograms under the send kernel's sweep, small receive path
     (8, 5, 4200, 512, 4, 64),  # E*M > 2^18: receive runs as index kernel + flat row copy
