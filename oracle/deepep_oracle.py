@@ -262,6 +262,9 @@ def per_token_cast_back(x_fp8: torch.Tensor, scales: torch.Tensor) -> torch.Tens
 def quantise_rows(x: torch.Tensor, fmt: int):
     """Payload bytes [T, data_bytes] u8 and scale bytes [T, scale_bytes] u8 of each token row."""
     t = x.shape[0]
+    if t == 0:
+        return (torch.zeros((0, row_data_bytes(x.shape[1], fmt)), dtype=torch.uint8),
+                torch.zeros((0, row_scale_bytes(x.shape[1], fmt)), dtype=torch.uint8))
     if fmt == ROW_BF16:
         return x.contiguous().view(torch.uint8).view(t, x.shape[1] * 2), torch.zeros((t, 0), dtype=torch.uint8)
     q, s = per_token_cast_to_fp8(x, round_scale=fmt != ROW_FP8, use_ue8m0=fmt == ROW_FP8_UE8M0)
