@@ -241,6 +241,10 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain row copy of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--cold-trace", type=int, default=0, metavar="N",
+                    help="only run N eager dispatch / combine pairs, each call after a 512 MiB flush of the caches "
+                         "(writes, or reads with --cold-by-reads), for a rocprofv3 kernel trace")
+    ap.add_argument("--cold-by-reads", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the expert-parallel world; --gpus must be 1 "
@@ -289,6 +293,19 @@ def main():
     meta_args = [_capi.ptr(routed), e, r, rank, t, r * t] + [_capi.ptr(meta_out[n]) for n in (
         "send_counts", "recv_counts", "totals", "combine_remote_recv_offset", "source_rank", "source_offset",
         "padded_index", "combine_send_offset", "num_recv_tokens", "tokens_per_expert")]
+
+    if args.cold_trace > 0:
+        flush = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
+        for i in range(args.cold_trace):
+            for call in (lambda: st.dispatch(x, topk), lambda: st.combine(y, topk, weights, out)):
+                if args.cold_by_reads:
+                    flush.max()
+                else:
+                    flush.fill_(i)
+                call()
+            torch.cuda.synchronize()
+        print(json.dumps({"cold_trace": args.cold_trace, "flush": "reads" if args.cold_by_reads else "writes"}))
+        return
 
     calls = {
         "exchange_metadata": lambda: _capi.check(lib.deepep_ll_exchange_metadata(
