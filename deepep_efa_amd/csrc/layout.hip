@@ -113,6 +113,7 @@ __global__ __launch_bounds__(kLayoutThreads) void layout_reduce_kernel(const int
 //   scatter: the count pass again, this time writing the ids.
 // Ascending token order inside a rank follows from the chunk/wave/lane order.
 // Reference: csrc/kernels/efa_kernels.cu:220-318 (one thread per rank there).
+// Small batches take the one-launch variant further down.
 // ---------------------------------------------------------------------
 constexpr int kSortChunk = 1024;
 
@@ -182,6 +183,76 @@ __global__ __launch_bounds__(256) void routing_sort_scan_kernel(int32_t* __restr
             chunk_table[int64_t(c) * num_ranks + r] = run;
             run += cnt;
         }
+    }
+}
+
+// ---------------------------------------------------------------------
+// The same sort in one launch, for up to 8192 tokens and 64 ranks: one workgroup per destination
+// rank, each thread a run of consecutive tokens.  The workgroup reads the whole membership matrix
+// (a few tens of KiB, from L2), so besides the positions of its own rank's tokens (a scan of one
+// count per thread) it gets the number of memberships of all lower ranks — where its ids start —
+// from the same data, without waiting for anybody.  One barrier; 10 us of three launches become 4.
+// ---------------------------------------------------------------------
+constexpr int kSingleSortTokensPerThread = 8;
+
+// Bit r of the result = is_token_in_rank[t][r] != 0, for up to 64 ranks.
+__device__ __forceinline__ uint64_t membership_mask(const uint8_t* row, int num_ranks) {
+    uint64_t mask = 0;
+    if ((num_ranks & 7) == 0 && (reinterpret_cast<uintptr_t>(row) & 7) == 0) {
+        for (int r8 = 0; r8 < num_ranks; r8 += 8) {
+            uint64_t v = *reinterpret_cast<const uint64_t*>(row + r8);
+            v |= v >> 4, v |= v >> 2, v |= v >> 1;  // any bit of a byte -> its bit 0
+            v &= 0x0101010101010101ull;
+            mask |= ((v * 0x0102040810204080ull) >> 56) << r8;  // gather the eight bit-0s into one byte
+        }
+    } else {
+        for (int r = 0; r < num_ranks; ++r) mask |= uint64_t(row[r] != 0) << r;
+    }
+    return mask;
+}
+
+__global__ __launch_bounds__(kSortChunk) void routing_sort_single_kernel(
+    const uint8_t* __restrict__ is_token_in_rank, int num_tokens, int num_ranks, int tokens_per_thread,
+    int32_t* __restrict__ send_counts, int64_t* __restrict__ send_cumsum, int64_t* __restrict__ sorted_token_ids) {
+    constexpr int kWaves = kSortChunk / kWave;
+    __shared__ int32_t wave_own[kWaves];    // tokens of this rank in each wave
+    __shared__ int32_t wave_lower[kWaves];  // memberships of lower ranks in each wave
+    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
+    const int r = blockIdx.x;
+    const uint64_t lower_mask = (uint64_t(1) << r) - 1;
+    const int first = tid * tokens_per_thread;
+    uint32_t own_bits = 0;  // bit i: token first + i goes to rank r
+    int lower = 0;
+#pragma unroll
+    for (int i = 0; i < kSingleSortTokensPerThread; ++i) {
+        const int t = first + i;
+        if (i < tokens_per_thread && t < num_tokens) {
+            const uint64_t m = membership_mask(is_token_in_rank + int64_t(t) * num_ranks, num_ranks);
+            own_bits |= uint32_t((m >> r) & 1) << i;
+            lower += __popcll(m & lower_mask);
+        }
+    }
+    const int own = __popc(own_bits);
+    const int incl = wave_inclusive_sum(own);
+    const int lower_wave = wave_inclusive_sum(lower);
+    if (lane == kWave - 1) wave_own[w] = incl, wave_lower[w] = lower_wave;
+    lds_barrier();
+    int before = 0, total = 0, base = 0;
+#pragma unroll
+    for (int w2 = 0; w2 < kWaves; ++w2) {
+        const int c = wave_own[w2];
+        if (w2 < w) before += c;
+        total += c;
+        base += wave_lower[w2];
+    }
+    int64_t pos = int64_t(base) + before + incl - own;
+#pragma unroll
+    for (int i = 0; i < kSingleSortTokensPerThread; ++i)
+        if ((own_bits >> i) & 1) sorted_token_ids[pos++] = first + i;
+    if (tid == 0) {
+        send_counts[r] = total;
+        send_cumsum[r] = base;
+        if (r == num_ranks - 1) send_cumsum[num_ranks] = int64_t(base) + total;
     }
 }
 
@@ -308,6 +379,13 @@ int deepep_moe_routing_sort(const uint8_t* is_token_in_rank, int num_tokens, int
     const int chunks = num_tokens == 0 ? 1 : (num_tokens + kSortChunk - 1) / kSortChunk;
     EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(chunks) * num_ranks * 4);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (num_tokens <= kSortChunk * kSingleSortTokensPerThread && num_ranks <= 64) {
+        const int per_thread = num_tokens == 0 ? 1 : (num_tokens + kSortChunk - 1) / kSortChunk;
+        routing_sort_single_kernel<<<num_ranks, kSortChunk, 0, s>>>(is_token_in_rank, num_tokens, num_ranks, per_thread,
+                                                                   send_counts, send_cumsum, sorted_token_ids);
+        EP_LAUNCH_CHECK();
+        return 0;
+    }
     int32_t* table = reinterpret_cast<int32_t*>(workspace);
     const size_t lds = size_t(kSortChunk / kWave) * num_ranks * 4;
     routing_sort_pass_kernel<false><<<chunks, kSortChunk, lds, s>>>(is_token_in_rank, num_tokens, num_ranks, table,
