@@ -31,7 +31,7 @@ __device__ __forceinline__ uint64_t bits_to_bool_bytes(uint32_t b) {
 // ---------------------------------------------------------------------
 __global__ __launch_bounds__(kLayoutThreads) void layout_count_kernel(
     const int64_t* __restrict__ topk_idx, int num_tokens, int num_topk, int num_ranks, int num_experts,
-    int num_nodes, uint8_t* __restrict__ is_token_in_rank, int32_t* __restrict__ partial,
+    uint32_t rank_magic, int num_nodes, uint8_t* __restrict__ is_token_in_rank, int32_t* __restrict__ partial,
     int32_t* __restrict__ per_rank, int32_t* __restrict__ per_node, int32_t* __restrict__ per_expert) {
     extern __shared__ int32_t hist[];  // [E + R + nodes]
     const int tid = threadIdx.x, lane = lane_id();
@@ -39,17 +39,23 @@ __global__ __launch_bounds__(kLayoutThreads) void layout_count_kernel(
     for (int j = tid; j < width; j += kLayoutThreads) hist[j] = 0;
     __syncthreads();
 
-    const int experts_per_rank = num_experts / num_ranks;
     const int t = blockIdx.x * kLayoutThreads + tid;
     uint64_t member[kMaxRankWords] = {0, 0, 0, 0};
     if (t < num_tokens) {
         const int64_t* row = topk_idx + int64_t(t) * num_topk;
-        for (int k = 0; k < num_topk; ++k) {
-            const int64_t e = row[k];
-            if (e >= 0 && e < num_experts) {
-                atomicAdd(&hist[int(e)], 1);
-                const int r = int(e) / experts_per_rank;
-                member[r >> 6] |= uint64_t(1) << (r & 63);
+        for (int k0 = 0; k0 < num_topk; k0 += 8) {
+            int64_t e[8];  // the eight loads of a round in flight before the first is used
+#pragma unroll
+            for (int u = 0; u < 8; ++u) e[u] = k0 + u < num_topk ? row[k0 + u] : -1;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (e[u] < 0 || e[u] >= num_experts) continue;
+                atomicAdd(&hist[int(e[u])], 1);
+                // e / E_l by multiply-high (exact below 2^16 experts); magic 0 stands for E_l == 1
+                const int r = rank_magic != 0 ? int(__umulhi(uint32_t(e[u]), rank_magic)) : int(e[u]);
+#pragma unroll
+                for (int q = 0; q < kMaxRankWords; ++q)
+                    if ((r >> 6) == q) member[q] |= uint64_t(1) << (r & 63);
             }
         }
         uint8_t* out = is_token_in_rank + int64_t(t) * num_ranks;
@@ -95,7 +101,13 @@ __global__ __launch_bounds__(kLayoutThreads) void layout_reduce_kernel(const int
     const int j = blockIdx.x * kLayoutThreads + threadIdx.x;
     if (j >= width) return;
     int sum = 0;
-    for (int p = 0; p < num_partials; ++p) sum += partial[int64_t(p) * width + j];
+    for (int p0 = 0; p0 < num_partials; p0 += 8) {  // eight loads in flight
+        int v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p0 + u < num_partials ? partial[int64_t(p0 + u) * width + j] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += v[u];
+    }
     if (j < num_experts)
         per_expert[j] = sum;
     else if (j < num_experts + num_ranks)
@@ -258,19 +270,29 @@ __global__ __launch_bounds__(kSortChunk) void routing_sort_single_kernel(
 
 // ---------------------------------------------------------------------
 // channel_prefix_matrix: one workgroup per destination rank, one wave per
-// channel, then an in-place prefix over channels.
+// channel (up to sixteen at a time), then an in-place prefix over channels.
 // Reference: csrc/kernels/intranode.cu:90-112.
 // ---------------------------------------------------------------------
-__global__ __launch_bounds__(256) void channel_prefix_kernel(const uint8_t* __restrict__ is_token_in_rank,
-                                                             int num_tokens, int num_ranks, int num_channels,
-                                                             int32_t* __restrict__ cpm) {
+__global__ __launch_bounds__(1024) void channel_prefix_kernel(const uint8_t* __restrict__ is_token_in_rank,
+                                                              int num_tokens, int num_ranks, int num_channels,
+                                                              int32_t* __restrict__ cpm) {
     extern __shared__ int32_t per_channel[];  // [C]
     const int dst = blockIdx.x, lane = lane_id(), w = wave_in_block();
+    const int waves = int(blockDim.x) >> 6;
     const int per = (num_tokens + num_channels - 1) / num_channels;
-    for (int ch = w; ch < num_channels; ch += 4) {
+    for (int ch = w; ch < num_channels; ch += waves) {
         const int begin = min(per * ch, num_tokens), end = min(begin + per, num_tokens);
         int count = 0;
-        for (int t = begin + lane; t < end; t += kWave) count += is_token_in_rank[int64_t(t) * num_ranks + dst] != 0;
+        for (int t0 = begin + lane; t0 < end; t0 += kWave * 8) {  // eight loads in flight per lane
+            uint8_t v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int t = t0 + u * kWave;
+                v[u] = t < end ? is_token_in_rank[int64_t(t) * num_ranks + dst] : uint8_t(0);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) count += v[u] != 0;
+        }
         count = wave_sum(count);
         if (lane == 0) per_channel[ch] = count;
     }
@@ -352,8 +374,12 @@ int deepep_get_dispatch_layout(const int64_t* topk_idx, int num_tokens, int num_
     EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(blocks) * width * 4);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     int32_t* partial = reinterpret_cast<int32_t*>(workspace);
+    const uint32_t experts_per_rank = uint32_t(num_experts / num_ranks);
+    EP_HOST_ASSERT(num_experts < 65536);
+    const uint32_t rank_magic =
+        experts_per_rank == 1 ? 0u : uint32_t(((uint64_t(1) << 32) + experts_per_rank - 1) / experts_per_rank);
     layout_count_kernel<<<blocks, kLayoutThreads, size_t(width) * 4, s>>>(
-        topk_idx, num_tokens, num_topk, num_ranks, num_experts, num_nodes, is_token_in_rank, partial,
+        topk_idx, num_tokens, num_topk, num_ranks, num_experts, rank_magic, num_nodes, is_token_in_rank, partial,
         num_tokens_per_rank, num_tokens_per_rdma_rank, num_tokens_per_expert);
     EP_LAUNCH_CHECK();
     if (blocks == 1) return 0;
@@ -408,7 +434,9 @@ int deepep_channel_prefix_matrix(const uint8_t* is_token_in_rank, int num_tokens
     EP_HOST_ASSERT(num_tokens >= 0 && num_ranks > 0 && num_channels > 0 && num_channels <= 4096);
     EP_HOST_ASSERT(channel_prefix_matrix != nullptr);
     EP_HOST_ASSERT(num_tokens == 0 || is_token_in_rank != nullptr);
-    channel_prefix_kernel<<<num_ranks, 256, size_t(num_channels) * 4, reinterpret_cast<hipStream_t>(stream)>>>(
+    // one wave per channel, up to sixteen at a time
+    const int threads = num_channels >= 16 ? 1024 : ((num_channels + 3) / 4) * 256;
+    channel_prefix_kernel<<<num_ranks, threads, size_t(num_channels) * 4, reinterpret_cast<hipStream_t>(stream)>>>(
         is_token_in_rank, num_tokens, num_ranks, num_channels, channel_prefix_matrix);
     EP_LAUNCH_CHECK();
     return 0;
