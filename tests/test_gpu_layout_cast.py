@@ -3,6 +3,8 @@
 Every call goes through the C ABI (ctypes on libdeepep_hip.so); the expected
 values come from the CPU oracle.  Integer and byte outputs must be bit-exact.
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -133,6 +135,40 @@ def test_routing_sort_channel_prefix(capi, t, r, p):
         capi.check(lib.deepep_channel_prefix_matrix(capi.ptr(dev), t, r, c, capi.ptr(cpm), stream()))
         torch.cuda.synchronize()
         assert torch.equal(cpm.cpu(), O.channel_prefix_matrix(is_in, c))
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("DEEPEP_TEST_RANDOM_SHAPES", "16"))))
+def test_layout_sort_prefix_seeded_random_shapes(capi, seed):
+    """Layout, routing sort and channel prefix on shapes nobody picked by hand (both sort paths)."""
+    g = np.random.default_rng(500 + seed)
+    r = int(g.choice([1, 2, 3, 5, 8, 9, 16, 24, 40, 64, 72, 96]))
+    epr = int(g.choice([1, 2, 3, 8]))
+    e = r * epr
+    k = int(g.integers(1, min(e, 10) + 1))
+    t = int(g.choice([0, 1, 5, 63, 64, 65, 255, 256, 257, 1000, 1025, 3000, 4097, 8192, 8193, 9000]))
+    topk = _topk(t, k, e, seed=seed, drop=int(g.integers(0, 20)))
+    got = run_layout(capi, topk, e, r)
+    want = O.get_dispatch_layout(topk, e, r)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[2], want[2]) and torch.equal(got[3], want[3])
+    assert (got[1] is None) == (want[1] is None) and (want[1] is None or torch.equal(got[1], want[1]))
+    lib = capi.load()
+    is_in = want[3]
+    dev = is_in.cuda()
+    ids = torch.full((max(1, t * r),), -1, dtype=torch.int64, device="cuda")
+    counts = torch.full((r,), -1, dtype=torch.int32, device="cuda")
+    cumsum = torch.full((r + 1,), -1, dtype=torch.int64, device="cuda")
+    ws = torch.empty(max(16, lib.deepep_routing_sort_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
+    capi.check(lib.deepep_moe_routing_sort(capi.ptr(dev), t, r, capi.ptr(ids), capi.ptr(counts), capi.ptr(cumsum),
+                                           capi.ptr(ws), ws.numel(), stream()))
+    torch.cuda.synchronize()
+    w_ids, w_counts, w_cumsum, total = O.moe_routing_sort(is_in)
+    assert torch.equal(counts.cpu(), w_counts) and torch.equal(cumsum.cpu(), w_cumsum)
+    assert torch.equal(ids[:total].cpu(), w_ids) and (ids[total:] == -1).all()
+    c = int(g.choice([1, 3, 10, 12, 17, 40]))
+    cpm = torch.full((r, c), -1, dtype=torch.int32, device="cuda")
+    capi.check(lib.deepep_channel_prefix_matrix(capi.ptr(dev), t, r, c, capi.ptr(cpm), stream()))
+    torch.cuda.synchronize()
+    assert torch.equal(cpm.cpu(), O.channel_prefix_matrix(is_in, c))
 
 
 @pytest.mark.parametrize("rows,row_bytes,scale_bytes", [(4096, 14336, 0), (4096, 7168, 224), (37, 256, 8), (5, 16, 0)])

@@ -7,6 +7,7 @@ must be bit-exact; the combine must match the float32 FMA-chain definition
 bit for bit and the float64 sum within 1e-2 relative.
 """
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -267,7 +268,7 @@ def _random_shape(seed):
     return r, int(g.integers(0, r)), t, m, h, k, e, fmt, int(g.integers(0, min(40, t * k) + 1))
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("DEEPEP_TEST_RANDOM_SHAPES", "24"))))
 @ONE_CALL
 def test_dispatch_and_combine_seeded_random_shapes(rt, seed, one_call):
     """Shapes nobody picked by hand: odd world sizes, hidden sizes with a ragged last piece, more slots
