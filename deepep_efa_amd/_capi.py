@@ -33,7 +33,7 @@ PROTOTYPES = {
     "deepep_ll_dispatch_recv": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _SZ, _VP]),
     "deepep_ll_combine_send": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I64, _VP, _SZ, _VP]),
     "deepep_ll_combine_recv": (_I, [_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP]),
-    "deepep_ll_dispatch_is_single_launch": (_I, [_I, _I, _I, _I]),
+    "deepep_ll_dispatch_is_single_launch": (_I, [_I, _I, _I, _I, _I64]),
     "deepep_ll_dispatch": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                 _VP, _I64, _VP, _SZ, _VP, _SZ, _VP]),
     "deepep_ll_combine": (_I, [_VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _I64, _VP, _SZ,

@@ -206,7 +206,7 @@ __global__ __launch_bounds__(1024) void ll_combine_recv_kernel(CombineRecvArgs a
 }
 
 // ---------------------------------------------------------------------
-// Single-launch combine for small batches (E*M <= 2^18): the reduce workgroups
+// Single-launch combine for small batches (at most 8192 expected rows): the reduce workgroups
 // and the row-return workgroups of the two kernels above in one grid.  No
 // workgroup waits on another: the reduce reads the answers of this rank's own
 // experts straight from x (layout_range says where each segment begins), so the
@@ -233,13 +233,13 @@ __global__ __launch_bounds__(256) void ll_combine_fused_kernel(CombineSendArgs s
 
 static CombineSendArgs make_combine_send_args(const void* x, const int64_t* layout_range, int hidden, int num_experts,
                                               int num_ranks, int rank, int max_tokens, void* combine_staging,
-                                              void* combine_send_slots) {
+                                              void* combine_send_slots, int64_t expected_rows) {
     CombineSendArgs sa;
     sa.x = reinterpret_cast<const uint8_t*>(x);
     sa.layout_range = layout_range;
     sa.hidden = hidden, sa.num_local_experts = num_experts / num_ranks, sa.num_ranks = num_ranks, sa.rank = rank;
     sa.max_tokens = max_tokens;
-    sa.parts_log2 = choose_row_parts_log2(int64_t(num_experts) * max_tokens, int64_t(hidden) * 2);
+    sa.parts_log2 = choose_row_parts_log2(estimated_rows(expected_rows, num_experts, max_tokens), int64_t(hidden) * 2);
     sa.combine_staging = reinterpret_cast<uint8_t*>(combine_staging);
     sa.combine_send_slots = reinterpret_cast<uint8_t*>(combine_send_slots);
     return sa;
@@ -307,7 +307,8 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
     const int num_local_experts = num_experts / num_ranks;
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
-    if (max_rows > kLargeBatchRows && workspace != nullptr) {
+    const bool large = estimated_rows(expected_rows, num_experts, num_max_dispatch_tokens_per_rank) > kLargeBatchRows;
+    if (large && workspace != nullptr) {
         EP_HOST_ASSERT(workspace_bytes >= size_t(segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank)));
         EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
         int32_t* flat = reinterpret_cast<int32_t*>(workspace);
@@ -330,9 +331,9 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
     }
     const CombineSendArgs sa = make_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
                                                       num_max_dispatch_tokens_per_rank, combine_staging,
-                                                      combine_send_slots);
+                                                      combine_send_slots, expected_rows);
     int64_t blocks = ((max_rows << sa.parts_log2) + 3) / 4;
-    const int64_t cap = max_rows > kLargeBatchRows ? 4096 : 1024;
+    const int64_t cap = large ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, 0, hs>>>(sa);
     EP_LAUNCH_CHECK();
@@ -370,7 +371,8 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     // measured as whole calls the single launch wins up to this bound (512 tokens: 36 us against 40 for
     // the phases back to back), although each phase timed alone on cache-warm data suggests otherwise
-    if (max_rows > kLargeBatchRows) {  // the two phases back to back
+    if (estimated_rows(expected_rows, num_experts, num_max_dispatch_tokens_per_rank) > kLargeBatchRows) {
+        // the two phases back to back
         if (int rc = deepep_ll_combine_send(x, layout_range, hidden, num_experts, num_ranks, rank,
                                             num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots,
                                             expected_rows, workspace, workspace_bytes, stream))
@@ -386,7 +388,7 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
         return rc;
     const CombineSendArgs sa = make_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
                                                       num_max_dispatch_tokens_per_rank, combine_staging,
-                                                      combine_send_slots);
+                                                      combine_send_slots, expected_rows);
     const CombineRecvArgs ra = make_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens,
                                                       hidden, num_topk, num_experts,
                                                       num_max_dispatch_tokens_per_rank, accumulate, out);

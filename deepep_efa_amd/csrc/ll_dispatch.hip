@@ -554,7 +554,7 @@ __global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a) {
 }
 
 // ---------------------------------------------------------------------
-// Single-launch dispatch for small batches (T*K <= 2048, E*M <= 2^18): the send
+// Single-launch dispatch for small batches (T*K <= 8192, at most 8192 expected rows): the send
 // workgroups, the counting workgroup and the receive workgroups of the two
 // kernels above in one grid.  No workgroup waits on another: the receive
 // workgroups copy only the peers' rows (already in the staging area when the
@@ -809,13 +809,15 @@ static int check_recv_args(const void* recv_staging, const int32_t* recv_count, 
 static RecvArgs make_recv_args(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
                                int num_ranks, int max_tokens, int row_format, void* packed_recv_x,
                                void* packed_recv_scales, int32_t* packed_recv_src_info,
-                               int64_t* packed_recv_layout_range, int32_t* packed_recv_count, int32_t* stats) {
+                               int64_t* packed_recv_layout_range, int32_t* packed_recv_count, int32_t* stats,
+                               int64_t expected_rows) {
     RecvArgs ra;
     ra.recv_staging = reinterpret_cast<const uint8_t*>(recv_staging);
     ra.recv_count = recv_count;
     ra.hidden = hidden, ra.num_local_experts = num_experts / num_ranks, ra.num_ranks = num_ranks;
     ra.max_tokens = max_tokens, ra.fmt = row_format;
-    ra.parts_log2 = choose_row_parts_log2(int64_t(num_experts) * max_tokens, row_data_bytes(hidden, row_format));
+    ra.parts_log2 = choose_row_parts_log2(estimated_rows(expected_rows, num_experts, max_tokens),
+                                          row_data_bytes(hidden, row_format));
     ra.packed_x = reinterpret_cast<uint8_t*>(packed_recv_x);
     ra.packed_scales = reinterpret_cast<uint8_t*>(packed_recv_scales);
     ra.src_info = packed_recv_src_info, ra.layout_range = packed_recv_layout_range;
@@ -837,7 +839,8 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
     const int num_local_experts = num_experts / num_ranks;
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
-    if (max_rows > kLargeBatchRows && workspace != nullptr) {
+    const bool large = estimated_rows(expected_rows, num_experts, num_max_dispatch_tokens_per_rank) > kLargeBatchRows;
+    if (large && workspace != nullptr) {
         EP_HOST_ASSERT(workspace_bytes >= size_t(segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank)));
         EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
         int32_t* flat = reinterpret_cast<int32_t*>(workspace);
@@ -867,9 +870,9 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
     const RecvArgs ra = make_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
                                        num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                                        packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
-                                       cumulative_local_expert_recv_stats);
+                                       cumulative_local_expert_recv_stats, expected_rows);
     int64_t blocks = ((max_rows << ra.parts_log2) + 3) / 4;
-    const int64_t cap = max_rows > kLargeBatchRows ? 4096 : 1024;
+    const int64_t cap = large ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(num_experts + 1) * sizeof(int32_t);
     ll_recv_kernel<<<dim3(unsigned(blocks) + 1), 256, lds, hs>>>(ra);  // + the metadata workgroup
@@ -878,9 +881,9 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
 }
 
 int deepep_ll_dispatch_is_single_launch(int num_tokens, int num_topk, int num_experts,
-                                        int num_max_dispatch_tokens_per_rank) {
+                                        int num_max_dispatch_tokens_per_rank, int64_t expected_rows) {
     return int64_t(num_tokens) * num_topk <= kFusedMaxEntries &&
-                   int64_t(num_experts) * num_max_dispatch_tokens_per_rank <= kLargeBatchRows
+                   estimated_rows(expected_rows, num_experts, num_max_dispatch_tokens_per_rank) <= kLargeBatchRows
                ? 1
                : 0;
 }
@@ -896,7 +899,7 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, i
     clear_error();
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     const bool fused = deepep_ll_dispatch_is_single_launch(num_tokens, num_topk, num_experts,
-                                                           num_max_dispatch_tokens_per_rank) != 0;
+                                                           num_max_dispatch_tokens_per_rank, expected_rows) != 0;
     if (!fused) {  // the two phases back to back
         if (int rc = deepep_ll_dispatch_send(x, topk_idx, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
                                              num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count,
@@ -922,7 +925,7 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, i
     const RecvArgs ra = make_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
                                        num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                                        packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
-                                       cumulative_local_expert_recv_stats);
+                                       cumulative_local_expert_recv_stats, expected_rows);
     int64_t rows = expected_rows > 0 ? expected_rows : int64_t(num_max_dispatch_tokens_per_rank) * num_topk;
     rows += rows / 8 + 16;
     if (rows > max_rows) rows = max_rows;

@@ -172,8 +172,8 @@ __device__ __forceinline__ void row_part_range(int num_vec, int parts, int part,
 
 // Host-side choice of the row split (log2 of the parts): small problems cannot fill the chip with
 // one wave per row.
-inline int choose_row_parts_log2(int64_t max_rows, int64_t row_bytes) {
-    if (max_rows > (int64_t(1) << 18)) return 0;
+inline int choose_row_parts_log2(int64_t estimated_rows, int64_t row_bytes) {
+    if (estimated_rows > 8192) return 0;
     if (const char* s = getenv("DEEPEP_ROW_PARTS")) {
         const int v = atoi(s);
         if (v == 1) return 0;
@@ -322,8 +322,15 @@ __host__ __device__ inline int64_t segment_workspace_bytes(int num_experts, int 
     return flat_bytes + int64_t(num_experts) * max_tokens * int64_t(sizeof(RowDesc));
 }
 
-// Rows above this bound on E*M take the index + flat-copy pair instead of the single fused kernel.
-constexpr int64_t kLargeBatchRows = int64_t(1) << 18;
+// Estimated rows above this bound take the index + flat-copy pair instead of the single fused kernel.
+constexpr int64_t kLargeBatchRows = 8192;
+
+// Rows a call will probably move: the caller's hint or, without one, a guess from the capacity
+// (E * M slots, of which a balanced world fills one in 32 at top-8 of 256 experts).  Only the
+// choice between equivalent kernels and the grid sizes depend on it.
+inline int64_t estimated_rows(int64_t expected_rows, int64_t num_experts, int64_t max_tokens) {
+    return expected_rows > 0 ? expected_rows : num_experts * max_tokens / 32;
+}
 
 inline unsigned flat_grid_blocks(int64_t expected_rows, int64_t max_rows, int max_tokens) {
     int64_t want = expected_rows > 0 ? expected_rows : int64_t(max_tokens) * 8;

@@ -71,9 +71,9 @@ class LowLatencyState:
         self.pair_slot = torch.full((m, s.num_topk), -1, **i32)
         self.workspace = torch.empty(max(256, lib.deepep_ll_dispatch_workspace_bytes(m, s.num_topk, e)), **u8)
         # index + flat-copy scratch of the receive / combine-send kernels, only needed for large batches
-        self.segment_workspace = (torch.empty(lib.deepep_ll_segment_workspace_bytes(e, m), **u8)
-                                  if e * m > (1 << 18) else None)
         self.expected_rows = m * s.num_topk
+        self.segment_workspace = (torch.empty(lib.deepep_ll_segment_workspace_bytes(e, m), **u8)
+                                  if self.expected_rows > 8192 else None)
         if s.fmt == ROW_BF16:
             self.packed_recv_x = torch.empty((el, r * m, h), dtype=torch.bfloat16, device=device)
             self.packed_recv_scales = None

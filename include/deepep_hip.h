@@ -243,9 +243,11 @@ int deepep_ll_dispatch_send(const void* x, const int64_t* topk_idx,
  *   packed_recv_count        [E_l] int32 (out)
  *   cumulative_local_expert_recv_stats [E_l] int32, += count, or NULL
  * Rows at or beyond packed_recv_count[e] are left untouched.
- *   expected_rows  launch-sizing hint only (0 = unknown); any value gives the same result.
- *   workspace      deepep_ll_segment_workspace_bytes(E, M) bytes, or NULL.  With it, batches
- *                  whose E*M exceeds 2^18 run as an index kernel plus a flat row copy (faster
+ *   expected_rows  the number of rows the caller expects this call to move (0 = unknown: E*M/32 is
+ *                  assumed); it sizes the grids and picks between equivalent kernels, and any
+ *                  value gives the same result.
+ *   workspace      deepep_ll_segment_workspace_bytes(E, M) bytes, or NULL.  With it, calls
+ *                  expecting more than 8192 rows run as an index kernel plus a flat row copy (faster
  *                  when bandwidth-bound); without it one fused kernel is used at every size.
  * Replaces ll_recv_unpack_v2 (csrc/kernels/efa_kernels.cu:2121-2231;
  * kernels :877-1389) and a2a_dispatch_recv (csrc/deep_ep.cpp:3709,
@@ -335,7 +337,7 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
  * send and a receive phase, csrc/kernels/coop_dispatch_send.cuh:304,
  * coop_dispatch_recv.cuh:42).  Arguments are those of the two calls; outputs
  * are identical, with one difference: for small batches
- * (num_tokens * num_topk <= 8192 and num_experts * M <= 2^18) both phases run
+ * (num_tokens * num_topk <= 8192 and at most 8192 rows expected) both phases run
  * as one kernel launch, and then this rank's rows for its own experts go
  * straight to their packed position — the own segment of recv_staging is not
  * written (recv_count, send_count, send_slots, pair_slot are written as by
@@ -347,7 +349,7 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
  * the reference, whose segment order is whatever its atomics produce; layout_range carries the
  * order either way. */
 int deepep_ll_dispatch_is_single_launch(int num_tokens, int num_topk, int num_experts,
-                                        int num_max_dispatch_tokens_per_rank);
+                                        int num_max_dispatch_tokens_per_rank, int64_t expected_rows);
 
 int deepep_ll_dispatch(const void* x, const int64_t* topk_idx,
                        int num_tokens, int hidden, int num_topk, int num_experts,
@@ -365,8 +367,8 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx,
  * whose remote experts' answers are already in combine_staging when the call
  * is made (the reference: Buffer::low_latency_combine,
  * csrc/deep_ep.cpp:1798-1920; kernel phases csrc/kernels/coop_combine_send.cuh:37,
- * coop_combine_recv.cuh:72).  `out` is identical to the two calls'.  For
- * num_experts * M <= 2^18 both phases run as one kernel launch, and then the
+ * coop_combine_recv.cuh:72).  `out` is identical to the two calls'.  When
+ * at most 8192 rows are expected both phases run as one kernel launch, and then the
  * answers of this rank's own experts are read from x directly — the own
  * experts' part of combine_staging is neither written nor read.  Larger
  * batches launch the phases back to back. */

@@ -61,7 +61,7 @@ def own_last(one_call, t, k, e, m):
     """The one-call dispatch runs as a single launch for small batches and then places this rank's own
     rows behind the peers' inside each expert's range; otherwise source ranks come in ascending order."""
     from deepep_efa_amd import _capi
-    return one_call and _capi.load().deepep_ll_dispatch_is_single_launch(t, k, e, m) == 1
+    return one_call and _capi.load().deepep_ll_dispatch_is_single_launch(t, k, e, m, m * k) == 1
 
 
 def poison_outputs(st):
@@ -134,7 +134,7 @@ def check_dispatch(st, want, fmt):
     (2, 1, 600, 512, 8, 16),   # a mid-sized batch: the send side sweeps every earlier entry, in the single launch too
     (4, 3, 300, 512, 11, 32),  # both
     (2, 0, 1100, 512, 8, 16),  # T*K > 8192: chunk histograms under the send kernel's sweep, small receive path
-    (8, 5, 4200, 512, 4, 64),  # E*M > 2^18: receive runs as index kernel + flat row copy
+    (8, 5, 4200, 512, 4, 64),  # more than 8192 expected rows: receive runs as index kernel + flat row copy
     (8, 2, 20, 512, 4, 512),   # more than 256 segments: 16 counts per lane in the register segment table
     (16, 9, 12, 512, 6, 1024),  # the most experts the path takes
     (1, 0, 16, 512, 2, 4),     # a world of one rank: every row is the rank's own
@@ -550,7 +550,7 @@ def test_empty_batch(rt, one_call):
 
 
 def test_large_batch_without_the_segment_workspace(rt, oracle_c):
-    """E*M > 2^18 slots but no workspace for the row index: receive and row return fall back to the
+    """A large batch but no workspace for the row index: receive and row return fall back to the
     kernels of the small-batch path and must give the same answers."""
     r, rank, t, h, k, e = 8, 5, 4200, 512, 4, 64
     x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=77, drop=10)
@@ -675,3 +675,38 @@ def test_exchange_metadata_through_the_host_module(rt):
         assert records[i, :n].cpu().tolist() == want[key][:n].tolist(), key
     with pytest.raises(RuntimeError, match="Assertion"):
         deep_ep_cpp.ll_exchange_metadata(routed, rank, m, cap)
+
+
+@pytest.mark.parametrize("hint", ["batch", "unknown", "huge"])
+def test_capacity_far_above_the_batch(rt, hint):
+    """A caller may size M for its largest batch and dispatch a small one.  The kernels are picked from the
+    expected-rows hint, not from the capacity; every hint gives the oracle's rows (the hint only decides
+    whether the one-call dispatch is a single launch, i.e. where an expert's own segment sits)."""
+    r, rank, t, m, h, k, e = 8, 2, 40, 5000, 512, 4, 64
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=4242, drop=7)
+    shape = rt.ll.LLShape(num_ranks=r, rank=rank, num_experts=e, max_tokens=m, hidden=h, num_topk=k, fmt=O.ROW_FP8)
+    st = rt.ll.LowLatencyState(shape)
+    st.expected_rows = {"batch": t * k, "unknown": 0, "huge": 10 ** 6}[hint]
+    if st.segment_workspace is None:
+        st.segment_workspace = torch.empty(rt.capi.load().deepep_ll_segment_workspace_bytes(e, m), dtype=torch.uint8,
+                                           device="cuda")
+    world = rt.lb.LoopbackWorld(r, rank, seed=0)
+    world.set_inputs(x_all.cuda(), topk_all.cuda())
+    x, topk = world.own_inputs()
+    run_dispatch(st, world, x, topk, None, one_call=True)
+    single = rt.capi.load().deepep_ll_dispatch_is_single_launch(t, k, e, m, st.expected_rows) == 1
+    assert single == (hint == "batch")
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, O.ROW_FP8, own_last=single)
+    check_dispatch(st, want, O.ROW_FP8)
+    # combine with identity experts
+    epr = e // r
+    y = torch.zeros((epr, r * m, h), dtype=torch.bfloat16)
+    count = st.packed_recv_count.cpu()
+    for le in range(epr):
+        n = int(count[le])
+        y[le, :n] = O.per_token_cast_back(st.packed_recv_x[le, :n].cpu(), st.packed_recv_scales[le, :n].cpu())
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    run_combine(st, world, y.cuda(), topk_all[rank].cuda(), w_all[rank].cuda(), out, mode=0, one_call=True)
+    wsum = w_all[rank].masked_fill(topk_all[rank] == -1, 0).sum(1).view(-1, 1)
+    live = wsum.view(-1) > 0
+    assert O.calc_diff((x_all[rank].float() * wsum)[live], out.cpu().float()[live]) < 2e-3
