@@ -487,7 +487,7 @@ struct Buffer {
             c.packed_recv_src_info.data_ptr<int>(), c.packed_recv_layout_range.data_ptr<int64_t>(),
             c.packed_recv_count.data_ptr<int>(),
             cumulative_local_expert_recv_stats.has_value() ? cumulative_local_expert_recv_stats->data_ptr<int>() : nullptr,
-            /*expected_rows=*/int64_t(num_tokens) * num_topk, c.workspace.data_ptr(),
+            /*expected_rows=*/std::max<int64_t>(num_tokens, 1) * num_topk, c.workspace.data_ptr(),
             size_t(c.workspace.numel()), c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
             c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));
         c.dispatched = true;
@@ -565,7 +565,7 @@ struct Buffer {
                                     topk_weights.data_ptr<float>(), c.pair_slot.data_ptr<int>(), num_combined_tokens,
                                     hidden, num_topk, num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,
                                     /*accumulate=*/0, c.combine_staging.data_ptr(), c.combine_send_slots.data_ptr(),
-                                    combined_x.data_ptr(), /*expected_rows=*/int64_t(num_combined_tokens) * num_topk,
+                                    combined_x.data_ptr(), /*expected_rows=*/std::max<int64_t>(num_combined_tokens, 1) * num_topk,
                                     c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
                                     c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));
 
