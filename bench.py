@@ -27,13 +27,14 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 
-def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0):
+def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0, packed=None):
     """Bytes each entry point must move (reads + writes), from the generated routing.
     p = live (token,k) pairs of this rank, rv = rows this rank receives, own = rows it sends to itself.
     The one-call entries handle the own rows once: quantised straight into the packed tensors on dispatch,
     read straight from the expert outputs on combine."""
     g = h // 128
-    packed = h + 4 * g + 4
+    if packed is None:  # FP8 payload + float32 scales + source index
+        packed = h + 4 * g + 4
     small = e * 4 + (e // r) * r * 8 + (e // r) * 4
     return {
         "dispatch_send": t * 2 * h + t * k * 8 + p * stride + t * k * 4 + e * 4,
@@ -241,6 +242,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain row copy of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--row-format", choices=["fp8", "bf16", "fp8_pow2", "fp8_ue8m0"], default="fp8",
+                    help="dispatch payload (the headline workload is fp8); other formats skip the CPU baseline")
     ap.add_argument("--cold-trace", type=int, default=0, metavar="N",
                     help="only run N eager dispatch / combine pairs, each call after a 512 MiB flush of the caches "
                          "(writes, or reads with --cold-by-reads), for a rocprofv3 kernel trace")
@@ -264,7 +267,11 @@ def main():
         print(json.dumps(bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args)))
         return
     t, h, k, e, r, rank = args.tokens, args.hidden, args.topk, args.experts, args.ranks, args.rank
-    shape = ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8)
+    fmt = {"fp8": ll_runtime.ROW_FP8, "bf16": ll_runtime.ROW_BF16, "fp8_pow2": ll_runtime.ROW_FP8_POW2,
+           "fp8_ue8m0": ll_runtime.ROW_FP8_UE8M0}[args.row_format]
+    if fmt != ll_runtime.ROW_FP8:
+        args.no_cpu_baseline = True
+    shape = ll_runtime.LLShape(r, rank, e, t, h, k, fmt)
     st = ll_runtime.LowLatencyState(shape)
     world = loopback.LoopbackWorld(r, rank, seed=args.seed)
     world.synthesise(t, h, k, e)
@@ -427,7 +434,7 @@ def main():
     us_per_step = graph_us if graph_us is not None else eager_us
     us_per_phase_step = graph_phase_us if graph_phase_us is not None else eager_phase_us
 
-    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r, own)
+    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r, own, packed=st.data_bytes + st.scale_bytes + 4)
     kernels = {n: {"us": round(per_call[n], 2), "bytes": nbytes[n],
                    "GBps": round(nbytes[n] / per_call[n] / 1e3, 1)} for n in calls}
     dom = max(step_calls, key=per_call.get)
@@ -443,7 +450,8 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "fp8_e4m3 dispatch (f32 scale math), bf16 combine (f32 accumulate)",
+        "dtype": ("fp8_e4m3 dispatch (f32 scale math)" if fmt != ll_runtime.ROW_BF16 else "bf16 dispatch") +
+                 ", bf16 combine (f32 accumulate)",
         "data": "synthetic",
         "config": {"workload": "LL dispatch+combine, one GPU's share of EP=32: 128 tokens x 7168, top-8 of 256 "
                                "experts, 8 local experts; 31 peers synthesised in HBM from a seed",
