@@ -142,6 +142,9 @@ def check_dispatch(st, want, fmt):
     (2, 1, 9, 512, 64, 128),   # the most selections per token
     (4, 2, 24, 1536, 4, 16),   # hidden not a multiple of 1024: the last row piece is partly empty
     (8, 3, 17, 5120, 8, 64),
+    (128, 77, 9, 512, 4, 128),   # many ranks, one expert each
+    (256, 3, 5, 512, 2, 512),
+    (512, 500, 3, 512, 2, 1024),  # the widest world the path takes
 ])
 @ONE_CALL
 def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
