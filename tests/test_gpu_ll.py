@@ -398,7 +398,9 @@ def test_reference_recipe_roundtrip(rt, use_fp8, one_call):
                                             (8, 3, 4200, 512, 4, 64),   # large-batch combine-send path
                                             (4, 2, 40, 512, 11, 64),    # more than eight selections per token
                                             (8, 6, 20, 512, 4, 512),    # more than 256 segments
-                                            (4, 1, 33, 1536, 5, 32)])   # hidden not a multiple of 512
+                                            (4, 1, 33, 1536, 5, 32),    # hidden not a multiple of 512
+                                            (128, 77, 9, 512, 4, 128),  # many ranks, one expert each
+                                            (512, 500, 3, 512, 2, 1024)])
 @ONE_CALL
 def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e, one_call):
     """Seeded expert outputs along the dispatch routing; combine vs the float32 chain and the float64 sum."""
