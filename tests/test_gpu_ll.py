@@ -467,9 +467,10 @@ def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e, one_ca
 
 
 @ONE_CALL
-def test_ll_config_full_size(rt, one_call):
-    """One GPU's share of EP=32 at 128 tokens x 7168, top-8 of 256 experts, seeded world."""
-    r, rank, t, h, k, e = 32, 11, 128, 7168, 8, 256
+@pytest.mark.parametrize("e,rank", [(256, 11), (288, 7)])  # 288 experts: the reference's own LL test, nine per rank
+def test_ll_config_full_size(rt, one_call, e, rank):
+    """One GPU's share of EP=32 at 128 tokens x 7168, top-8 of 256 (or 288) experts, seeded world."""
+    r, t, h, k = 32, 128, 7168, 8
     shape = rt.ll.LLShape(r, rank, e, t, h, k, O.ROW_FP8)
     st = rt.ll.LowLatencyState(shape)
     world = rt.lb.LoopbackWorld(r, rank, seed=2024)
