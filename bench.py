@@ -468,6 +468,11 @@ def main():
         "cold_cache_read_flush_us_per_step": round(cold_reads_us, 2),  # the same after 512 MiB of reads
         "cold_cache_read_flush_two_trivial_launches_us": round(cold_reads_floor_us, 2),
         "kernels": kernels,
+        # the reference's own bandwidth accounting (tests/test_low_latency.py:236-242): bytes per valid
+        # selection H + H/128*4 + 16 for the FP8 dispatch and 2H for the combine, over the call's time
+        "reference_formula_GBps": {
+            "dispatch": round(p * (h + h // 128 * 4 + 16) / per_call["dispatch"] / 1e3, 1),
+            "combine": round(p * 2 * h / per_call["combine"] / 1e3, 1)},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
     }
