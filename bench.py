@@ -209,15 +209,19 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args):
     torch.cuda.synchronize()
     p = int((st.pair_slot[:t] >= 0).sum())
     rv = int(st.packed_recv_count.sum())
-    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r)
+    own = int((st.packed_recv_layout_range[:, rank] & 0xFFFFFFFF).sum())
+    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r, own)
     calls = {
         "dispatch_send": lambda: st.dispatch_send(x, topk),
         "dispatch_recv": lambda: st.dispatch_recv(),
         "combine_send": lambda: st.combine_send(y),
         "combine_recv": lambda: st.combine_recv(topk, weights, out),
+        # the one-call entries (what deep_ep.Buffer launches): the rank's own rows are written / read in place
+        "dispatch": lambda: st.dispatch(x, topk),
+        "combine": lambda: st.combine(y, topk, weights, out),
     }
     res = {"workload": "LL dispatch+combine at 4096 tokens x 7168, top-8 of 256 experts, 8 ranks x 32 experts",
-           "pairs_sent": p, "rows_received": rv}
+           "pairs_sent": p, "rows_received": rv, "rows_to_own_experts": own}
     for name, fn in calls.items():
         us = time_calls(torch, fn, max(10, args.steps // 10))
         res[name] = {"us": round(us, 2), "bytes": nbytes[name], "GBps": round(nbytes[name] / us / 1e3, 1),

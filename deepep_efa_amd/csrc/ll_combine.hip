@@ -88,8 +88,9 @@ __device__ __forceinline__ void combine_send_rows(const CombineSendArgs& a, int 
         combine_send_rows_impl<16>(a, block, num_blocks, skip_own);
 }
 
-__global__ __launch_bounds__(256) void ll_combine_send_kernel(CombineSendArgs a) {
-    combine_send_rows(a, blockIdx.x, gridDim.x, false);
+// skip_own: the rows owed to this rank itself stay where they are (the reduce reads them from x).
+__global__ __launch_bounds__(256) void ll_combine_send_kernel(CombineSendArgs a, bool skip_own) {
+    combine_send_rows(a, blockIdx.x, gridDim.x, skip_own);
 }
 
 // ---------------------------------------------------------------------
@@ -198,11 +199,23 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
 }
 
 // kStream: the gathered rows exceed what the caches hold, so they are read (and the result written)
-// with the non-temporal hint.
+// with the non-temporal hint.  own_x != null: the answers of this rank's own experts are read from
+// the expert-output tensor directly (layout_range says where each own segment begins).
 template <bool kStream>
-__global__ __launch_bounds__(1024) void ll_combine_recv_kernel(CombineRecvArgs a) {
-    combine_recv_piece<kStream>(a, int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(), nullptr, nullptr, 0, 0,
-                                0);
+__global__ __launch_bounds__(1024) void ll_combine_recv_kernel(CombineRecvArgs a, const uint8_t* own_x,
+                                                               const int64_t* layout_range, int rank,
+                                                               int num_local_experts, int num_ranks) {
+    extern __shared__ int32_t own_begin[];  // [E_l], with own_x only
+    if (own_x != nullptr) {
+        for (int le = threadIdx.x; le < num_local_experts; le += blockDim.x) {
+            const int64_t lr = layout_range[le * num_ranks + rank];
+            own_begin[le] = (lr & 0xffffffffll) > 0 ? int(lr >> 32) : 0;
+        }
+        lds_barrier();
+    }
+    combine_recv_piece<kStream>(a, int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(), own_x,
+                                own_x != nullptr ? own_begin : nullptr, rank * num_local_experts, num_local_experts,
+                                int64_t(a.max_tokens) * num_ranks);
 }
 
 // ---------------------------------------------------------------------
@@ -296,11 +309,11 @@ using namespace deepep;
 
 extern "C" {
 
-int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidden, int num_experts, int num_ranks,
-                           int rank, int num_max_dispatch_tokens_per_rank, void* combine_staging,
-                           void* combine_send_slots, int64_t expected_rows, void* workspace, size_t workspace_bytes,
-                           void* stream) {
-    clear_error();
+// skip_own: the rows owed to this rank itself are not moved (the reduce will read them from x).
+static int launch_combine_send(const void* x, const int64_t* layout_range, int hidden, int num_experts, int num_ranks,
+                               int rank, int num_max_dispatch_tokens_per_rank, void* combine_staging,
+                               void* combine_send_slots, int64_t expected_rows, void* workspace,
+                               size_t workspace_bytes, bool skip_own, void* stream) {
     if (int rc = check_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
                                          num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots))
         return rc;
@@ -315,7 +328,8 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
         RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) +
                                                    (((int64_t(num_experts) + 1) * 4 + 255) & ~int64_t(255)));
         ll_segment_index_kernel<<<num_experts, kIndexThreads, 0, hs>>>(
-            1, nullptr, layout_range, num_local_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank, nullptr,
+            skip_own ? 2 : 1, nullptr, layout_range, num_local_experts, num_ranks, rank,
+            num_max_dispatch_tokens_per_rank, nullptr,
             nullptr, nullptr, flat, desc);
         EP_LAUNCH_CHECK();
         const int num_vec = hidden * 2 / 16;
@@ -335,15 +349,27 @@ int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidde
     int64_t blocks = ((max_rows << sa.parts_log2) + 3) / 4;
     const int64_t cap = large ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
-    ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, 0, hs>>>(sa);
+    ll_combine_send_kernel<<<dim3(unsigned(blocks)), 256, 0, hs>>>(sa, skip_own);
     EP_LAUNCH_CHECK();
     return 0;
 }
 
-int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx, const float* topk_weights,
-                           const int32_t* pair_slot, int num_tokens, int hidden, int num_topk, int num_experts,
-                           int num_max_dispatch_tokens_per_rank, int accumulate, void* out, void* stream) {
+int deepep_ll_combine_send(const void* x, const int64_t* layout_range, int hidden, int num_experts, int num_ranks,
+                           int rank, int num_max_dispatch_tokens_per_rank, void* combine_staging,
+                           void* combine_send_slots, int64_t expected_rows, void* workspace, size_t workspace_bytes,
+                           void* stream) {
     clear_error();
+    return launch_combine_send(x, layout_range, hidden, num_experts, num_ranks, rank,
+                               num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots, expected_rows,
+                               workspace, workspace_bytes, false, stream);
+}
+
+// own_x != null: the answers of this rank's own experts are read from own_x at the positions
+// layout_range gives, instead of from combine_staging.
+static int launch_combine_recv(const void* combine_staging, const int64_t* topk_idx, const float* topk_weights,
+                               const int32_t* pair_slot, int num_tokens, int hidden, int num_topk, int num_experts,
+                               int num_max_dispatch_tokens_per_rank, int accumulate, void* out, const void* own_x,
+                               const int64_t* layout_range, int rank, int num_ranks, void* stream) {
     if (int rc = check_combine_recv_args(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden,
                                          num_topk, num_experts, num_max_dispatch_tokens_per_rank, out))
         return rc;
@@ -354,12 +380,26 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
     const int waves = 4;  // block shape makes no measurable difference (1..16 waves: within 5 %)
     const int64_t blocks = (int64_t(num_tokens) * ra.pieces_per_row + waves - 1) / waves;
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    const int num_local_experts = own_x != nullptr ? num_experts / num_ranks : 0;
+    const size_t lds = size_t(num_local_experts) * sizeof(int32_t);
+    const uint8_t* own = reinterpret_cast<const uint8_t*>(own_x);
     if (int64_t(num_tokens) * num_topk * hidden * 2 > stream_bytes())
-        ll_combine_recv_kernel<true><<<dim3(unsigned(blocks)), waves * kWave, 0, hs>>>(ra);
+        ll_combine_recv_kernel<true><<<dim3(unsigned(blocks)), waves * kWave, lds, hs>>>(ra, own, layout_range, rank,
+                                                                                        num_local_experts, num_ranks);
     else
-        ll_combine_recv_kernel<false><<<dim3(unsigned(blocks)), waves * kWave, 0, hs>>>(ra);
+        ll_combine_recv_kernel<false><<<dim3(unsigned(blocks)), waves * kWave, lds, hs>>>(ra, own, layout_range, rank,
+                                                                                         num_local_experts, num_ranks);
     EP_LAUNCH_CHECK();
     return 0;
+}
+
+int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx, const float* topk_weights,
+                           const int32_t* pair_slot, int num_tokens, int hidden, int num_topk, int num_experts,
+                           int num_max_dispatch_tokens_per_rank, int accumulate, void* out, void* stream) {
+    clear_error();
+    return launch_combine_recv(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden, num_topk,
+                               num_experts, num_max_dispatch_tokens_per_rank, accumulate, out, nullptr, nullptr, 0, 1,
+                               stream);
 }
 
 int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t* topk_idx, const float* topk_weights,
@@ -372,13 +412,15 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
     // measured as whole calls the single launch wins up to this bound (512 tokens: 36 us against 40 for
     // the phases back to back), although each phase timed alone on cache-warm data suggests otherwise
     if (estimated_rows(expected_rows, num_experts, num_max_dispatch_tokens_per_rank) > kLargeBatchRows) {
-        // the two phases back to back
-        if (int rc = deepep_ll_combine_send(x, layout_range, hidden, num_experts, num_ranks, rank,
-                                            num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots,
-                                            expected_rows, workspace, workspace_bytes, stream))
+        // the two phases back to back, with the single launch's shortcut: the rows owed to this rank
+        // itself are not moved, the reduce reads them from x
+        if (int rc = launch_combine_send(x, layout_range, hidden, num_experts, num_ranks, rank,
+                                         num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots,
+                                         expected_rows, workspace, workspace_bytes, true, stream))
             return rc;
-        return deepep_ll_combine_recv(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden, num_topk,
-                                      num_experts, num_max_dispatch_tokens_per_rank, accumulate, out, stream);
+        return launch_combine_recv(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden, num_topk,
+                                   num_experts, num_max_dispatch_tokens_per_rank, accumulate, out, x, layout_range,
+                                   rank, num_ranks, stream);
     }
     if (int rc = check_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
                                          num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots))

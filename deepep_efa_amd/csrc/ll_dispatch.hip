@@ -391,15 +391,14 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
 }
 
 template <int kFmt>
-__global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs a) {
+__global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs a, DirectOut direct) {
     extern __shared__ int32_t lds_hist[];  // [E], counting workgroups only
     __shared__ SendLds lds;
     if (int(blockIdx.y) == a.num_tokens) {  // the counting row of the grid
         if (blockIdx.x == 0) send_count_block(a, blockIdx.z, lds_hist);
         return;
     }
-    const DirectOut none = {nullptr, nullptr, nullptr};
-    send_token_block<kFmt>(a, none, blockIdx.z, blockIdx.y, blockIdx.x, lds);
+    send_token_block<kFmt>(a, direct, blockIdx.z, blockIdx.y, blockIdx.x, lds);
 }
 
 // ---------------------------------------------------------------------
@@ -547,10 +546,12 @@ __device__ __forceinline__ void recv_rows(const RecvArgs& a, int block, int num_
         recv_rows_impl<16>(a, block, num_copy_blocks, own_topk, own_entries, own_rank, lds, wave_totals);
 }
 
-__global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a) {
-    extern __shared__ int32_t flat[];  // [num_segments + 1], used by the metadata workgroup (the last one)
+// own_topk != null: the send side has already put this rank's own rows at their packed position.
+__global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a, const int64_t* own_topk, int own_entries,
+                                                      int own_rank) {
+    extern __shared__ int32_t flat[];  // [num_segments + 1 + E_l], used by the metadata workgroup (the last one)
     __shared__ int32_t wave_totals[kMaxBlockWaves];
-    recv_rows(a, blockIdx.x, int(gridDim.x) - 1, nullptr, 0, 0, flat, wave_totals);
+    recv_rows(a, blockIdx.x, int(gridDim.x) - 1, own_topk, own_entries, own_rank, flat, wave_totals);
 }
 
 // ---------------------------------------------------------------------
@@ -631,7 +632,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
                             int max_tokens, int row_format, void* recv_staging, int32_t* recv_count,
                             void* send_slots, int32_t* send_count, int32_t* pair_slot, void* workspace,
                             size_t workspace_bytes, hipStream_t stream, const RecvArgs* fused_recv = nullptr,
-                            int64_t fused_recv_wave_items = 0) {
+                            int64_t fused_recv_wave_items = 0, const DirectOut* own_rows_direct = nullptr) {
     const int64_t scratch_bytes = route_scratch_bytes(num_tokens, num_topk, num_experts);
     EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(scratch_bytes) * size_t(num_src));
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
@@ -713,7 +714,11 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
 
     const dim3 grid(blocks_per_token, num_tokens + 1, num_src);  // + the counting workgroup
     const size_t lds = size_t(num_experts) * sizeof(int32_t);
-#define DEEPEP_LAUNCH_SEND(FMT) ll_send_kernel<FMT><<<grid, waves * kWave, lds, stream>>>(sa)
+    // own_rows_direct (the two-launch form of the one-call dispatch): as in the single launch, the rows
+    // for this rank's own experts go straight to their packed position behind the peers' rows
+    EP_HOST_ASSERT(own_rows_direct == nullptr || (num_src == 1 && src_ranks == nullptr));
+    const DirectOut direct = own_rows_direct != nullptr ? *own_rows_direct : DirectOut{nullptr, nullptr, nullptr};
+#define DEEPEP_LAUNCH_SEND(FMT) ll_send_kernel<FMT><<<grid, waves * kWave, lds, stream>>>(sa, direct)
     switch (row_format) {
         case kRowBF16: DEEPEP_LAUNCH_SEND(kRowBF16); break;
         case kRowFP8: DEEPEP_LAUNCH_SEND(kRowFP8); break;
@@ -825,13 +830,16 @@ static RecvArgs make_recv_args(const void* recv_staging, const int32_t* recv_cou
     return ra;
 }
 
-int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
+// own_rank >= 0: this rank's own rows are already at their packed position, behind the peers' rows
+// of each expert (the send side put them there); they are not copied, and own_topk [own_entries] is
+// the rank's routing, from which the small-batch kernel recounts them.
+static int launch_recv_side(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
                             int num_ranks, int num_max_dispatch_tokens_per_rank, int row_format,
                             void* packed_recv_x, void* packed_recv_scales, int32_t* packed_recv_src_info,
                             int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
                             int32_t* cumulative_local_expert_recv_stats, int64_t expected_rows, void* workspace,
-                            size_t workspace_bytes, void* stream) {
-    clear_error();
+                            size_t workspace_bytes, const int64_t* own_topk, int own_entries, int own_rank,
+                            void* stream) {
     if (int rc = check_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
                                  num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                                  packed_recv_src_info, packed_recv_layout_range, packed_recv_count))
@@ -847,7 +855,7 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
         RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) +
                                                    (((int64_t(num_experts) + 1) * 4 + 255) & ~int64_t(255)));
         ll_segment_index_kernel<<<num_experts, kIndexThreads, 0, hs>>>(
-            0, recv_count, nullptr, num_local_experts, num_ranks, 0, num_max_dispatch_tokens_per_rank,
+            0, recv_count, nullptr, num_local_experts, num_ranks, own_rank, num_max_dispatch_tokens_per_rank,
             packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, flat, desc);
         EP_LAUNCH_CHECK();
         const int64_t data_bytes = row_data_bytes(hidden, row_format);
@@ -874,10 +882,25 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
     int64_t blocks = ((max_rows << ra.parts_log2) + 3) / 4;
     const int64_t cap = large ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
-    const size_t lds = size_t(num_experts + 1) * sizeof(int32_t);
-    ll_recv_kernel<<<dim3(unsigned(blocks) + 1), 256, lds, hs>>>(ra);  // + the metadata workgroup
+    const size_t lds = size_t(num_experts + 1 + num_local_experts) * sizeof(int32_t);
+    ll_recv_kernel<<<dim3(unsigned(blocks) + 1), 256, lds, hs>>>(ra, own_rank >= 0 ? own_topk : nullptr, own_entries,
+                                                                 own_rank);  // + the metadata workgroup
     EP_LAUNCH_CHECK();
     return 0;
+}
+
+int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
+                            int num_ranks, int num_max_dispatch_tokens_per_rank, int row_format,
+                            void* packed_recv_x, void* packed_recv_scales, int32_t* packed_recv_src_info,
+                            int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
+                            int32_t* cumulative_local_expert_recv_stats, int64_t expected_rows, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+    clear_error();
+    return launch_recv_side(recv_staging, recv_count, hidden, num_experts, num_ranks,
+                            num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
+                            packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
+                            cumulative_local_expert_recv_stats, expected_rows, workspace, workspace_bytes, nullptr, 0,
+                            -1, stream);
 }
 
 int deepep_ll_dispatch_is_single_launch(int num_tokens, int num_topk, int num_experts,
@@ -900,20 +923,35 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, i
     const int64_t max_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;
     const bool fused = deepep_ll_dispatch_is_single_launch(num_tokens, num_topk, num_experts,
                                                            num_max_dispatch_tokens_per_rank, expected_rows) != 0;
-    if (!fused) {  // the two phases back to back
-        if (int rc = deepep_ll_dispatch_send(x, topk_idx, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
-                                             num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count,
-                                             send_slots, send_count, pair_slot, workspace, workspace_bytes, stream))
-            return rc;
-        return deepep_ll_dispatch_recv(recv_staging, recv_count, hidden, num_experts, num_ranks,
-                                       num_max_dispatch_tokens_per_rank, row_format, packed_recv_x,
-                                       packed_recv_scales, packed_recv_src_info, packed_recv_layout_range,
-                                       packed_recv_count, cumulative_local_expert_recv_stats, expected_rows,
-                                       segment_workspace, segment_workspace_bytes, stream);
-    }
     if (int rc = check_ll_shape(num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
                                 num_max_dispatch_tokens_per_rank, row_format))
         return rc;
+    if (!fused) {
+        // The two phases back to back, with the same placement as the single launch: the send side
+        // writes the rows for this rank's own experts straight to their packed position behind the
+        // peers' rows (whose counts are in recv_count already), and the receive side copies the rest.
+        EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
+        EP_HOST_ASSERT(recv_staging != nullptr && recv_count != nullptr && pair_slot != nullptr && send_count != nullptr);
+        EP_HOST_ASSERT(workspace != nullptr);
+        EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+        EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(send_slots) & 15) == 0);
+        if (int rc = check_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
+                                     num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
+                                     packed_recv_src_info, packed_recv_layout_range, packed_recv_count))
+            return rc;
+        const DirectOut direct = {reinterpret_cast<uint8_t*>(packed_recv_x),
+                                  reinterpret_cast<uint8_t*>(packed_recv_scales), packed_recv_src_info};
+        if (int rc = launch_send_side(x, topk_idx, nullptr, 1, num_tokens, hidden, num_topk, num_experts, num_ranks,
+                                      rank, num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count,
+                                      send_slots, send_count, pair_slot, workspace, workspace_bytes,
+                                      reinterpret_cast<hipStream_t>(stream), nullptr, 0, &direct))
+            return rc;
+        return launch_recv_side(recv_staging, recv_count, hidden, num_experts, num_ranks,
+                                num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
+                                packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
+                                cumulative_local_expert_recv_stats, expected_rows, segment_workspace,
+                                segment_workspace_bytes, topk_idx, num_tokens * num_topk, rank, stream);
+    }
     EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
     EP_HOST_ASSERT(send_count != nullptr && pair_slot != nullptr);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);

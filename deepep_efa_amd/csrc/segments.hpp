@@ -215,8 +215,9 @@ __device__ __forceinline__ int block_exclusive_scan_1024(int v, int32_t* wave_to
 }
 
 // mode 0 (dispatch receive): counts = recv_count; writes layout_range / packed_count / stats;
-//        descriptor = {staging row seg*M + j, packed row e_l*N + begin + j}.
-// mode 1 (combine send): counts and begins from layout_range;
+//        descriptor = {staging row seg*M + j, packed row e_l*N + begin + j}; rank = -1, or the rank
+//        whose own rows are already in the packed tensors.
+// mode 1 (combine send; mode 2: the same without this rank's own rows): counts and begins from layout_range;
 //        descriptor = {expert-output row e_l*N + begin + j, seg*M + j for other ranks or
 //        -(1 + (rank*E_l + e_l)*M + j) for this rank's own rows}.
 static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
@@ -236,9 +237,15 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
             const int64_t lr = layout_in[tid];
             c = int(lr & 0xffffffffll);
             begin_in[tid] = int(lr >> 32);
+            if (mode == 2 && tid % num_ranks == rank) c = 0;  // own rows stay where they are
         }
         c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
     }
+    // mode 0 with rank >= 0: the rank's own rows are already in place behind the peers' rows of each
+    // expert; they take no descriptors, and their range starts where the peers' rows end
+    const bool own_placed = mode == 0 && rank >= 0 && tid < num_segments && tid % num_ranks == rank;
+    const int c_true = c;
+    if (own_placed) c = 0;
     int total;
     const int prefix = block_exclusive_scan_1024(c, wave_totals, total);
     if (tid < num_segments) flat[tid] = prefix;
@@ -250,11 +257,17 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
         if (mode == 0) {
             if (tid < num_segments) {
                 const int le = tid / num_ranks;
-                const int64_t cnt = c, begin = flat[tid] - flat[le * num_ranks];
+                const int64_t cnt = c_true;
+                const int64_t begin = own_placed ? flat[(le + 1) * num_ranks] - flat[le * num_ranks]
+                                                 : flat[tid] - flat[le * num_ranks];
                 layout_out[tid] = cnt > 0 ? ((begin << 32) | cnt) : 0;
             }
             if (tid < num_local_experts) {
-                const int n = flat[(tid + 1) * num_ranks] - flat[tid * num_ranks];
+                int n = flat[(tid + 1) * num_ranks] - flat[tid * num_ranks];
+                if (rank >= 0) {
+                    const int own = counts32[tid * num_ranks + rank];
+                    n += own < 0 ? 0 : (own > max_tokens ? max_tokens : own);
+                }
                 packed_count[tid] = n;
                 if (stats != nullptr) stats[tid] += n;
             }
@@ -264,7 +277,7 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
     const int le = seg / num_ranks, s = seg - le * num_ranks;
     const int cnt = flat[seg + 1] - flat[seg];
     const int64_t begin = mode == 0 ? flat[seg] - flat[le * num_ranks] : begin_in[seg];
-    if (mode == 1 && (begin < 0 || begin + cnt > slots_per_expert)) return;  // malformed range: emit nothing
+    if (mode != 0 && (begin < 0 || begin + cnt > slots_per_expert)) return;  // malformed range: emit nothing
     for (int j = tid; j < cnt; j += kIndexThreads) {
         RowDesc d;
         if (mode == 0) {

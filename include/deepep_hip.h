@@ -335,19 +335,19 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
  * the call is made (the reference's dispatch is one call too:
  * Buffer::low_latency_dispatch, csrc/deep_ep.cpp:1658-1796; its kernel has a
  * send and a receive phase, csrc/kernels/coop_dispatch_send.cuh:304,
- * coop_dispatch_recv.cuh:42).  Arguments are those of the two calls; outputs
- * are identical, with one difference: for small batches
- * (num_tokens * num_topk <= 8192 and at most 8192 rows expected) both phases run
- * as one kernel launch, and then this rank's rows for its own experts go
- * straight to their packed position — the own segment of recv_staging is not
- * written (recv_count, send_count, send_slots, pair_slot are written as by
- * deepep_ll_dispatch_send).  Larger batches launch the phases back to back.
+ * coop_dispatch_recv.cuh:42).  Arguments are those of the two calls.  One
+ * thing differs from calling them in turn: this rank's rows for its own experts
+ * go straight to their packed position, behind the rows of all the peers, so
+ * inside an expert's range the source ranks come in ascending order with this
+ * rank last (layout_range says so) and the own segment of recv_staging is not
+ * written; recv_count, send_count, send_slots and pair_slot are written as by
+ * deepep_ll_dispatch_send.  Small batches (num_tokens * num_topk <= 8192 and at
+ * most 8192 rows expected) run as one kernel launch, larger ones as the send
+ * and receive launches back to back; the result is the same.
  *   workspace          as for deepep_ll_dispatch_send
  *   segment_workspace  as the workspace of deepep_ll_dispatch_recv */
-/* 1 when deepep_ll_dispatch runs a batch of this shape as one kernel launch (and so places the
- * rank's own segment behind the peers' inside each expert's range), else 0.  No counterpart in
- * the reference, whose segment order is whatever its atomics produce; layout_range carries the
- * order either way. */
+/* 1 when deepep_ll_dispatch runs a batch of this shape as one kernel launch, else 0 (the result
+ * does not depend on it).  No counterpart in the reference. */
 int deepep_ll_dispatch_is_single_launch(int num_tokens, int num_topk, int num_experts,
                                         int num_max_dispatch_tokens_per_rank, int64_t expected_rows);
 
@@ -367,11 +367,11 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx,
  * whose remote experts' answers are already in combine_staging when the call
  * is made (the reference: Buffer::low_latency_combine,
  * csrc/deep_ep.cpp:1798-1920; kernel phases csrc/kernels/coop_combine_send.cuh:37,
- * coop_combine_recv.cuh:72).  `out` is identical to the two calls'.  When
- * at most 8192 rows are expected both phases run as one kernel launch, and then the
+ * coop_combine_recv.cuh:72).  `out` is identical to the two calls'.  The
  * answers of this rank's own experts are read from x directly — the own
- * experts' part of combine_staging is neither written nor read.  Larger
- * batches launch the phases back to back. */
+ * experts' part of combine_staging is neither written nor read.  When at most
+ * 8192 rows are expected both phases run as one kernel launch, larger batches
+ * launch them back to back. */
 int deepep_ll_combine(const void* x, const int64_t* layout_range,
                       const int64_t* topk_idx, const float* topk_weights,
                       const int32_t* pair_slot,

@@ -58,10 +58,9 @@ ONE_CALL = pytest.mark.parametrize("one_call", [False, True], ids=["two_calls", 
 
 
 def own_last(one_call, t, k, e, m):
-    """The one-call dispatch runs as a single launch for small batches and then places this rank's own
-    rows behind the peers' inside each expert's range; otherwise source ranks come in ascending order."""
-    from deepep_efa_amd import _capi
-    return one_call and _capi.load().deepep_ll_dispatch_is_single_launch(t, k, e, m, m * k) == 1
+    """The one-call dispatch places this rank's own rows behind the peers' inside each expert's range,
+    whether it runs as one launch or two; the separate send / receive calls keep ascending source ranks."""
+    return one_call
 
 
 def poison_outputs(st):
@@ -686,8 +685,7 @@ def test_exchange_metadata_through_the_host_module(rt):
 @pytest.mark.parametrize("hint", ["batch", "unknown", "huge"])
 def test_capacity_far_above_the_batch(rt, hint):
     """A caller may size M for its largest batch and dispatch a small one.  The kernels are picked from the
-    expected-rows hint, not from the capacity; every hint gives the oracle's rows (the hint only decides
-    whether the one-call dispatch is a single launch, i.e. where an expert's own segment sits)."""
+    expected-rows hint, not from the capacity, and every hint gives the same result."""
     r, rank, t, m, h, k, e = 8, 2, 40, 5000, 512, 4, 64
     x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=4242, drop=7)
     shape = rt.ll.LLShape(num_ranks=r, rank=rank, num_experts=e, max_tokens=m, hidden=h, num_topk=k, fmt=O.ROW_FP8)
@@ -702,7 +700,7 @@ def test_capacity_far_above_the_batch(rt, hint):
     run_dispatch(st, world, x, topk, None, one_call=True)
     single = rt.capi.load().deepep_ll_dispatch_is_single_launch(t, k, e, m, st.expected_rows) == 1
     assert single == (hint == "batch")
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, O.ROW_FP8, own_last=single)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, O.ROW_FP8, own_last=True)
     check_dispatch(st, want, O.ROW_FP8)
     # combine with identity experts
     epr = e // r

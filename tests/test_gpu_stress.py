@@ -17,10 +17,14 @@ from oracle import deepep_oracle as O
 pytestmark = pytest.mark.gpu
 
 
-def test_skew_stress_full_size():
+@pytest.mark.parametrize("one_call", [False, True], ids=["two_calls", "one_call"])
+def test_skew_stress_full_size(one_call):
     from deepep_efa_amd import _capi, ll_runtime, loopback
     _capi.load()
     assert torch.cuda.is_available(), "this test needs the MI355X"
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()  # what earlier tests left in the caching allocator
     free, _ = torch.cuda.mem_get_info()
     if free < 170 * 2 ** 30:
         pytest.skip("needs ~150 GB of free HBM")
@@ -31,9 +35,13 @@ def test_skew_stress_full_size():
     world = loopback.LoopbackWorld(r, rank, seed=seed)
     world.synthesise(t, h, k, e, popularity="zipf", outlier_period=100)
     x, topk = world.own_inputs()
-    st.dispatch_send(x, topk)
-    world.dispatch_from_peers(st)
-    st.dispatch_recv()
+    if one_call:  # peers' rows first, then send + receive in one call: own segments sit behind the peers'
+        world.dispatch_from_peers(st)
+        st.dispatch(x, topk)
+    else:
+        st.dispatch_send(x, topk)
+        world.dispatch_from_peers(st)
+        st.dispatch_recv()
     torch.cuda.synchronize()
 
     # (a) integer outputs against the oracle, in full
@@ -47,7 +55,7 @@ def test_skew_stress_full_size():
     for le in range(epr):
         expert = rank * epr + le
         begin = 0
-        for s in range(r):
+        for s in ([q for q in range(r) if q != rank] + [rank] if one_call else range(r)):
             tok = (np.nonzero(flat[s] == expert)[0] // k).astype(np.int32)
             seg_tokens[(le, s)] = (begin, tok)
             want = ((begin << 32) | len(tok)) if len(tok) else 0
@@ -92,10 +100,13 @@ def test_skew_stress_full_size():
             q = st.packed_recv_x[le, b0:b1].float().view(b1 - b0, h // 128, 128)
             y[le, b0:b1] = (q * st.packed_recv_scales[le, b0:b1].unsqueeze(-1)).view(b1 - b0, h).to(torch.bfloat16)
     world.combine_from_peers(st, mode=0)
-    st.combine_send(y)
     w = torch.softmax(torch.randn((t, k), generator=torch.Generator().manual_seed(2)), dim=-1).cuda()
     out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
-    st.combine_recv(topk, w, out)
+    if one_call:
+        st.combine(y, topk, w, out)
+    else:
+        st.combine_send(y)
+        st.combine_recv(topk, w, out)
     torch.cuda.synchronize()
     want = x.double() * w.double().sum(1, keepdim=True)
     got = out.double()
