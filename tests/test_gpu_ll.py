@@ -714,3 +714,41 @@ def test_capacity_far_above_the_batch(rt, hint):
     wsum = w_all[rank].masked_fill(topk_all[rank] == -1, 0).sum(1).view(-1, 1)
     live = wsum.view(-1) > 0
     assert O.calc_diff((x_all[rank].float() * wsum)[live], out.cpu().float()[live]) < 2e-3
+
+
+@ONE_CALL
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
+def test_tokens_naming_an_expert_more_than_once(rt, fmt, one_call):
+    """Top-k never does it, but the path defines it: every pair gets its own slot in (token, k) order, and
+    pairs beyond the M slots of a (source, expert) segment are dropped (slot -1, not counted, not combined)."""
+    r, rank, t, m, h, k, e = 2, 1, 6, 6, 256, 4, 4
+    g = torch.Generator().manual_seed(5)
+    x_all = torch.randn((r, t, h), generator=g).to(torch.bfloat16)
+    topk_all = torch.tensor([[[3, 3, 3, 3]] * t,                       # 24 pairs for expert 3: 6 kept, 18 dropped
+                             [[2, 2, 0, -1], [2, 3, 3, 1], [0, 0, 0, 0], [2, 1, 2, 1], [-1, -1, 3, 3], [2, 2, 2, 2]]])
+    w_all = torch.rand((r, t, k), generator=g) + 0.1
+    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, m, fmt, one_call=one_call)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, fmt, own_last=one_call)
+    check_dispatch(st, want, fmt)
+    send_count, pair_slot = O.route(topk_all[rank], e, m)
+    assert torch.equal(st.send_count.cpu(), send_count) and torch.equal(st.pair_slot[:t].cpu(), pair_slot)
+    # what rank 0 sent to expert 3 (on rank 1): exactly M rows, the first M pairs in (token, k) order
+    lr = int(st.packed_recv_layout_range[1, 0])
+    assert lr & 0xFFFFFFFF == m
+    assert st.packed_recv_src_info[1, (lr >> 32):(lr >> 32) + m].cpu().tolist() == [0, 0, 0, 0, 1, 1]
+    # combine: identity experts on the received rows; dropped pairs contribute nothing
+    epr = e // r
+    y = torch.zeros((epr, r * m, h), dtype=torch.bfloat16)
+    count = st.packed_recv_count.cpu()
+    for le in range(epr):
+        n = int(count[le])
+        if fmt == O.ROW_BF16:
+            y[le, :n] = st.packed_recv_x[le, :n].cpu()
+        else:
+            y[le, :n] = O.per_token_cast_back(st.packed_recv_x[le, :n].cpu(), st.packed_recv_scales[le, :n].cpu())
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    run_combine(st, world, y.cuda(), topk_all[rank].cuda(), w_all[rank].cuda(), out, mode=0, one_call=one_call)
+    live = pair_slot >= 0
+    back = x_all[rank] if fmt == O.ROW_BF16 else O.per_token_cast_back(*O.per_token_cast_to_fp8(x_all[rank]))
+    chain = O.ll_combine_f32_chain(back.unsqueeze(1).expand(-1, k, -1).contiguous(), w_all[rank], live)
+    assert torch.equal(out.cpu().view(torch.int16), chain.view(torch.int16))
