@@ -281,13 +281,19 @@ struct Buffer {
         EP_HOST_ASSERT(num_experts > 0);
 
         auto compute_stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+        // A synchronous call with nothing to wait for is ordered on the caller's stream either way: the
+        // reference moves the work to its communication stream and back through two events
+        // (csrc/deep_ep.cpp:526-537,559-574), which on this GPU costs more than the kernels (27 us against 7);
+        // here such a call runs on the caller's stream directly.  Every other form keeps the hand-off.
+        const bool in_place = not async and not previous_event.has_value() and not allocate_on_comm_stream;
+        auto work_stream = in_place ? compute_stream : comm_stream;
         if (allocate_on_comm_stream) {
             EP_HOST_ASSERT(previous_event.has_value() and async);
             c10::hip::setCurrentHIPStreamMasqueradingAsCUDA(comm_stream);
         }
         if (previous_event.has_value())
             stream_wait(comm_stream, previous_event.value());
-        else
+        else if (not in_place)
             stream_wait(comm_stream, compute_stream);
 
         const int num_tokens = static_cast<int>(topk_idx.size(0)), num_topk = static_cast<int>(topk_idx.size(1));
@@ -308,7 +314,7 @@ struct Buffer {
             num_tokens_per_rank.data_ptr<int>(),
             num_tokens_per_rdma_rank.has_value() ? num_tokens_per_rdma_rank->data_ptr<int>() : nullptr,
             num_tokens_per_expert.data_ptr<int>(), reinterpret_cast<uint8_t*>(is_token_in_rank.data_ptr<bool>()),
-            layout_workspace.data_ptr(), size_t(layout_workspace.numel()), comm_stream.stream()));
+            layout_workspace.data_ptr(), size_t(layout_workspace.numel()), work_stream.stream()));
 
         std::optional<EventHandle> event;
         if (async) {
@@ -321,7 +327,7 @@ struct Buffer {
                 num_tokens_per_rdma_rank->record_stream(comm_stream);
                 if (allocate_on_comm_stream) num_tokens_per_rdma_rank->record_stream(compute_stream);
             }
-        } else {
+        } else if (not in_place) {
             stream_wait(compute_stream, comm_stream);
         }
         if (allocate_on_comm_stream) c10::hip::setCurrentHIPStreamMasqueradingAsCUDA(compute_stream);
