@@ -187,14 +187,19 @@ def bench_pack(torch, _capi, lib, loopback, args):
     return res
 
 
-def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args):
-    """The same four LL entry points at 4096 tokens (8 ranks x 32 experts), where they are HBM-bound."""
-    t, h, k, e, r, rank = 4096, 7168, 8, 256, 8, 3
+def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
+    """The same four LL entry points at 4096 tokens (8 ranks x 32 experts), where they are HBM-bound;
+    skewed: at 8192 tokens, 64 ranks x 4 experts, Zipf(1.2) expert popularity with rank 0 holding the hottest
+    experts and 1 % of the rows scaled by 100 (needs ~150 GB of HBM)."""
+    t, h, k, e, r, rank = (8192, 7168, 8, 256, 64, 0) if skewed else (4096, 7168, 8, 256, 8, 3)
     h = int(os.environ.get("DEEPEP_BENCH_LARGE_HIDDEN", h))  # tuning aid
     shape = ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8)
     st = ll_runtime.LowLatencyState(shape)
     world = loopback.LoopbackWorld(r, rank, seed=args.seed + 7)
-    world.synthesise(t, h, k, e)
+    if skewed:
+        world.synthesise(t, h, k, e, popularity="zipf", outlier_period=100)
+    else:
+        world.synthesise(t, h, k, e)
     x, topk = world.own_inputs()
     weights = torch.softmax(torch.randn((t, k), generator=torch.Generator().manual_seed(1)), dim=-1).cuda()
     out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
@@ -220,10 +225,11 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args):
         "dispatch": lambda: st.dispatch(x, topk),
         "combine": lambda: st.combine(y, topk, weights, out),
     }
-    res = {"workload": "LL dispatch+combine at 4096 tokens x 7168, top-8 of 256 experts, 8 ranks x 32 experts",
+    res = {"workload": f"LL dispatch+combine at {t} tokens x {h}, top-{k} of {e} experts, {r} ranks x {epr} experts"
+                       + (", Zipf(1.2) expert popularity, 1 % outlier rows" if skewed else ""),
            "pairs_sent": p, "rows_received": rv, "rows_to_own_experts": own}
     for name, fn in calls.items():
-        us = time_calls(torch, fn, max(10, args.steps // 10))
+        us = time_calls(torch, fn, 5 if skewed else max(10, args.steps // 10))
         res[name] = {"us": round(us, 2), "bytes": nbytes[name], "GBps": round(nbytes[name] / us / 1e3, 1),
                      "frac_of_8TBps": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBS, 4)}
     return res
@@ -252,6 +258,8 @@ def main():
                     help="only run N eager dispatch / combine pairs, each call after a 512 MiB flush of the caches "
                          "(writes, or reads with --cold-by-reads), for a rocprofv3 kernel trace")
     ap.add_argument("--cold-by-reads", action="store_true")
+    ap.add_argument("--skew-stress", action="store_true",
+                    help="only time the LL entry points at the skewed 8192-token, 64-rank stress size and print that")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the expert-parallel world; --gpus must be 1 "
@@ -266,6 +274,9 @@ def main():
     torch.cuda.set_device(0)
     if args.calibrate_copy:
         calibrate_copy(torch, _capi, lib)
+        return
+    if args.skew_stress:
+        print(json.dumps(bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=True)))
         return
     if os.environ.get("DEEPEP_BENCH_ONLY_LARGE") == "1":  # tuning aid: the 4096-token section alone
         print(json.dumps(bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args)))

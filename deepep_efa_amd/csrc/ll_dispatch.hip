@@ -191,7 +191,7 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
     const int64_t data_pad = align16(data_bytes);
     const int64_t scale_bytes = row_scale_bytes(a.hidden, kFmt);
     const int64_t scale_pad = align16(scale_bytes);
-    const int64_t stride = data_pad + scale_pad + kRowTailBytes;
+    const int64_t stride = row_stride_bytes(a.hidden, kFmt);
 
     DEEPEP_PHASE(0);
     // ---- issue this wave's row loads ------------------------------------
@@ -507,7 +507,7 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
     const int64_t data_bytes = row_data_bytes(a.hidden, a.fmt);
     const int64_t data_pad = align16(data_bytes);
     const int64_t scale_bytes = row_scale_bytes(a.hidden, a.fmt);
-    const int64_t stride = data_pad + align16(scale_bytes) + kRowTailBytes;
+    const int64_t stride = row_stride_bytes(a.hidden, a.fmt);
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
     const int waves_total = num_copy_blocks * waves;
     const int num_vec = int(data_bytes / 16);
