@@ -126,8 +126,8 @@ struct SendArgs {
 };
 
 // Final destination of the rows a rank sends to its own experts, used by the
-// single-launch dispatch: they skip the staging area and land where the
-// receive side would have copied them.
+// one-call dispatch (as one launch or two): they skip the staging area and land
+// behind the peers' rows of the expert, where nothing else is written.
 struct DirectOut {
     uint8_t* packed_x;  // null: stage own rows like everyone else's
     uint8_t* packed_scales;
