@@ -271,3 +271,12 @@ class Buffer:
 
     def combine(self, *args, **kwargs):
         raise NotImplementedError("normal-mode combine moves tokens between GPUs; not part of this build")
+
+    def internode_dispatch(self, *args, **kwargs):
+        raise NotImplementedError("internode dispatch moves tokens between nodes; not part of this build (its "
+                                  "GPU-side steps are deep_ep_cpp.moe_routing_sort, pack_rows, topk_remap and "
+                                  "build_recv_src_meta)")
+
+    def internode_combine(self, *args, **kwargs):
+        raise NotImplementedError("internode combine moves tokens between nodes; not part of this build (its "
+                                  "GPU-side reduction is deep_ep_cpp.combine_reduce)")

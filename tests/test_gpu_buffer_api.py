@@ -242,8 +242,10 @@ def test_api_argument_errors_and_masks(deep_ep):
     buffer.low_latency_clean_mask_buffer()
     buffer.low_latency_query_mask_buffer(status)
     assert status.tolist() == [0, 0, 0, 0]
-    with pytest.raises(NotImplementedError):
-        buffer.dispatch(x)
+    for moves_tokens_between_gpus in (buffer.dispatch, buffer.combine, buffer.internode_dispatch,
+                                      buffer.internode_combine):
+        with pytest.raises(NotImplementedError):
+            moves_tokens_between_gpus(x)
     t = buffer.get_local_buffer_tensor(torch.int32, use_rdma_buffer=True)
     assert t.dtype == torch.int32 and t.is_cuda
     assert isinstance(buffer.get_comm_stream(), torch.cuda.Stream)
