@@ -30,7 +30,7 @@ struct CombineSendArgs {
 };
 
 // No LDS and no barrier: each wave holds the segment counts and begins in registers.
-template <int kPer>
+template <int kPer, bool kStream>
 __device__ __forceinline__ void combine_send_rows_impl(const CombineSendArgs& a, int block, int num_blocks,
                                                        bool skip_own) {
     const int lane = lane_id(), w = wave_in_block();
@@ -77,20 +77,21 @@ __device__ __forceinline__ void combine_send_rows_impl(const CombineSendArgs& a,
             continue;
         int v_begin, v_end;
         row_part_range(num_vec, parts, part, v_begin, v_end);
-        wave_copy_vec16<4>(src, dst, v_begin, v_end, lane);
+        wave_copy_vec16<4, kStream>(src, dst, v_begin, v_end, lane);
     }
 }
 
+template <bool kStream>
 __device__ __forceinline__ void combine_send_rows(const CombineSendArgs& a, int block, int num_blocks, bool skip_own) {
     if (a.num_local_experts * a.num_ranks <= 4 * kWave)
-        combine_send_rows_impl<4>(a, block, num_blocks, skip_own);
+        combine_send_rows_impl<4, kStream>(a, block, num_blocks, skip_own);
     else
-        combine_send_rows_impl<16>(a, block, num_blocks, skip_own);
+        combine_send_rows_impl<16, kStream>(a, block, num_blocks, skip_own);
 }
 
 // skip_own: the rows owed to this rank itself stay where they are (the reduce reads them from x).
 __global__ __launch_bounds__(256) void ll_combine_send_kernel(CombineSendArgs a, bool skip_own) {
-    combine_send_rows(a, blockIdx.x, gridDim.x, skip_own);
+    combine_send_rows<false>(a, blockIdx.x, gridDim.x, skip_own);
 }
 
 // ---------------------------------------------------------------------
@@ -227,6 +228,7 @@ __global__ __launch_bounds__(1024) void ll_combine_recv_kernel(CombineRecvArgs a
 // (The reference's combine is one kernel with a send and a receive phase as
 // well: csrc/kernels/coop_combine_send.cuh:37, coop_combine_recv.cuh:72.)
 // ---------------------------------------------------------------------
+template <bool kStream>
 __global__ __launch_bounds__(256) void ll_combine_fused_kernel(CombineSendArgs sa, CombineRecvArgs ra,
                                                                int num_recv_blocks) {
     extern __shared__ int32_t dyn_lds[];  // reduce workgroups: own_begin[E_l]
@@ -237,10 +239,11 @@ __global__ __launch_bounds__(256) void ll_combine_fused_kernel(CombineSendArgs s
             dyn_lds[le] = (lr & 0xffffffffll) > 0 ? int(lr >> 32) : 0;
         }
         lds_barrier();
-        combine_recv_piece<false>(ra, int64_t(block) * 4 + wave_in_block(), sa.x, dyn_lds, sa.rank * sa.num_local_experts,
-                           sa.num_local_experts, int64_t(sa.max_tokens) * sa.num_ranks);
+        combine_recv_piece<kStream>(ra, int64_t(block) * 4 + wave_in_block(), sa.x, dyn_lds,
+                                    sa.rank * sa.num_local_experts, sa.num_local_experts,
+                                    int64_t(sa.max_tokens) * sa.num_ranks);
     } else {
-        combine_send_rows(sa, block - num_recv_blocks, int(gridDim.x) - num_recv_blocks, true);
+        combine_send_rows<kStream>(sa, block - num_recv_blocks, int(gridDim.x) - num_recv_blocks, true);
     }
 }
 
@@ -442,8 +445,14 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
     if (send_blocks > 1024) send_blocks = 1024;
     if (recv_blocks + send_blocks == 0) return 0;
     const size_t lds = size_t(sa.num_local_experts) * sizeof(int32_t);
-    ll_combine_fused_kernel<<<dim3(unsigned(recv_blocks + send_blocks)), 256, lds,
-                              reinterpret_cast<hipStream_t>(stream)>>>(sa, ra, int(recv_blocks));
+    // rows returned (read + written) plus rows gathered: past what the caches hold, stream
+    const int64_t traffic = (2 * rows + int64_t(num_tokens) * num_topk) * hidden * 2;
+    if (traffic > stream_bytes())
+        ll_combine_fused_kernel<true><<<dim3(unsigned(recv_blocks + send_blocks)), 256, lds,
+                                        reinterpret_cast<hipStream_t>(stream)>>>(sa, ra, int(recv_blocks));
+    else
+        ll_combine_fused_kernel<false><<<dim3(unsigned(recv_blocks + send_blocks)), 256, lds,
+                                         reinterpret_cast<hipStream_t>(stream)>>>(sa, ra, int(recv_blocks));
     EP_LAUNCH_CHECK();
     return 0;
 }

@@ -142,22 +142,20 @@ __device__ __forceinline__ int wave_segments_find(const WaveSegments<kPer>& t, i
 }
 
 // Copies 16-byte vectors [v_begin, v_end) of a row with one wave, kDepth loads in flight per lane.
-template <int kDepth>
+template <int kDepth, bool kStream = false>
 __device__ __forceinline__ void wave_copy_vec16(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
                                                 int v_begin, int v_end, int lane) {
-    const u32x4* s = reinterpret_cast<const u32x4*>(src);
-    u32x4* d = reinterpret_cast<u32x4*>(dst);
     for (int base = v_begin; base < v_end; base += kWave * kDepth) {
         u32x4 r[kDepth];
 #pragma unroll
         for (int u = 0; u < kDepth; ++u) {
             const int v = base + u * kWave + lane;
-            if (v < v_end) r[u] = s[v];
+            if (v < v_end) r[u] = load_u32x4<kStream>(src + int64_t(v) * 16);
         }
 #pragma unroll
         for (int u = 0; u < kDepth; ++u) {
             const int v = base + u * kWave + lane;
-            if (v < v_end) d[v] = r[u];
+            if (v < v_end) store_u32x4<kStream>(dst + int64_t(v) * 16, r[u]);
         }
     }
 }
