@@ -398,6 +398,7 @@ def test_reference_recipe_roundtrip(rt, use_fp8, one_call):
 
 @pytest.mark.parametrize("r,rank,t,h,k,e", [(32, 5, 128, 7168, 8, 256), (4, 0, 16, 512, 3, 8),
                                             (8, 3, 4200, 512, 4, 64),   # large-batch combine-send path
+                                            (8, 3, 1024, 4096, 8, 64),  # the largest single launch: moves > 192 MB, so it streams
                                             (4, 2, 40, 512, 11, 64),    # more than eight selections per token
                                             (8, 6, 20, 512, 4, 512),    # more than 256 segments
                                             (4, 1, 33, 1536, 5, 32),    # hidden not a multiple of 512
