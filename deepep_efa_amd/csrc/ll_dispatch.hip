@@ -127,7 +127,8 @@ struct SendArgs {
 
 // Final destination of the rows a rank sends to its own experts, used by the
 // one-call dispatch (as one launch or two): they skip the staging area and land
-// behind the peers' rows of the expert, where nothing else is written.
+// in the packed tensors behind the rows of the lower source ranks, which is where
+// the reference's ascending-source ranges put them.
 struct DirectOut {
     uint8_t* packed_x;  // null: stage own rows like everyone else's
     uint8_t* packed_scales;
@@ -226,19 +227,20 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
         }
     }
     if (direct.packed_x != nullptr && tid < kWave) {
-        // Rows for this rank's own experts go straight to the packed tensors, behind the rows of all
-        // the peers: for each such selection wave 0 adds up the peers' counts of that expert.
+        // Rows for this rank's own experts go straight to the packed tensors, at the place the
+        // reference's range builder gives them: behind the rows of the lower source ranks
+        // (csrc/kernels/efa_kernels.cu:991-1010).  For each such selection wave 0 adds up those
+        // ranks' counts of the expert.
         uint64_t to_own = __ballot(my_expert >= 0 && dst_rank == a.rank);
         while (to_own != 0) {
             const int k = __builtin_ctzll(to_own);
             to_own &= to_own - 1;
             const int le = __builtin_amdgcn_readlane(local, k);
             int part = 0;
-            for (int s = lane; s < a.num_ranks; s += kWave)
-                if (s != a.rank) {
-                    const int c = a.recv_count[le * a.num_ranks + s];
-                    part += c < 0 ? 0 : (c > a.max_tokens ? a.max_tokens : c);
-                }
+            for (int s = lane; s < a.rank; s += kWave) {
+                const int c = a.recv_count[le * a.num_ranks + s];
+                part += c < 0 ? 0 : (c > a.max_tokens ? a.max_tokens : c);
+            }
             const int sum = __builtin_amdgcn_readlane(wave_inclusive_sum(part), kWave - 1);
             if (lane == k) direct_begin = sum;
         }
@@ -402,17 +404,23 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs 
 }
 
 // ---------------------------------------------------------------------
-// Receive side.  Every workgroup rebuilds the segment prefix from the E
-// counts (a few hundred ints) in LDS, then its waves walk the flat row index
-// space: row -> (segment, j) by binary search, one wave per row part.
-// Slot order is fixed by the staging order, not by atomics
-// (reference: csrc/kernels/efa_kernels.cu:1017-1052 for the ranges,
-// :1059-1213 for the deterministic scatter).
+// Receive side.  Every copying wave rebuilds the segment prefix from the E
+// counts (a few hundred ints) in its registers, then walks the flat row index
+// space: row -> (segment, j) by ballot, one wave per row part.
+// Ranges are the reference's: inside an expert's packed range the source ranks
+// come in ascending order, begin(e, s) = sum of cnt(e, s') over s' < s
+// (csrc/kernels/efa_kernels.cu:991-1010, :1031-1050); the slot order inside a
+// segment is fixed by the staging order, not by atomics (:1059-1213 is the
+// reference's deterministic scatter).
 //
-// own_topk != null (single-launch dispatch): the rows this rank sends to its own
-// experts are not in the staging area — the send workgroups of the same launch
-// put them straight into the packed tensors — so the own segments' counts are
-// recounted here from the rank's own indices, and their rows are skipped.
+// own_rank >= 0 (one-call dispatch): the rows this rank sends to its own
+// experts are not in the staging area — the send side puts them straight into
+// the packed tensors, behind the rows of the lower ranks — so the copying waves
+// skip the own segments and move the segments of the higher ranks up by the
+// expert's own count.  With own_topk (single launch) that count is recounted
+// from the rank's own indices, because the launch that reads recv_count's own
+// entries is the one that writes them; without it (the send kernel has
+// finished) recv_count holds it.
 // ---------------------------------------------------------------------
 struct RecvArgs {
     const uint8_t* recv_staging;
@@ -430,14 +438,47 @@ __device__ __forceinline__ int clamp_count(int c, int max_tokens) {
     return c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
 }
 
+// own_cnt[e_l] (LDS, unclamped) = rows this rank sends to its own expert e_l, by the whole workgroup;
+// ends with a barrier.
+__device__ __forceinline__ void own_row_counts(const RecvArgs& a, const int64_t* own_topk, int own_entries,
+                                               int own_rank, int32_t* own_cnt) {
+    const int tid = threadIdx.x, threads = blockDim.x;
+    if (own_topk == nullptr) {
+        for (int le = tid; le < a.num_local_experts; le += threads)
+            own_cnt[le] = a.recv_count[le * a.num_ranks + own_rank];
+        lds_barrier();
+        return;
+    }
+    constexpr int kAhead = 4;  // loads in flight per thread
+    int64_t v[kAhead];
+#pragma unroll
+    for (int r = 0; r < kAhead; ++r) {
+        const int i = tid + r * threads;
+        v[r] = i < own_entries ? own_topk[i] : -1;
+    }
+    for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
+    lds_barrier();
+    const int64_t first = int64_t(own_rank) * a.num_local_experts;
+    for (int base = 0; base < own_entries; base += kAhead * threads) {
+        int64_t next[kAhead];
+#pragma unroll
+        for (int r = 0; r < kAhead; ++r) {
+            const int i = base + (kAhead + r) * threads + tid;
+            next[r] = i < own_entries ? own_topk[i] : -1;
+        }
+#pragma unroll
+        for (int r = 0; r < kAhead; ++r) {
+            const int64_t d = v[r] - first;
+            if (v[r] >= 0 && d >= 0 && d < a.num_local_experts) atomicAdd(&own_cnt[int(d)], 1);
+            v[r] = next[r];
+        }
+    }
+    lds_barrier();
+}
+
 // Workgroups [0, num_copy_blocks) copy rows; workgroup num_copy_blocks writes layout_range,
 // packed_count and stats and copies nothing.  A copying wave builds the segment prefix in its own
-// registers (WaveSegments) from the E counts: no LDS, no barrier.
-//
-// With own_topk (single-launch dispatch) this rank's own rows are not in the staging area: the
-// send workgroups of the same launch put them straight into the packed tensors, behind the rows
-// of all the peers.  The copying waves then see the peers' segments only and need nothing from
-// the own routing; the metadata workgroup recounts the own rows from own_topk for layout_range.
+// registers (WaveSegments) from the E counts.
 // lds: [num_segments + 1 + num_local_experts] ints; wave_totals: 16 ints.
 template <int kPer>
 __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int num_copy_blocks,
@@ -447,38 +488,26 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
     const int threads = blockDim.x, waves = threads >> 6;
     const int num_ranks = a.num_ranks, max_tokens = a.max_tokens;
     const int num_segments = a.num_local_experts * num_ranks;
-    const bool own_last = own_topk != nullptr;
+    const bool own_placed = own_rank >= 0;
 
     if (block == num_copy_blocks) {  // the metadata workgroup
         int32_t* own_cnt = lds + num_segments + 1;
-        if (own_last) {
-            for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
-            lds_barrier();
-            const int64_t first = int64_t(own_rank) * a.num_local_experts;
-            for (int i = tid; i < own_entries; i += threads) {
-                const int64_t v = own_topk[i] - first;
-                if (v >= 0 && v < a.num_local_experts) atomicAdd(&own_cnt[int(v)], 1);
-            }
-        }
+        if (own_placed) own_row_counts(a, own_topk, own_entries, own_rank, own_cnt);
         for (int s = tid; s < num_segments; s += threads) {
-            const bool own = own_last && s % num_ranks == own_rank;
-            lds[s] = own ? 0 : clamp_count(a.recv_count[s], max_tokens);
+            const int le = s / num_ranks;
+            const bool own = own_placed && s - le * num_ranks == own_rank;
+            lds[s] = clamp_count(own ? own_cnt[le] : a.recv_count[s], max_tokens);
         }
         lds_barrier();
         block_exclusive_scan(lds, num_segments, wave_totals);
         for (int s = tid; s < num_segments; s += threads) {
             const int le = s / num_ranks;
-            int64_t cnt = lds[s + 1] - lds[s];
-            int64_t begin = lds[s] - lds[le * num_ranks];
-            if (own_last && s - le * num_ranks == own_rank) {
-                cnt = clamp_count(own_cnt[le], max_tokens);
-                begin = lds[(le + 1) * num_ranks] - lds[le * num_ranks];  // behind all the peers
-            }
+            const int64_t cnt = lds[s + 1] - lds[s];
+            const int64_t begin = lds[s] - lds[le * num_ranks];
             a.layout_range[s] = cnt > 0 ? ((begin << 32) | cnt) : 0;
         }
         for (int le = tid; le < a.num_local_experts; le += threads) {
-            int c = lds[(le + 1) * num_ranks] - lds[le * num_ranks];
-            if (own_last) c += clamp_count(own_cnt[le], max_tokens);
+            const int c = lds[(le + 1) * num_ranks] - lds[le * num_ranks];
             a.packed_count[le] = c;
             if (a.stats != nullptr) a.stats[le] += c;
         }
@@ -488,12 +517,14 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
     WaveSegments<kPer> seg_table;
     DEEPEP_PHASE(0);
     wave_load_int32<kPer>(a.recv_count, num_segments, lane, seg_table.cnt);
+    int32_t* own_cnt = lds;  // [E_l]
+    if (own_placed) own_row_counts(a, own_topk, own_entries, own_rank, own_cnt);
 #pragma unroll
     for (int u = 0; u < kPer; ++u) {
         seg_table.aux[u] = 0;
         seg_table.cnt[u] = clamp_count(seg_table.cnt[u], max_tokens);
     }
-    if (own_last) {  // whatever recv_count holds for the own segments (le * R + own_rank) is stale
+    if (own_placed) {  // the own segments (le * R + own_rank) hold nothing to copy
         int source = (lane * kPer) % num_ranks;  // source rank of this lane's first segment
 #pragma unroll
         for (int u = 0; u < kPer; ++u) {
@@ -519,7 +550,8 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
         const int seg = wave_segments_find(seg_table, row, seg_first, unused);
         const int le = seg / num_ranks;
         const int j = row - seg_first;
-        const int slot = row - wave_segments_prefix(seg_table, le * num_ranks);
+        int slot = row - wave_segments_prefix(seg_table, le * num_ranks);
+        if (own_placed && seg - le * num_ranks > own_rank) slot += clamp_count(own_cnt[le], max_tokens);
         const uint8_t* src = a.recv_staging + (int64_t(seg) * max_tokens + j) * stride;
         const int64_t out_row = int64_t(le) * slots_per_expert + slot;
         int v_begin, v_end;
@@ -546,10 +578,10 @@ __device__ __forceinline__ void recv_rows(const RecvArgs& a, int block, int num_
         recv_rows_impl<16>(a, block, num_copy_blocks, own_topk, own_entries, own_rank, lds, wave_totals);
 }
 
-// own_topk != null: the send side has already put this rank's own rows at their packed position.
+// own_rank >= 0: the send side has already put this rank's own rows at their packed position.
 __global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a, const int64_t* own_topk, int own_entries,
                                                       int own_rank) {
-    extern __shared__ int32_t flat[];  // [num_segments + 1 + E_l], used by the metadata workgroup (the last one)
+    extern __shared__ int32_t flat[];  // [num_segments + 1 + E_l]
     __shared__ int32_t wave_totals[kMaxBlockWaves];
     recv_rows(a, blockIdx.x, int(gridDim.x) - 1, own_topk, own_entries, own_rank, flat, wave_totals);
 }
@@ -560,11 +592,10 @@ __global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a, const int64_t*
 // kernels above in one grid.  No workgroup waits on another: the receive
 // workgroups copy only the peers' rows (already in the staging area when the
 // launch starts); the send workgroups place the rank's rows for its own
-// experts at their final packed position, behind the rows of all the peers,
-// which they find from the peers' counts.  Inside an expert's packed range
-// the order of the source ranks is therefore "peers ascending, then this
-// rank"; layout_range says so (the reference assigns the ranges in arrival
-// order, csrc/kernels/efa_kernels.cu:1017-1052 being its deterministic variant).
+// experts at their final packed position, which they find from the lower
+// ranks' counts, and the receive workgroups make room for them by recounting
+// them from the rank's own indices.  The packed ranges are the reference's
+// (ascending source rank, csrc/kernels/efa_kernels.cu:991-1010).
 // (The reference's dispatch is one kernel with a send and a receive phase as
 // well: csrc/kernels/coop_dispatch_send.cuh:304, coop_dispatch_recv.cuh:42.)
 // ---------------------------------------------------------------------
@@ -715,7 +746,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     const dim3 grid(blocks_per_token, num_tokens + 1, num_src);  // + the counting workgroup
     const size_t lds = size_t(num_experts) * sizeof(int32_t);
     // own_rows_direct (the two-launch form of the one-call dispatch): as in the single launch, the rows
-    // for this rank's own experts go straight to their packed position behind the peers' rows
+    // for this rank's own experts go straight to their packed position behind the lower ranks' rows
     EP_HOST_ASSERT(own_rows_direct == nullptr || (num_src == 1 && src_ranks == nullptr));
     const DirectOut direct = own_rows_direct != nullptr ? *own_rows_direct : DirectOut{nullptr, nullptr, nullptr};
 #define DEEPEP_LAUNCH_SEND(FMT) ll_send_kernel<FMT><<<grid, waves * kWave, lds, stream>>>(sa, direct)
@@ -830,16 +861,14 @@ static RecvArgs make_recv_args(const void* recv_staging, const int32_t* recv_cou
     return ra;
 }
 
-// own_rank >= 0: this rank's own rows are already at their packed position, behind the peers' rows
-// of each expert (the send side put them there); they are not copied, and own_topk [own_entries] is
-// the rank's routing, from which the small-batch kernel recounts them.
+// own_rank >= 0: the send kernel, which has finished, put this rank's own rows at their packed
+// position and their counts into recv_count; they are not copied again.
 static int launch_recv_side(const void* recv_staging, const int32_t* recv_count, int hidden, int num_experts,
                             int num_ranks, int num_max_dispatch_tokens_per_rank, int row_format,
                             void* packed_recv_x, void* packed_recv_scales, int32_t* packed_recv_src_info,
                             int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
                             int32_t* cumulative_local_expert_recv_stats, int64_t expected_rows, void* workspace,
-                            size_t workspace_bytes, const int64_t* own_topk, int own_entries, int own_rank,
-                            void* stream) {
+                            size_t workspace_bytes, int own_rank, void* stream) {
     if (int rc = check_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
                                  num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                                  packed_recv_src_info, packed_recv_layout_range, packed_recv_count))
@@ -883,8 +912,7 @@ static int launch_recv_side(const void* recv_staging, const int32_t* recv_count,
     const int64_t cap = large ? 4096 : 1024;
     if (blocks > cap) blocks = cap;
     const size_t lds = size_t(num_experts + 1 + num_local_experts) * sizeof(int32_t);
-    ll_recv_kernel<<<dim3(unsigned(blocks) + 1), 256, lds, hs>>>(ra, own_rank >= 0 ? own_topk : nullptr, own_entries,
-                                                                 own_rank);  // + the metadata workgroup
+    ll_recv_kernel<<<dim3(unsigned(blocks) + 1), 256, lds, hs>>>(ra, nullptr, 0, own_rank);  // + the metadata workgroup
     EP_LAUNCH_CHECK();
     return 0;
 }
@@ -899,8 +927,7 @@ int deepep_ll_dispatch_recv(const void* recv_staging, const int32_t* recv_count,
     return launch_recv_side(recv_staging, recv_count, hidden, num_experts, num_ranks,
                             num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                             packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
-                            cumulative_local_expert_recv_stats, expected_rows, workspace, workspace_bytes, nullptr, 0,
-                            -1, stream);
+                            cumulative_local_expert_recv_stats, expected_rows, workspace, workspace_bytes, -1, stream);
 }
 
 int deepep_ll_dispatch_is_single_launch(int num_tokens, int num_topk, int num_experts,
@@ -927,9 +954,9 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, i
                                 num_max_dispatch_tokens_per_rank, row_format))
         return rc;
     if (!fused) {
-        // The two phases back to back, with the same placement as the single launch: the send side
-        // writes the rows for this rank's own experts straight to their packed position behind the
-        // peers' rows (whose counts are in recv_count already), and the receive side copies the rest.
+        // The two phases back to back, with the single launch's shortcut: the send side writes the
+        // rows for this rank's own experts straight to their packed position behind the lower ranks'
+        // rows (whose counts are in recv_count already), and the receive side copies the rest.
         EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
         EP_HOST_ASSERT(recv_staging != nullptr && recv_count != nullptr && pair_slot != nullptr && send_count != nullptr);
         EP_HOST_ASSERT(workspace != nullptr);
@@ -950,7 +977,7 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, i
                                 num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                                 packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
                                 cumulative_local_expert_recv_stats, expected_rows, segment_workspace,
-                                segment_workspace_bytes, topk_idx, num_tokens * num_topk, rank, stream);
+                                segment_workspace_bytes, rank, stream);
     }
     EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
     EP_HOST_ASSERT(send_count != nullptr && pair_slot != nullptr);

@@ -214,7 +214,8 @@ __device__ __forceinline__ int block_exclusive_scan_1024(int v, int32_t* wave_to
 
 // mode 0 (dispatch receive): counts = recv_count; writes layout_range / packed_count / stats;
 //        descriptor = {staging row seg*M + j, packed row e_l*N + begin + j}; rank = -1, or the rank
-//        whose own rows are already in the packed tensors.
+//        whose own rows the send side has already put at their packed position (they keep their
+//        place in the ranges, in ascending source order, and get no descriptors).
 // mode 1 (combine send; mode 2: the same without this rank's own rows): counts and begins from layout_range;
 //        descriptor = {expert-output row e_l*N + begin + j, seg*M + j for other ranks or
 //        -(1 + (rank*E_l + e_l)*M + j) for this rank's own rows}.
@@ -222,9 +223,11 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
     int mode, const int32_t* __restrict__ counts32, const int64_t* __restrict__ layout_in, int num_local_experts,
     int num_ranks, int rank, int max_tokens, int64_t* __restrict__ layout_out, int32_t* __restrict__ packed_count,
     int32_t* __restrict__ stats, int32_t* __restrict__ flat_out, RowDesc* __restrict__ desc) {
-    __shared__ int32_t flat[kIndexThreads + 1];
+    __shared__ int32_t flat[kIndexThreads + 1];   // prefix over the rows that get descriptors
+    __shared__ int32_t place[kIndexThreads + 1];  // mode 0: prefix over all rows (where a segment lands)
     __shared__ int32_t begin_in[kIndexThreads];
     __shared__ int32_t wave_totals[kIndexThreads / kWave];
+    __shared__ int32_t wave_totals_place[kIndexThreads / kWave];
     const int tid = threadIdx.x;
     const int num_segments = num_local_experts * num_ranks;
     int c = 0;
@@ -239,15 +242,22 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
         }
         c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
     }
-    // mode 0 with rank >= 0: the rank's own rows are already in place behind the peers' rows of each
-    // expert; they take no descriptors, and their range starts where the peers' rows end
-    const bool own_placed = mode == 0 && rank >= 0 && tid < num_segments && tid % num_ranks == rank;
-    const int c_true = c;
-    if (own_placed) c = 0;
+    // mode 0 with rank >= 0: the rank's own rows are already in place (reference order: a range
+    // begins where the lower source ranks' rows end, csrc/kernels/efa_kernels.cu:991-1010), so
+    // they count towards where the later segments land but take no descriptors
+    const bool own_placed = mode == 0 && rank >= 0;
+    const int c_all = c;
+    if (own_placed && tid < num_segments && tid % num_ranks == rank) c = 0;
     int total;
     const int prefix = block_exclusive_scan_1024(c, wave_totals, total);
     if (tid < num_segments) flat[tid] = prefix;
     if (tid == 0) flat[num_segments] = total;
+    if (mode == 0) {
+        int total_all = total, prefix_all = prefix;
+        if (own_placed) prefix_all = block_exclusive_scan_1024(c_all, wave_totals_place, total_all);
+        if (tid < num_segments) place[tid] = prefix_all;
+        if (tid == 0) place[num_segments] = total_all;
+    }
     __syncthreads();
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
     if (blockIdx.x == 0) {
@@ -255,17 +265,12 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
         if (mode == 0) {
             if (tid < num_segments) {
                 const int le = tid / num_ranks;
-                const int64_t cnt = c_true;
-                const int64_t begin = own_placed ? flat[(le + 1) * num_ranks] - flat[le * num_ranks]
-                                                 : flat[tid] - flat[le * num_ranks];
+                const int64_t cnt = c_all;
+                const int64_t begin = place[tid] - place[le * num_ranks];
                 layout_out[tid] = cnt > 0 ? ((begin << 32) | cnt) : 0;
             }
             if (tid < num_local_experts) {
-                int n = flat[(tid + 1) * num_ranks] - flat[tid * num_ranks];
-                if (rank >= 0) {
-                    const int own = counts32[tid * num_ranks + rank];
-                    n += own < 0 ? 0 : (own > max_tokens ? max_tokens : own);
-                }
+                const int n = place[(tid + 1) * num_ranks] - place[tid * num_ranks];
                 packed_count[tid] = n;
                 if (stats != nullptr) stats[tid] += n;
             }
@@ -274,7 +279,7 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
     const int seg = blockIdx.x;
     const int le = seg / num_ranks, s = seg - le * num_ranks;
     const int cnt = flat[seg + 1] - flat[seg];
-    const int64_t begin = mode == 0 ? flat[seg] - flat[le * num_ranks] : begin_in[seg];
+    const int64_t begin = mode == 0 ? place[seg] - place[le * num_ranks] : begin_in[seg];
     if (mode != 0 && (begin < 0 || begin + cnt > slots_per_expert)) return;  // malformed range: emit nothing
     for (int j = tid; j < cnt; j += kIndexThreads) {
         RowDesc d;

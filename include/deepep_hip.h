@@ -335,12 +335,13 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
  * the call is made (the reference's dispatch is one call too:
  * Buffer::low_latency_dispatch, csrc/deep_ep.cpp:1658-1796; its kernel has a
  * send and a receive phase, csrc/kernels/coop_dispatch_send.cuh:304,
- * coop_dispatch_recv.cuh:42).  Arguments are those of the two calls.  One
- * thing differs from calling them in turn: this rank's rows for its own experts
- * go straight to their packed position, behind the rows of all the peers, so
- * inside an expert's range the source ranks come in ascending order with this
- * rank last (layout_range says so) and the own segment of recv_staging is not
- * written; recv_count, send_count, send_slots and pair_slot are written as by
+ * coop_dispatch_recv.cuh:42).  Arguments and every packed_* output are those
+ * of the two calls: inside an expert's range the source ranks come in ascending
+ * order, begin(e, s) = sum of the counts of the ranks below s
+ * (csrc/kernels/efa_kernels.cu:991-1010).  One thing differs from calling them
+ * in turn: this rank's rows for its own experts go straight to their packed
+ * position and the own segment of recv_staging is not written; recv_count,
+ * send_count, send_slots and pair_slot are written as by
  * deepep_ll_dispatch_send.  Small batches (num_tokens * num_topk <= 8192 and at
  * most 8192 rows expected) run as one kernel launch, larger ones as the send
  * and receive launches back to back; the result is the same.

@@ -28,7 +28,7 @@ generative on CUDA RNG streams that cannot be replayed here):
   kernels (``_serial_dispatch``) compared against the vectorised form.
 * combine — the closed form ``x * sum(w)`` of ``tests/test_low_latency.py:181``
   and a float64 sum.
-* layout, route slots, dispatch outputs (both segment orders) and the combine — also a
+* layout, route slots, dispatch outputs and the combine — also a
   two-rank world worked out on paper, ``tests/golden/ll_tiny_world.json``.
 * ``topk_remap``, ``build_recv_src_meta`` — the torch expressions the reference's kernels
   replaced (named in their headers, ``csrc/kernels/efa_kernels.cu:321-337,438-446``), pinned
@@ -299,14 +299,14 @@ def route(topk_idx: torch.Tensor, num_experts: int, max_tokens: int):
     return send_count, pair_slot.view(t, k)
 
 
-def ll_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_tokens: int, fmt: int = ROW_FP8,
-                own_last: bool = False):
+def ll_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_tokens: int, fmt: int = ROW_FP8):
     """What rank `rank` receives when every rank of the world dispatches.
 
-    own_last: inside each expert's packed range the source ranks come in ascending order with
-    `rank`'s own segment moved behind all the others (the order of the single-launch dispatch);
-    otherwise plain ascending order.  The reference fixes no order across source ranks (its live
-    kernel claims ranges with atomics); layout_range carries whichever is used.
+    Inside each expert's packed range the source ranks come in ascending order:
+    begin(e, s) = sum of cnt(e, s') over s' < s, the serial prefix of the reference's range
+    builders (csrc/kernels/efa_kernels.cu:991-1010 and :1031-1050).  Its atomics only decide
+    the order of the rows inside one (expert, source) segment (:1227-1389); here that order is
+    the sender's ascending (token, k) order, as in its deterministic scatter.
 
     all_x: list of R tensors [T_s, H] bf16; all_topk_idx: list of R tensors [T_s, K] int64.
     Follows deep_ep/buffer.py:1816-1887,2266-2457 (nccl-fallback branch) with
@@ -333,10 +333,9 @@ def ll_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_tokens: in
         _, pair_slot = route(all_topk_idx[s], num_experts, max_tokens)
         data, scales = quantise_rows(all_x[s], fmt)
         per_src.append((pair_slot, data, scales))
-    order = [s for s in range(r) if s != rank] + [rank] if own_last else list(range(r))
     for le in range(epr):
         e = rank * epr + le
-        for s in order:
+        for s in range(r):
             pair_slot, data, scales = per_src[s]
             sel = (all_topk_idx[s] == e) & (pair_slot >= 0)
             tok, kk = torch.nonzero(sel, as_tuple=True)

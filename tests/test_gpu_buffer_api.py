@@ -166,8 +166,8 @@ def test_dispatch_matches_oracle_through_the_api(deep_ep):
     assert hook is None
     topk_all = O.synth_topk_idx(O.uniform_cdf(e), np.arange(num_ranks), t, k, 77)
     x_all = O.synth_bf16_rows(np.arange(num_ranks * t, dtype=np.uint32), h, 77).view(num_ranks, t, h)
-    # at this size the API's dispatch is one launch: this rank's own rows sit behind the peers'
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8, own_last=True)
+    # at this size the API's dispatch is one launch
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
     assert torch.equal(recv_count.cpu(), want["packed_recv_count"])
     assert torch.equal(handle[1].cpu(), want["packed_recv_layout_range"])
     px, ps, si = recv_x.view(torch.uint8).cpu(), recv_scales.view(torch.uint8).cpu(), handle[0].cpu()

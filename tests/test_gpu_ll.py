@@ -57,12 +57,6 @@ def make_world(r, t, h, k, e, seed, drop=10, recipe="randn"):
 ONE_CALL = pytest.mark.parametrize("one_call", [False, True], ids=["two_calls", "one_call"])
 
 
-def own_last(one_call, t, k, e, m):
-    """The one-call dispatch places this rank's own rows behind the peers' inside each expert's range,
-    whether it runs as one launch or two; the separate send / receive calls keep ascending source ranks."""
-    return one_call
-
-
 def poison_outputs(st):
     """Fresh tensors may reuse memory that an earlier test left holding the right answer."""
     st.packed_recv_x.view(torch.uint8).fill_(0xEE)
@@ -149,15 +143,15 @@ def check_dispatch(st, want, fmt):
 def test_dispatch_small_worlds(rt, fmt, r, rank, t, h, k, e, one_call):
     x_all, topk_all, _ = make_world(r, t, h, k, e, seed=r * 100 + t, drop=min(5, t))
     st, _ = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt, one_call=one_call)
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt, own_last=own_last(one_call, t, k, e, t))
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
     check_dispatch(st, want, fmt)
     send_count, pair_slot = O.route(topk_all[rank], e, t)
     assert torch.equal(st.send_count.cpu(), send_count)
     assert torch.equal(st.pair_slot[:t].cpu(), pair_slot)
 
 
-@pytest.mark.parametrize("key,rank,one_call", [("rank0_ascending", 0, False), ("rank0_own_last", 0, True),
-                                               ("rank1_ascending", 1, False)])
+@pytest.mark.parametrize("key,rank", [("rank0_ascending", 0), ("rank1_ascending", 1)])
+@ONE_CALL
 @pytest.mark.parametrize("fmt", [O.ROW_BF16, O.ROW_FP8])
 def test_hand_derived_world(rt, key, rank, one_call, fmt):
     """The HIP path against values worked out on paper (tests/golden/ll_tiny_world.json): no oracle involved."""
@@ -281,7 +275,7 @@ def test_dispatch_and_combine_seeded_random_shapes(rt, seed, one_call):
     r, rank, t, m, h, k, e, fmt, drop = _random_shape(seed)
     x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=1000 + seed, drop=drop)
     st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, m, fmt, one_call=one_call)
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, fmt, own_last=own_last(one_call, t, k, e, m))
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, fmt)
     check_dispatch(st, want, fmt)
     send_count, pair_slot = O.route(topk_all[rank], e, m)
     assert torch.equal(st.send_count.cpu(), send_count)
@@ -421,7 +415,7 @@ def test_combine_random_expert_outputs(rt, oracle_c, r, rank, t, h, k, e, one_ca
     # oracle: which row does each of this rank's pairs get back?
     topk, w = topk_all[rank], w_all[rank]
     _, pair_slot = O.route(topk, e, t)
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8, own_last=own_last(one_call, t, k, e, t))
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
     keys_local, keys_remote = [], []
     pair_rows = torch.zeros((t, k, h), dtype=torch.bfloat16)
     live = pair_slot >= 0
@@ -485,7 +479,7 @@ def test_ll_config_full_size(rt, one_call, e, rank):
     assert torch.equal(world.topk_idx_all.cpu(), topk_all)
     x_all = O.synth_bf16_rows(np.arange(r * t, dtype=np.uint32), h, 2024).view(r, t, h)
     assert torch.equal(world.x_all.cpu().view(torch.int16), x_all.view(torch.int16))
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8, own_last=own_last(one_call, t, k, e, t))
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
     check_dispatch(st, want, O.ROW_FP8)
     assert int(st.packed_recv_count.sum()) == int(((topk_all // (e // r)) == rank).sum())
 
@@ -504,7 +498,7 @@ def test_skewed_routing_roundtrip(rt, one_call):
     x_all = O.synth_bf16_rows(np.arange(r * t, dtype=np.uint32), h, 99, outlier_period=100).view(r, t, h)
     assert torch.equal(world.topk_idx_all.cpu(), topk_all)
     assert torch.equal(world.x_all.cpu().view(torch.int16), x_all.view(torch.int16))
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8, own_last=own_last(one_call, t, k, e, t))
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, O.ROW_FP8)
     check_dispatch(st, want, O.ROW_FP8)
     assert int(st.packed_recv_count[0]) > r * t // 2, "the hottest expert should fill over half its slots"
     # round trip with identity experts: combined == x * sum(w) within FP8 error
@@ -553,7 +547,7 @@ def test_empty_batch(rt, one_call):
     run_dispatch(st, world, x_all[rank, :0].cuda(), topk_all[rank, :0].cuda(), one_call=one_call)
     xs, tks = list(x_all), list(topk_all)
     xs[rank], tks[rank] = xs[rank][:0], tks[rank][:0]
-    want = O.ll_dispatch(xs, tks, rank, e, t, O.ROW_FP8, own_last=own_last(one_call, 0, k, e, t))
+    want = O.ll_dispatch(xs, tks, rank, e, t, O.ROW_FP8)
     check_dispatch(st, want, O.ROW_FP8)
     assert (st.send_count == 0).all()
 
@@ -704,7 +698,7 @@ def test_capacity_far_above_the_batch(rt, hint):
     run_dispatch(st, world, x, topk, None, one_call=True)
     single = rt.capi.load().deepep_ll_dispatch_is_single_launch(t, k, e, m, st.expected_rows) == 1
     assert single == (hint == "batch")
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, O.ROW_FP8, own_last=True)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, O.ROW_FP8)
     check_dispatch(st, want, O.ROW_FP8)
     # combine with identity experts
     epr = e // r
@@ -732,7 +726,7 @@ def test_tokens_naming_an_expert_more_than_once(rt, fmt, one_call):
                              [[2, 2, 0, -1], [2, 3, 3, 1], [0, 0, 0, 0], [2, 1, 2, 1], [-1, -1, 3, 3], [2, 2, 2, 2]]])
     w_all = torch.rand((r, t, k), generator=g) + 0.1
     st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, m, fmt, one_call=one_call)
-    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, fmt, own_last=one_call)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, fmt)
     check_dispatch(st, want, fmt)
     send_count, pair_slot = O.route(topk_all[rank], e, m)
     assert torch.equal(st.send_count.cpu(), send_count) and torch.equal(st.pair_slot[:t].cpu(), pair_slot)

@@ -35,7 +35,7 @@ def test_skew_stress_full_size(one_call):
     world = loopback.LoopbackWorld(r, rank, seed=seed)
     world.synthesise(t, h, k, e, popularity="zipf", outlier_period=100)
     x, topk = world.own_inputs()
-    if one_call:  # peers' rows first, then send + receive in one call: own segments sit behind the peers'
+    if one_call:  # peers' rows first, then send + receive in one call
         world.dispatch_from_peers(st)
         st.dispatch(x, topk)
     else:
@@ -55,7 +55,7 @@ def test_skew_stress_full_size(one_call):
     for le in range(epr):
         expert = rank * epr + le
         begin = 0
-        for s in ([q for q in range(r) if q != rank] + [rank] if one_call else range(r)):
+        for s in range(r):  # csrc/kernels/efa_kernels.cu:991-1010: ascending source rank
             tok = (np.nonzero(flat[s] == expert)[0] // k).astype(np.int32)
             seg_tokens[(le, s)] = (begin, tok)
             want = ((begin << 32) | len(tok)) if len(tok) else 0

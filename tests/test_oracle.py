@@ -221,29 +221,20 @@ def test_vectorised_dispatch_equals_serial_restatement(fmt):
             assert torch.equal(a[key], b[key]), (rank, key)
 
 
-def test_own_last_order_is_the_ascending_order_with_one_segment_moved():
-    """own_last only permutes whole segments: every (expert, source) segment keeps its rows and their order,
-    the own segment starts where the peers' rows end, the peers keep ascending order among themselves."""
+def test_ranges_are_the_serial_prefix_over_ascending_source_ranks():
+    """csrc/kernels/efa_kernels.cu:991-1010: begin(e, s) is the running sum of cnt(e, s') over s' < s, a
+    range is 0 where the count is 0, and the counts are the pairs naming the expert on each source."""
     xs, tk = _world(4, 8, 512, 3, 16, seed=5, drop=4)
     for rank in range(4):
-        a = O.ll_dispatch(xs, tk, rank, 16, 8, O.ROW_FP8)
-        b = O.ll_dispatch(xs, tk, rank, 16, 8, O.ROW_FP8, own_last=True)
-        assert torch.equal(a["packed_recv_count"], b["packed_recv_count"])
+        got = O.ll_dispatch(xs, tk, rank, 16, 8, O.ROW_FP8)
         for le in range(4):
-            la, lb = a["packed_recv_layout_range"][le], b["packed_recv_layout_range"][le]
-            assert torch.equal(la & 0xFFFFFFFF, lb & 0xFFFFFFFF)
             cursor = 0
-            for s in [x for x in range(4) if x != rank] + [rank]:
-                cnt = int(lb[s] & 0xFFFFFFFF)
-                if cnt == 0:
-                    assert int(lb[s]) == 0
-                    continue
-                assert int(lb[s] >> 32) == cursor
-                ba = int(la[s] >> 32)
-                for key in ("packed_recv_x", "packed_recv_scales", "packed_recv_src_info"):
-                    assert torch.equal(a[key][le, ba:ba + cnt], b[key][le, cursor:cursor + cnt]), (rank, le, s, key)
+            for s in range(4):
+                cnt = sum(1 for row in tk[s].tolist() for e in row if e == rank * 4 + le)
+                lr = int(got["packed_recv_layout_range"][le, s])
+                assert lr == (((cursor << 32) | cnt) if cnt else 0), (rank, le, s)
                 cursor += cnt
-            assert cursor == int(b["packed_recv_count"][le])
+            assert cursor == int(got["packed_recv_count"][le])
 
 
 def test_dispatch_invariants_of_reference_test():
@@ -466,13 +457,12 @@ def test_combine_reduce_definitions_agree():
 from tiny_world import load_tiny_world, tiny_world_expected  # noqa: E402
 
 
-@pytest.mark.parametrize("key,rank,own_last", [("rank0_ascending", 0, False), ("rank0_own_last", 0, True),
-                                               ("rank1_ascending", 1, False)])
+@pytest.mark.parametrize("key,rank", [("rank0_ascending", 0), ("rank1_ascending", 1)])
 @pytest.mark.parametrize("fmt", [O.ROW_BF16, O.ROW_FP8])
-def test_oracle_against_the_hand_derived_world(key, rank, own_last, fmt):
+def test_oracle_against_the_hand_derived_world(key, rank, fmt):
     g, x_all, topk_all = load_tiny_world()
     e, m, h = g["num_experts"], g["max_tokens"], g["hidden"]
-    got = O.ll_dispatch(x_all, topk_all, rank, e, m, fmt, own_last=own_last)
+    got = O.ll_dispatch(x_all, topk_all, rank, e, m, fmt)
     want, layout = tiny_world_expected(g, key)
     assert got["packed_recv_count"].tolist() == want["count"]
     assert torch.equal(got["packed_recv_layout_range"], layout)

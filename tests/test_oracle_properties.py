@@ -63,12 +63,12 @@ def test_route_slots_are_the_serial_scan(w):
 
 
 @settings(max_examples=60, deadline=None)
-@given(worlds(), st.booleans())
-def test_dispatch_is_the_brute_force_gather(w, own_last):
+@given(worlds())
+def test_dispatch_is_the_brute_force_gather(w):
     r, e, k, t, m, rank, x_all, topk_all = w
-    got = O.ll_dispatch(x_all, topk_all, rank, e, m, O.ROW_BF16, own_last=own_last)
+    got = O.ll_dispatch(x_all, topk_all, rank, e, m, O.ROW_BF16)
     epr = e // r
-    order = [s for s in range(r) if s != rank] + [rank] if own_last else list(range(r))
+    order = list(range(r))  # csrc/kernels/efa_kernels.cu:991-1010: ascending source rank
     for le in range(epr):
         ex = rank * epr + le
         rows, srcs, begin = [], [], {}
