@@ -438,47 +438,70 @@ __device__ __forceinline__ int clamp_count(int c, int max_tokens) {
     return c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
 }
 
-// own_cnt[e_l] (LDS, unclamped) = rows this rank sends to its own expert e_l, by the whole workgroup;
-// ends with a barrier.
-__device__ __forceinline__ void own_row_counts(const RecvArgs& a, const int64_t* own_topk, int own_entries,
-                                               int own_rank, int32_t* own_cnt) {
+// own_cnt[e_l] (LDS, unclamped) = rows this rank sends to its own expert e_l, counted by the whole
+// workgroup in two steps so that other loads can be issued in between: `begin` issues the first index
+// loads and clears the counters, `finish` counts and ends with a barrier.
+constexpr int kOwnAhead = 4;  // index loads in flight per thread
+
+struct OwnCountLoads {
+    int64_t v[kOwnAhead];
+};
+
+__device__ __forceinline__ void own_row_counts_begin(const RecvArgs& a, const int64_t* own_topk, int own_entries,
+                                                     int32_t* own_cnt, OwnCountLoads& loads) {
     const int tid = threadIdx.x, threads = blockDim.x;
-    if (own_topk == nullptr) {
+    if (own_topk == nullptr) return;
+#pragma unroll
+    for (int r = 0; r < kOwnAhead; ++r) {
+        const int i = tid + r * threads;
+        loads.v[r] = i < own_entries ? own_topk[i] : -1;
+    }
+    for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
+    lds_barrier();
+}
+
+__device__ __forceinline__ void own_row_counts_finish(const RecvArgs& a, const int64_t* own_topk, int own_entries,
+                                                      int own_rank, int32_t* own_cnt, OwnCountLoads& loads) {
+    const int tid = threadIdx.x, threads = blockDim.x;
+    if (own_topk == nullptr) {  // the send kernel has finished: recv_count holds the own counts
         for (int le = tid; le < a.num_local_experts; le += threads)
             own_cnt[le] = a.recv_count[le * a.num_ranks + own_rank];
         lds_barrier();
         return;
     }
-    constexpr int kAhead = 4;  // loads in flight per thread
-    int64_t v[kAhead];
-#pragma unroll
-    for (int r = 0; r < kAhead; ++r) {
-        const int i = tid + r * threads;
-        v[r] = i < own_entries ? own_topk[i] : -1;
-    }
-    for (int le = tid; le < a.num_local_experts; le += threads) own_cnt[le] = 0;
-    lds_barrier();
     const int64_t first = int64_t(own_rank) * a.num_local_experts;
-    for (int base = 0; base < own_entries; base += kAhead * threads) {
-        int64_t next[kAhead];
+    for (int base = 0; base < own_entries; base += kOwnAhead * threads) {
+        int64_t next[kOwnAhead];
 #pragma unroll
-        for (int r = 0; r < kAhead; ++r) {
-            const int i = base + (kAhead + r) * threads + tid;
+        for (int r = 0; r < kOwnAhead; ++r) {
+            const int i = base + (kOwnAhead + r) * threads + tid;
             next[r] = i < own_entries ? own_topk[i] : -1;
         }
 #pragma unroll
-        for (int r = 0; r < kAhead; ++r) {
-            const int64_t d = v[r] - first;
-            if (v[r] >= 0 && d >= 0 && d < a.num_local_experts) atomicAdd(&own_cnt[int(d)], 1);
-            v[r] = next[r];
+        for (int r = 0; r < kOwnAhead; ++r) {
+            const int64_t d = loads.v[r] - first;
+            if (loads.v[r] >= 0 && d >= 0 && d < a.num_local_experts) atomicAdd(&own_cnt[int(d)], 1);
+            loads.v[r] = next[r];
         }
     }
     lds_barrier();
 }
 
+// One unit of the copying waves' work: a run of 16-byte vectors of one staged row.
+struct RecvItem {
+    const uint8_t* src;
+    int le, source, slot;  // slot: the row's place among the rows copied for the expert, own rows not counted
+    int v_begin, v_end;
+    bool carries_tail;  // also moves the row's scales and source index
+};
+
+constexpr int kRecvDepth = 4;  // 16-byte loads in flight per lane
+
 // Workgroups [0, num_copy_blocks) copy rows; workgroup num_copy_blocks writes layout_range,
 // packed_count and stats and copies nothing.  A copying wave builds the segment prefix in its own
-// registers (WaveSegments) from the E counts.
+// registers (WaveSegments) from the E counts.  Where a row lands may depend on the own count of its
+// expert, where it comes from does not: a wave issues the loads of its first item before the
+// workgroup settles the own counts.
 // lds: [num_segments + 1 + num_local_experts] ints; wave_totals: 16 ints.
 template <int kPer>
 __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int num_copy_blocks,
@@ -489,10 +512,14 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
     const int num_ranks = a.num_ranks, max_tokens = a.max_tokens;
     const int num_segments = a.num_local_experts * num_ranks;
     const bool own_placed = own_rank >= 0;
+    OwnCountLoads own_loads;
 
     if (block == num_copy_blocks) {  // the metadata workgroup
         int32_t* own_cnt = lds + num_segments + 1;
-        if (own_placed) own_row_counts(a, own_topk, own_entries, own_rank, own_cnt);
+        if (own_placed) {
+            own_row_counts_begin(a, own_topk, own_entries, own_cnt, own_loads);
+            own_row_counts_finish(a, own_topk, own_entries, own_rank, own_cnt, own_loads);
+        }
         for (int s = tid; s < num_segments; s += threads) {
             const int le = s / num_ranks;
             const bool own = own_placed && s - le * num_ranks == own_rank;
@@ -514,11 +541,11 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
         return;
     }
 
+    int32_t* own_cnt = lds;  // [E_l]
     WaveSegments<kPer> seg_table;
     DEEPEP_PHASE(0);
+    if (own_placed) own_row_counts_begin(a, own_topk, own_entries, own_cnt, own_loads);
     wave_load_int32<kPer>(a.recv_count, num_segments, lane, seg_table.cnt);
-    int32_t* own_cnt = lds;  // [E_l]
-    if (own_placed) own_row_counts(a, own_topk, own_entries, own_rank, own_cnt);
 #pragma unroll
     for (int u = 0; u < kPer; ++u) {
         seg_table.aux[u] = 0;
@@ -544,29 +571,66 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
     const int num_vec = int(data_bytes / 16);
     const int parts = 1 << a.parts_log2;
     const int num_items = seg_table.total << a.parts_log2;
-    for (int item = block * waves + w; item < num_items; item += waves_total) {
+
+    auto decode = [&](int item, RecvItem& it) {
         const int row = item >> a.parts_log2, part = item & (parts - 1);
         int seg_first, unused;
         const int seg = wave_segments_find(seg_table, row, seg_first, unused);
-        const int le = seg / num_ranks;
-        const int j = row - seg_first;
-        int slot = row - wave_segments_prefix(seg_table, le * num_ranks);
-        if (own_placed && seg - le * num_ranks > own_rank) slot += clamp_count(own_cnt[le], max_tokens);
-        const uint8_t* src = a.recv_staging + (int64_t(seg) * max_tokens + j) * stride;
-        const int64_t out_row = int64_t(le) * slots_per_expert + slot;
-        int v_begin, v_end;
-        row_part_range(num_vec, parts, part, v_begin, v_end);
-        DEEPEP_PHASE(2);
-        wave_copy_vec16<4>(src, a.packed_x + out_row * data_bytes, v_begin, v_end, lane);
-        DEEPEP_PHASE(3);
-        if (part != parts - 1) continue;  // the last part is the shortest: it also carries scales and source index
+        it.le = seg / num_ranks;
+        it.source = seg - it.le * num_ranks;
+        it.slot = row - wave_segments_prefix(seg_table, it.le * num_ranks);
+        it.src = a.recv_staging + (int64_t(seg) * max_tokens + (row - seg_first)) * stride;
+        row_part_range(num_vec, parts, part, it.v_begin, it.v_end);
+        it.carries_tail = part == parts - 1;  // the last part is the shortest
+    };
+    auto load_first = [&](const RecvItem& it, u32x4 (&r)[kRecvDepth]) {
+#pragma unroll
+        for (int u = 0; u < kRecvDepth; ++u) {
+            const int v = it.v_begin + u * kWave + lane;
+            if (v < it.v_end) r[u] = load_u32x4<false>(it.src + int64_t(v) * 16);
+        }
+    };
+    auto finish = [&](const RecvItem& it, const u32x4 (&r)[kRecvDepth]) {
+        int slot = it.slot;
+        if (own_placed && it.source > own_rank) slot += clamp_count(own_cnt[it.le], max_tokens);
+        const int64_t out_row = int64_t(it.le) * slots_per_expert + slot;
+        uint8_t* dst = a.packed_x + out_row * data_bytes;
+#pragma unroll
+        for (int u = 0; u < kRecvDepth; ++u) {
+            const int v = it.v_begin + u * kWave + lane;
+            if (v < it.v_end) store_u32x4<false>(dst + int64_t(v) * 16, r[u]);
+        }
+        wave_copy_vec16<kRecvDepth>(it.src, dst, it.v_begin + kRecvDepth * kWave, it.v_end, lane);
+        if (!it.carries_tail) return;
         if (a.packed_scales != nullptr && scale_bytes > 0) {
-            const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src + data_pad);
+            const uint32_t* s32 = reinterpret_cast<const uint32_t*>(it.src + data_pad);
             uint32_t* d32 = reinterpret_cast<uint32_t*>(a.packed_scales + out_row * scale_bytes);
             for (int v = lane; v < int(scale_bytes / 4); v += kWave) d32[v] = s32[v];
         }
         if (lane == 0)
-            a.src_info[out_row] = *reinterpret_cast<const int32_t*>(src + data_pad + align16(scale_bytes));
+            a.src_info[out_row] = *reinterpret_cast<const int32_t*>(it.src + data_pad + align16(scale_bytes));
+    };
+
+    RecvItem it;
+    u32x4 r[kRecvDepth];
+    int item = block * waves + w;
+    const bool have_first = item < num_items;
+    if (have_first) {
+        decode(item, it);
+        DEEPEP_PHASE(2);
+        load_first(it, r);
+    }
+    // every wave of the workgroup passes here, with or without rows to copy
+    if (own_placed) own_row_counts_finish(a, own_topk, own_entries, own_rank, own_cnt, own_loads);
+    if (have_first) {
+        finish(it, r);
+        DEEPEP_PHASE(3);
+        item += waves_total;
+    }
+    for (; item < num_items; item += waves_total) {
+        decode(item, it);
+        load_first(it, r);
+        finish(it, r);
     }
 }
 
