@@ -29,6 +29,7 @@ PROTOTYPES = {
     "deepep_per_token_cast_to_fp8": (_I, [_VP, _I, _I, _I, _VP, _VP, _VP]),
     "deepep_ll_dispatch_workspace_bytes": (_SZ, [_I, _I, _I]),
     "deepep_ll_dispatch_send": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
+    "deepep_ll_dispatch_send_static": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP]),
     "deepep_ll_segment_workspace_bytes": (_SZ, [_I, _I]),
     "deepep_ll_dispatch_recv": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _VP, _I64, _VP, _SZ, _VP]),
     "deepep_ll_combine_send": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _VP, _VP, _I64, _VP, _SZ, _VP]),

@@ -17,8 +17,16 @@
 #include "quant.hpp"
 #include "segments.hpp"
 #include <cstdlib>
+#include <mutex>
 
 #include "../../include/deepep_hip.h"
+
+// Route scratch (the chunk histograms of ll_chunk_hist_kernel) for deepep_ll_dispatch_send_static,
+// whose callers cannot allocate.  The array is part of the code object: every GPU the library runs
+// on holds its own copy, at its own address, until the process ends.  Host code never passes this
+// name to a kernel; it passes the device address hipGetSymbolAddress returns (static_route_scratch).
+constexpr size_t kStaticScratchBytes = size_t(1) << 20;
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
 
 namespace deepep {
 
@@ -861,6 +869,59 @@ int deepep_ll_dispatch_send(const void* x, const int64_t* topk_idx, int num_toke
     return launch_send_side(x, topk_idx, nullptr, 1, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
                             num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count, send_slots,
                             send_count, pair_slot, workspace, workspace_bytes,
+                            reinterpret_cast<hipStream_t>(stream));
+}
+
+// Device address of `scratch` on the GPU that `stream` runs on, looked up once per device.
+static int static_route_scratch(hipStream_t stream, void** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static void* address[kMaxDevices] = {};
+    int device = -1;
+    EP_HIP_CHECK(hipGetDevice(&device));
+    EP_HOST_ASSERT(device >= 0 && device < kMaxDevices);
+    if (stream != nullptr) {  // the symbol's address is per device: the stream must be the current device's
+        int stream_device = -1;
+        EP_HIP_CHECK(hipStreamGetDevice(stream, &stream_device));
+        EP_HOST_ASSERT(stream_device == device);
+    }
+    std::lock_guard<std::mutex> lock(mutex);
+    if (address[device] == nullptr) {
+        void* p = nullptr;
+        EP_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        EP_HOST_ASSERT(p != nullptr);
+        address[device] = p;
+    }
+    *out = address[device];
+    return 0;
+}
+
+int deepep_ll_dispatch_send_static(const void* x, const int64_t* topk_idx, int num_tokens, int hidden, int num_topk,
+                                   int num_experts, int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                                   int row_format, void* recv_staging, int32_t* recv_count, void* send_slots,
+                                   int32_t* send_count, int32_t* pair_slot, void* stream) {
+    clear_error();
+    if (int rc = check_ll_shape(num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                                num_max_dispatch_tokens_per_rank, row_format))
+        return rc;
+    const size_t need = size_t(route_scratch_bytes(num_tokens, num_topk, num_experts));
+    if (need > kStaticScratchBytes) {
+        set_error("Assertion", __FILE_NAME__, __LINE__,
+                  "batch too large for the static route scratch: ceil(num_tokens / floor(2048 / num_topk)) * "
+                  "num_experts * 4 bytes must not exceed 1 MiB; use deepep_ll_dispatch_send with a workspace");
+        return 1;
+    }
+    void* route_scratch = nullptr;
+    if (int rc = static_route_scratch(reinterpret_cast<hipStream_t>(stream), &route_scratch)) return rc;
+    EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
+    EP_HOST_ASSERT(recv_staging != nullptr && recv_count != nullptr);
+    EP_HOST_ASSERT(send_count != nullptr && pair_slot != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_staging) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(send_slots) & 15) == 0);
+    return launch_send_side(x, topk_idx, nullptr, 1, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                            num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count, send_slots,
+                            send_count, pair_slot, route_scratch, kStaticScratchBytes,
                             reinterpret_cast<hipStream_t>(stream));
 }
 

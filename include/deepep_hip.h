@@ -232,6 +232,28 @@ int deepep_ll_dispatch_send(const void* x, const int64_t* topk_idx,
                             void* send_slots, int32_t* send_count, int32_t* pair_slot,
                             void* workspace, size_t workspace_bytes, void* stream);
 
+/* deepep_ll_dispatch_send without the workspace arguments: the route scratch is an array inside
+ * the library image (1 MiB on every GPU the library runs on, held until the process ends), so the
+ * call allocates nothing and needs nothing allocated for it.  No counterpart in the reference; it
+ * is for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  Same arguments, outputs and errors as
+ * deepep_ll_dispatch_send otherwise.
+ *   Limit: deepep_ll_dispatch_workspace_bytes(T, K, E) <= 1 MiB, i.e.
+ *   ceil(T / floor(2048 / K)) * E * 4 <= 1048576 (at K = 8, E = 256: T <= 262144); a larger batch
+ *   fails with a message that says so.
+ *   `stream` must belong to the current device.  The array's address is looked up on the first
+ *   call on each device (a host-side query, no device work).
+ *   Every call on a GPU shares that GPU's array: two calls that overlap in time on one GPU (on
+ *   different streams, or from different threads) race.  Nothing in it has to start at zero: a
+ *   call overwrites every word it later reads. */
+int deepep_ll_dispatch_send_static(const void* x, const int64_t* topk_idx,
+                                   int num_tokens, int hidden, int num_topk, int num_experts,
+                                   int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                                   int row_format,
+                                   void* recv_staging, int32_t* recv_count,
+                                   void* send_slots, int32_t* send_count, int32_t* pair_slot,
+                                   void* stream);
+
 /* Receive side: compacts the staged rows of every (local expert, source
  * rank) segment into the packed layout.
  *   begin(e,s) = sum_{s' < s} recv_count[e,s'];  rows [begin, begin+cnt)
