@@ -192,7 +192,6 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
     skewed: at 8192 tokens, 64 ranks x 4 experts, Zipf(1.2) expert popularity with rank 0 holding the hottest
     experts and 1 % of the rows scaled by 100 (needs ~150 GB of HBM)."""
     t, h, k, e, r, rank = (8192, 7168, 8, 256, 64, 0) if skewed else (4096, 7168, 8, 256, 8, 3)
-    h = int(os.environ.get("DEEPEP_BENCH_LARGE_HIDDEN", h))  # tuning aid
     shape = ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8)
     st = ll_runtime.LowLatencyState(shape)
     world = loopback.LoopbackWorld(r, rank, seed=args.seed + 7)
@@ -258,6 +257,8 @@ def main():
                     help="only run N eager dispatch / combine pairs, each call after a 512 MiB flush of the caches "
                          "(writes, or reads with --cold-by-reads), for a rocprofv3 kernel trace")
     ap.add_argument("--cold-by-reads", action="store_true")
+    ap.add_argument("--only-ll-4096", action="store_true",
+                    help="only time the LL entry points at 4096 tokens (8 ranks x 32 experts) and print that section")
     ap.add_argument("--skew-stress", action="store_true",
                     help="only time the LL entry points at the skewed 8192-token, 64-rank stress size and print that")
     args = ap.parse_args()
@@ -278,7 +279,7 @@ def main():
     if args.skew_stress:
         print(json.dumps(bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=True)))
         return
-    if os.environ.get("DEEPEP_BENCH_ONLY_LARGE") == "1":  # tuning aid: the 4096-token section alone
+    if args.only_ll_4096:
         print(json.dumps(bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args)))
         return
     t, h, k, e, r, rank = args.tokens, args.hidden, args.topk, args.experts, args.ranks, args.rank

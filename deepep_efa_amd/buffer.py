@@ -208,6 +208,8 @@ class Buffer:
           handle   (src_info [E_l, N] int32, layout_range [E_l, R] int64 = (begin << 32) | count,
                    num_max_dispatch_tokens_per_rank, hidden, num_experts);
           the returned tensors are reused by the next call with the same shape.
+        async_finish is accepted and an event is returned either way, as in the reference
+        (deep_ep/buffer.py:2449 returns EventOverlap(EventHandle()) whatever the flag says).
         """
         prof = None
         if _PROFILE_ENABLED:
@@ -228,12 +230,19 @@ class Buffer:
     def low_latency_combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor, handle: tuple,
                             use_logfmt: bool = False, zero_copy: bool = False, async_finish: bool = False,
                             return_recv_hook: bool = False, out: Optional[torch.Tensor] = None,
-                            combine_wait_recv_cost_stats: Optional[torch.Tensor] = None):
+                            combine_wait_recv_cost_stats: Optional[torch.Tensor] = None, *,
+                            accumulate: bool = False):
         """x [E_l, N, H] bf16 expert outputs laid out like the dispatch result.
 
         Returns (combined_x [T, H] bf16, event, hook) with
         combined_x[t] = bf16(sum_k [topk_idx[t,k] >= 0] * topk_weights[t,k] * x_returned[t,k]), float32 accumulate.
+        accumulate (needs `out`): the sum starts from float32(out[t]) instead of zero — the flag the
+        reference's reduce takes (csrc/kernels/coop_combine_recv.cuh:174-179) and its Python fixes to False
+        (deep_ep/buffer.py:2541).
+        async_finish is accepted and an event is returned either way, as in the reference
+        (deep_ep/buffer.py:2801-2803 returns EventOverlap(EventHandle()) whatever the flag says).
         """
+        assert not accumulate or out is not None, "accumulate adds to `out`"
         src_info, layout_range, num_max_dispatch_tokens_per_rank, hidden, num_experts = handle
         prof = None
         if _PROFILE_ENABLED:
@@ -243,7 +252,8 @@ class Buffer:
             prof.mark("start")
         combined_x, event, hook = self.runtime.low_latency_combine(
             x, topk_idx, topk_weights, src_info, layout_range, combine_wait_recv_cost_stats,
-            num_max_dispatch_tokens_per_rank, num_experts, use_logfmt, zero_copy, True, return_recv_hook, out)
+            num_max_dispatch_tokens_per_rank, num_experts, use_logfmt, zero_copy, True, return_recv_hook, out,
+            accumulate)
         if prof:
             prof.mark("end")
             prof.finish_iter()

@@ -98,15 +98,8 @@ __device__ __forceinline__ void store_u32x4(uint8_t* p, u32x4 v) {
     if constexpr (kStream) __builtin_nontemporal_store(v, (global_u32x4*)(p));
     else *(global_u32x4*)(p) = v;
 }
-// Traffic above which a kernel streams (the memory-side cache holds 256 MB).  DEEPEP_STREAM_MB
-// overrides the bound, for tuning.
-inline int64_t stream_bytes() {
-    static const int64_t v = [] {
-        const char* s = getenv("DEEPEP_STREAM_MB");
-        return (s != nullptr ? int64_t(atoll(s)) : int64_t(192)) << 20;
-    }();
-    return v;
-}
+// Traffic above which a kernel streams (the memory-side cache holds 256 MB).
+inline int64_t stream_bytes() { return int64_t(192) << 20; }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
 // outstanding global load and store of the wave, which stalls kernels that keep row loads in

@@ -17,6 +17,7 @@
 #include <optional>
 #include <string>
 #include <tuple>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/deepep_hip.h"
@@ -185,7 +186,8 @@ struct Buffer {
     bool available = false, destroyed = false;
     int device_id = 0;
     HostStream comm_stream;
-    torch::Tensor nvl_buffer, rdma_buffer, layout_workspace, mask_status;
+    torch::Tensor nvl_buffer, rdma_buffer, mask_status;
+    std::unordered_map<int64_t, torch::Tensor> layout_workspaces;  // one per stream that has run the layout kernel
     LowLatencyCache ll;
     std::vector<torch::Tensor> combine_input_buffers;
     int combine_buffer_idx = 0;
@@ -249,7 +251,7 @@ struct Buffer {
         if (available) (void)hipDeviceSynchronize();
         nvl_buffer = torch::Tensor();
         rdma_buffer = torch::Tensor();
-        layout_workspace = torch::Tensor();
+        layout_workspaces.clear();
         ll = LowLatencyCache();
         combine_input_buffers.clear();
         world_x.reset();
@@ -306,8 +308,12 @@ struct Buffer {
 
         const int64_t ws_bytes =
             std::max<int64_t>(256, int64_t(deepep_layout_workspace_bytes(num_tokens, num_ranks, num_experts)));
-        if (!layout_workspace.defined() or layout_workspace.numel() < ws_bytes)
+        // the kernel's scratch belongs to the stream the kernel runs on: a call on the buffer's own stream and
+        // one on the caller's stream may be in flight together
+        torch::Tensor& layout_workspace = layout_workspaces[int64_t(work_stream.id())];
+        if (!layout_workspace.defined() or layout_workspace.numel() < ws_bytes) {
             layout_workspace = torch::empty({ws_bytes}, torch::dtype(torch::kUInt8).device(torch::kCUDA));
+        }
 
         abi_check(deepep_get_dispatch_layout(
             topk_idx.data_ptr<int64_t>(), num_tokens, num_topk, num_ranks, num_experts,
@@ -513,8 +519,11 @@ struct Buffer {
         const torch::Tensor& src_info, const torch::Tensor& layout_range,
         const std::optional<torch::Tensor>& combine_wait_recv_cost_stats, int num_max_dispatch_tokens_per_rank,
         int num_experts, bool use_logfmt, bool zero_copy, bool async, bool return_recv_hook,
-        const std::optional<torch::Tensor>& out) {
+        const std::optional<torch::Tensor>& out, bool accumulate) {
         (void)use_logfmt;
+        // accumulate: the sum starts from what `out` holds (the reference has the flag on its reduce binding,
+        // csrc/deep_ep.cpp:3850-3857, kernel csrc/kernels/coop_combine_recv.cuh:174-179)
+        EP_HOST_ASSERT(not accumulate or out.has_value());
         EP_HOST_ASSERT(low_latency_mode);
         // reference checks: csrc/deep_ep.cpp:1816-1837
         EP_HOST_ASSERT(x.dim() == 3 and x.is_contiguous() and x.scalar_type() == torch::kBFloat16);
@@ -570,7 +579,7 @@ struct Buffer {
         abi_check(deepep_ll_combine(src.data_ptr(), layout_range.data_ptr<int64_t>(), topk_idx.data_ptr<int64_t>(),
                                     topk_weights.data_ptr<float>(), c.pair_slot.data_ptr<int>(), num_combined_tokens,
                                     hidden, num_topk, num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,
-                                    /*accumulate=*/0, c.combine_staging.data_ptr(), c.combine_send_slots.data_ptr(),
+                                    accumulate ? 1 : 0, c.combine_staging.data_ptr(), c.combine_send_slots.data_ptr(),
                                     combined_x.data_ptr(), /*expected_rows=*/std::max<int64_t>(num_combined_tokens, 1) * num_topk,
                                     c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
                                     c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));
@@ -858,7 +867,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         .def("get_dispatch_layout", &deep_ep::Buffer::get_dispatch_layout)
         .def("clean_low_latency_buffer", &deep_ep::Buffer::clean_low_latency_buffer)
         .def("low_latency_dispatch", &deep_ep::Buffer::low_latency_dispatch)
-        .def("low_latency_combine", &deep_ep::Buffer::low_latency_combine)
+        .def("low_latency_combine", &deep_ep::Buffer::low_latency_combine, py::arg("x"), py::arg("topk_idx"),
+             py::arg("topk_weights"), py::arg("src_info"), py::arg("layout_range"),
+             py::arg("combine_wait_recv_cost_stats"), py::arg("num_max_dispatch_tokens_per_rank"),
+             py::arg("num_experts"), py::arg("use_logfmt"), py::arg("zero_copy"), py::arg("async"),
+             py::arg("return_recv_hook"), py::arg("out"), py::arg("accumulate") = false)
         .def("low_latency_update_mask_buffer", &deep_ep::Buffer::low_latency_update_mask_buffer)
         .def("low_latency_query_mask_buffer", &deep_ep::Buffer::low_latency_query_mask_buffer)
         .def("low_latency_clean_mask_buffer", &deep_ep::Buffer::low_latency_clean_mask_buffer)

@@ -706,30 +706,6 @@ static int check_ll_shape(int num_tokens, int hidden, int num_topk, int num_expe
     return 0;
 }
 
-static int send_split_override() {
-    static const int v = [] {
-        const char* s = getenv("DEEPEP_SEND_SPLIT");
-        return s != nullptr ? atoi(s) : 0;
-    }();
-    return v;
-}
-
-static int self_rank_max_override() {
-    static const int v = [] {
-        const char* s = getenv("DEEPEP_SELF_RANK_MAX");
-        return s != nullptr ? atoi(s) : 0;
-    }();
-    return v;
-}
-
-static int send_waves_override() {
-    static const int v = [] {
-        const char* s = getenv("DEEPEP_SEND_WAVES");
-        return s != nullptr ? atoi(s) : 0;
-    }();
-    return v;
-}
-
 static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_t* src_ranks, int num_src,
                             int num_tokens, int hidden, int num_topk, int num_experts, int num_ranks, int rank,
                             int max_tokens, int row_format, void* recv_staging, int32_t* recv_count,
@@ -743,8 +719,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     uint8_t* ws = reinterpret_cast<uint8_t*>(workspace);
     // How slots get ranked: up to kSelfRankMaxEntries entries the send kernel sweeps every earlier
     // entry itself; beyond, it sweeps its own chunk on top of the per-chunk histograms.
-    const int self_rank_max = self_rank_max_override() > 0 ? self_rank_max_override() : kSelfRankMaxEntries;
-    const int tpc = n <= self_rank_max || fused_recv != nullptr ? 0 : sweep_chunk_tokens(num_topk);
+    const int tpc = n <= kSelfRankMaxEntries || fused_recv != nullptr ? 0 : sweep_chunk_tokens(num_topk);
     if (tpc > 0) {
         const int chunks = (num_tokens + tpc - 1) / tpc;
         ll_chunk_hist_kernel<<<dim3(chunks, num_src), 1024, size_t(num_experts) * sizeof(int32_t), stream>>>(
@@ -759,13 +734,8 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     // In the single launch the receive workgroups share the chip: whole tokens per workgroup, and
     // workgroups small enough that two fit a compute unit.
     if (fused_recv != nullptr) split_log2 = 0;
-    if (send_split_override() == 1) split_log2 = 0;
-    if (send_split_override() == 2) split_log2 = 1;
-    if (send_split_override() == 4) split_log2 = 2;
     const int items = pieces << split_log2;  // waves per token
-    int max_waves = kSendMaxWaves;
-    if (send_waves_override() >= 1 && send_waves_override() <= kSendMaxWaves) max_waves = send_waves_override();
-    if (fused_recv != nullptr && max_waves > 8) max_waves = 8;
+    const int max_waves = fused_recv != nullptr ? 8 : kSendMaxWaves;
     int waves = items < max_waves ? items : max_waves;
     const int blocks_per_token = (items + waves - 1) / waves;
     if (fused_recv != nullptr && waves < 4) waves = 4;  // the receive workgroups want a few waves each

@@ -5,8 +5,6 @@
 // of kernels for large batches.
 #pragma once
 
-#include <cstdlib>
-
 #include "common.hpp"
 
 namespace deepep {
@@ -172,13 +170,6 @@ __device__ __forceinline__ void row_part_range(int num_vec, int parts, int part,
 // one wave per row.
 inline int choose_row_parts_log2(int64_t estimated_rows, int64_t row_bytes) {
     if (estimated_rows > 8192) return 0;
-    if (const char* s = getenv("DEEPEP_ROW_PARTS")) {
-        const int v = atoi(s);
-        if (v == 1) return 0;
-        if (v == 2) return 1;
-        if (v == 4) return 2;
-        if (v == 8) return 3;
-    }
     return row_bytes > 8192 ? 2 : 1;
 }
 

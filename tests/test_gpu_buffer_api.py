@@ -179,6 +179,60 @@ def test_dispatch_matches_oracle_through_the_api(deep_ep):
     buffer.destroy()
 
 
+def test_combine_accumulates_into_out_through_the_api(deep_ep):
+    """accumulate=True starts the float32 sum from what `out` holds (csrc/kernels/coop_combine_recv.cuh:174-179):
+    checked bit for bit against the float32 FMA chain started from the previous contents."""
+    num_ranks, rank, t, h, k, e = 8, 5, 48, 1024, 4, 64
+    buffer = deep_ep.Buffer(None, low_latency_mode=True, explicitly_destroy=True, sim_num_ranks=num_ranks,
+                            sim_rank=rank, sim_seed=11)
+    x, topk_idx = buffer.loopback_synthesise(t, h, k, e)
+    topk_idx = topk_idx.clone()
+    topk_idx[7, 2] = -1
+    topk_idx[9, :] = -1  # a token sent nowhere keeps what `out` held
+    w = torch.rand((t, k), generator=torch.Generator().manual_seed(2)).cuda()
+    recv_x, recv_count, handle, _, _ = buffer.low_latency_dispatch(x, topk_idx, t, e, use_fp8=False)
+    y = recv_x.clone()  # identity experts on the bf16 rows: every pair's answer is x[t] itself
+    prev = torch.randn((t, h), generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    plain, _, _ = buffer.low_latency_combine(y, topk_idx, w, handle)
+    plain = plain.clone()
+    out = prev.cuda()
+    got, _, _ = buffer.low_latency_combine(y, topk_idx, w, handle, out=out, accumulate=True)
+    torch.cuda.synchronize()
+    assert got.data_ptr() == out.data_ptr()
+    pair_rows = x.cpu().unsqueeze(1).expand(t, k, h)
+    live = topk_idx.cpu() >= 0
+    want_plain = O.ll_combine_f32_chain(pair_rows, w.cpu(), live)
+    want_acc = O.ll_combine_f32_chain(pair_rows, w.cpu(), live, initial=prev)
+    assert torch.equal(plain.cpu().view(torch.int16), want_plain.view(torch.int16))
+    assert torch.equal(got.cpu().view(torch.int16), want_acc.view(torch.int16))
+    assert torch.equal(got[9].cpu().view(torch.int16), prev[9].view(torch.int16))
+    with pytest.raises(AssertionError, match="accumulate adds to `out`"):
+        buffer.low_latency_combine(y, topk_idx, w, handle, accumulate=True)
+    buffer.destroy()
+
+
+def test_layout_calls_on_two_streams_in_flight_together(deep_ep):
+    """An asynchronous call (on the buffer's stream) followed by a synchronous one (on the caller's) before
+    the first event is waited on: each stream has its own scratch, so both give the right counts."""
+    num_ranks, num_experts, num_tokens, num_topk = 8, 256, 4096, 8
+    buffer = deep_ep.Buffer(None, explicitly_destroy=True, sim_num_ranks=num_ranks, sim_rank=1)
+    g = torch.Generator().manual_seed(99)
+    topk_a = torch.topk(torch.rand((num_tokens, num_experts), generator=g), num_topk, dim=-1)[1]
+    topk_b = torch.topk(torch.rand((num_tokens, num_experts), generator=g), num_topk, dim=-1)[1]
+    dev_a, dev_b = topk_a.cuda(), topk_b.cuda()
+    want_a = O.get_dispatch_layout(topk_a, num_experts, num_ranks)
+    want_b = O.get_dispatch_layout(topk_b, num_experts, num_ranks)
+    for _ in range(20):
+        ra = buffer.get_dispatch_layout(dev_a, num_experts, async_finish=True)
+        rb = buffer.get_dispatch_layout(dev_b, num_experts)
+        ra[4].current_stream_wait()
+        torch.cuda.synchronize()
+        for got, want in ((ra, want_a), (rb, want_b)):
+            assert torch.equal(got[0].cpu(), want[0]) and torch.equal(got[2].cpu(), want[2])
+            assert torch.equal(got[3].cpu(), want[3])
+    buffer.destroy()
+
+
 def test_get_dispatch_layout_api(deep_ep):
     """tests/test_intranode.py:35-66 recipe, plus the event plumbing of csrc/deep_ep.cpp:526-574."""
     for num_ranks, num_experts, num_tokens, num_topk in ((8, 256, 4096, 8), (16, 256, 128, 8), (64, 256, 333, 6)):
