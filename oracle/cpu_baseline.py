@@ -71,8 +71,17 @@ class CpuRankStep:
         return out, layout, len(owed)
 
 
+def host_threads() -> int:
+    """Threads the CPU legs run on: every core the host reports, or the share of them the job was
+    given when the launcher says so through OMP_NUM_THREADS (a GPU box hands one GPU's job 16 cores of a
+    host that reports many more)."""
+    n = os.cpu_count() or 1
+    share = os.environ.get("OMP_NUM_THREADS", "")
+    return min(n, int(share)) if share.isdigit() and int(share) > 0 else n
+
+
 def time_cpu_step(step: CpuRankStep, budget_s: float = 15.0, min_runs: int = 5):
-    threads = min(os.cpu_count() or 1, 16)
+    threads = host_threads()
     torch.set_num_threads(threads)
     for _ in range(2):
         step.step()
@@ -81,6 +90,45 @@ def time_cpu_step(step: CpuRankStep, budget_s: float = 15.0, min_runs: int = 5):
     while len(times) < min_runs or (time.perf_counter() - t0 < budget_s and len(times) < 200):
         a = time.perf_counter()
         step.step()
+        times.append(time.perf_counter() - a)
+    times.sort()
+    return times[len(times) // 2], threads, len(times)
+
+
+class CpuReferenceCase:
+    """The reference's own CPU-runnable case: 128 tokens x 7168 bf16 ~N(0,1), 256 experts, top-8 uniform without
+    replacement, weights = softmax of N(0,1) logits, simulated EP=16 (16 local experts per rank).  One pass =
+    get_dispatch_layout counts (csrc/kernels/layout.cu:9-121), the per-token per-128-channel FP8 cast
+    (deep_ep/buffer.py:1590-1621) and the top-k weighted combine sum with float32 accumulation
+    (csrc/kernels/coop_combine_recv.cuh:222-260) over the dequantised rows."""
+
+    def __init__(self, num_tokens=128, hidden=7168, num_experts=256, num_topk=8, num_ranks=16, seed=0):
+        g = torch.Generator().manual_seed(seed)
+        self.x = torch.randn((num_tokens, hidden), generator=g).to(torch.bfloat16)
+        self.topk = torch.stack([torch.randperm(num_experts, generator=g)[:num_topk] for _ in range(num_tokens)])
+        self.w = torch.softmax(torch.randn((num_tokens, num_topk), generator=g), dim=-1)
+        self.e, self.r, self.k = num_experts, num_ranks, num_topk
+
+    def step(self):
+        per_rank, _, per_expert, is_in = O.get_dispatch_layout(self.topk, self.e, self.r)
+        q, s = O.per_token_cast_to_fp8(self.x)
+        y = O.per_token_cast_back(q, s)  # every expert returns the row it was sent
+        pair_rows = y.unsqueeze(1).expand(-1, self.k, -1)
+        out = O.ll_combine_f32_chain(pair_rows, self.w, self.topk >= 0)
+        return per_rank, per_expert, is_in, q, s, out
+
+
+def time_reference_case(budget_s: float = 5.0, min_runs: int = 5):
+    case = CpuReferenceCase()
+    threads = host_threads()
+    torch.set_num_threads(threads)
+    for _ in range(2):
+        case.step()
+    times = []
+    t0 = time.perf_counter()
+    while len(times) < min_runs or (time.perf_counter() - t0 < budget_s and len(times) < 200):
+        a = time.perf_counter()
+        case.step()
         times.append(time.perf_counter() - a)
     times.sort()
     return times[len(times) // 2], threads, len(times)
