@@ -45,6 +45,8 @@ def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0, packed=None):
                      + (rv - own) * (stride + packed) + small),
         "combine": (rv - own) * 2 * h * 2 + (e // r) * r * 8 + p * 2 * h + t * k * 16 + t * 2 * h,
         "exchange_metadata": r * e * 4 + rv * 16 + r * 24,
+        # the staged receive's bytes plus, per row, the record, the tail read and the descriptor
+        "dispatch_recv_by_source": rv * stride + rv * packed + small + rv * 12,
     }
 
 
@@ -110,6 +112,39 @@ def read_traffic_summary(kernel, stamp):
         if len(parts) >= 4 and parts[0] == kernel and parts[1].isdigit() and parts[2].isdigit():
             return int(parts[1]) + int(parts[2])
     return None
+
+
+def by_source_receive(torch, _capi, lib, ll_runtime, st, world):
+    """Sets up the receive path a source-grouped transport feeds: the staged rows regrouped by source rank
+    into one slotted buffer (slot = the most rows one source can send), the exchange-metadata records for the
+    world's route counts, and the call that consumes both.  Returns (callable, rows expected)."""
+    sh = st.shape
+    r, e, m, el = sh.num_ranks, sh.num_experts, sh.max_tokens, sh.num_local_experts
+    slot_rows = m * min(sh.num_topk, el)
+    staging = st.recv_staging.view(el, r, m, st.stride)
+    count = st.recv_count.view(el, r).cpu()
+    buf = torch.empty((r * slot_rows, st.stride), dtype=torch.uint8, device="cuda")
+    for src in range(r):
+        off = src * slot_rows
+        for le in range(el):
+            c = int(count[le, src])
+            buf[off:off + c] = staging[le, src, :c]
+            off += c
+    tk = world.topk_idx_all.view(r, -1)
+    routed = torch.stack([torch.bincount(tk[s][tk[s] >= 0], minlength=e) for s in range(r)]).to(torch.int32)
+    rows = int(count.sum())
+    meta = ll_runtime.exchange_metadata(routed, sh.rank, slot_rows, rows)
+    ws = torch.empty(lib.deepep_ll_by_source_workspace_bytes(e, rows), dtype=torch.uint8, device="cuda")
+    tokens_per_expert = torch.empty(el, dtype=torch.int32, device="cuda")
+
+    def call():
+        _capi.check(lib.deepep_ll_dispatch_recv_by_source(
+            _capi.ptr(buf), slot_rows, _capi.ptr(meta["recv_counts"]), _capi.ptr(meta["source_offset"]),
+            _capi.ptr(meta["num_recv_tokens"]), rows, sh.hidden, e, r, m, sh.fmt, _capi.ptr(st.packed_recv_x),
+            _capi.ptr(st.packed_recv_scales), _capi.ptr(st.packed_recv_src_info),
+            _capi.ptr(st.packed_recv_layout_range), _capi.ptr(st.packed_recv_count), None,
+            _capi.ptr(tokens_per_expert), _capi.ptr(ws), ws.numel(), torch.cuda.current_stream().cuda_stream))
+    return call, rows
 
 
 def bench_pack(torch, _capi, lib, loopback, args):
@@ -242,6 +277,8 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
         "dispatch": lambda: st.dispatch(x, topk),
         "combine": lambda: st.combine(y, topk, weights, out),
     }
+    if not skewed:  # the receive side fed by a source-grouped transport (same bytes as dispatch_recv)
+        calls["dispatch_recv_by_source"], _ = by_source_receive(torch, _capi, lib, ll_runtime, st, world)
     res = {"workload": f"LL dispatch+combine at {t} tokens x {h}, top-{k} of {e} experts, {r} ranks x {epr} experts"
                        + (", Zipf(1.2) expert popularity, 1 % outlier rows" if skewed else ""),
            "pairs_sent": p, "rows_received": rv, "rows_to_own_experts": own}
@@ -427,6 +464,8 @@ def main():
         "combine_send": lambda: st.combine_send(y),
         "combine_recv": lambda: st.combine_recv(topk, weights, out),
     }
+    # the receive side fed by a source-grouped transport: consumes the exchange-metadata records
+    calls["dispatch_recv_by_source"], _ = by_source_receive(torch, _capi, lib, ll_runtime, st, world)
     step_calls = ("dispatch", "combine")  # what deep_ep.Buffer.low_latency_dispatch / _combine launch
     phase_calls = ("dispatch_send", "dispatch_recv", "combine_send", "combine_recv")
 

@@ -42,6 +42,9 @@ PROTOTYPES = {
     "deepep_topk_remap": (_I, [_VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP]),
     "deepep_build_recv_src_meta": (_I, [_VP, _I, _I, _I64, _VP, _VP]),
     "deepep_ll_exchange_metadata": (_I, [_VP, _I, _I, _I, _I, _I64] + [_VP] * 11),
+    "deepep_ll_by_source_workspace_bytes": (_SZ, [_I, _I64]),
+    "deepep_ll_dispatch_recv_by_source": (_I, [_VP, _I64, _VP, _VP, _VP, _I64, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP,
+                                               _VP, _VP, _VP, _VP, _SZ, _VP]),
     "deepep_combine_reduce_workspace_bytes": (_SZ, [_I, _I]),
     "deepep_combine_reduce": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP, _SZ, _VP]),
     "deepep_synth_topk_idx": (_I, [_VP, _VP, _I, _I, _I, _I, _U32, _VP, _VP]),

@@ -12,7 +12,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdeepep_hip.so")
-SOURCES = ["lib.cpp", "ll_dispatch.hip", "ll_combine.hip", "ll_exchange_meta.hip", "layout.hip", "normal_meta.hip", "cast.hip", "loopback.hip"]
+SOURCES = ["lib.cpp", "ll_dispatch.hip", "ll_combine.hip", "ll_exchange_meta.hip", "ll_recv_by_source.hip", "layout.hip", "normal_meta.hip", "cast.hip", "loopback.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
          "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

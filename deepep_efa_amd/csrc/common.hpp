@@ -46,7 +46,7 @@ enum RowFormat : int { kRowBF16 = 0, kRowFP8 = 1, kRowFP8Pow2 = 2, kRowFP8UE8M0 
 
 constexpr int kWave = 64;
 constexpr int kGroup = 128;        // channels per FP8 scale group
-constexpr int kRowTailBytes = 16;  // {src_token, topk_slot, src_rank, 0}
+constexpr int kRowTailBytes = 16;  // {src_token, topk_slot, src_rank, local expert}
 
 __host__ __device__ inline int64_t align16(int64_t v) { return (v + 15) & ~int64_t(15); }
 

@@ -8,7 +8,7 @@
 //                 order of the sender.
 //   recv_count    [E_l][R] int32 — rows present in each segment.
 //   send_slots    [E][M] rows — this rank's rows for remote experts.
-// A staged row is [data | pad16][scales | pad16][src_token, k, src_rank, 0].
+// A staged row is [data | pad16][scales | pad16][src_token, k, src_rank, local expert].
 //
 // Work is cut per wavefront, never per thread block: one wave owns one 1 KiB
 // piece of one row, so a 64-lane 16-byte access is one contiguous KiB and no
@@ -362,7 +362,7 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
         if (block_in_token == 0) {
             if (a.pair_slot != nullptr) a.pair_slot[entry0 + tid] = my_slot;
             if (staged) {
-                u32x4 tail = {uint32_t(t), uint32_t(tid), uint32_t(src_rank), 0u};
+                u32x4 tail = {uint32_t(t), uint32_t(tid), uint32_t(src_rank), uint32_t(local)};
                 *reinterpret_cast<u32x4*>(row + data_pad + scale_pad) = tail;
             }
         }

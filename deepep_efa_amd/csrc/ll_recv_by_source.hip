@@ -1,0 +1,263 @@
+// Receive side of the low-latency dispatch for a transport that delivers rows grouped by source
+// rank, the way an all-to-all does: the rows of source s sit in slot s of one buffer in the order
+// they arrived, and the records of deepep_ll_exchange_metadata say where each expected row is
+// (source_offset).  Every row carries its local expert in the last word of its tail, as the
+// reference's packed rows carry [token, local_eid] (csrc/kernels/efa_kernels.cu:797-800).
+//
+// Same outputs as deepep_ll_dispatch_recv.  Reference: ll_recv_unpack_v2
+// (csrc/kernels/efa_kernels.cu:2121-2231): count the (expert, source) pairs from the rows' metadata
+// (:877-923, slot addressing :906-913), build the ranges as a prefix over ascending source rank
+// (:991-1010), scatter every row to range begin + its rank inside the pair (:1227-1389).  The
+// reference claims that rank with an atomic; here it is the row's arrival order inside its source,
+// so the result does not depend on scheduling.
+//
+// Three launches: pair counts (one workgroup per source), ranges + one {source row, packed row}
+// descriptor per record (one workgroup per source), and the flat row copy the other large-batch
+// paths use.
+#include "common.hpp"
+#include "segments.hpp"
+#include "../../include/deepep_hip.h"
+
+namespace deepep {
+
+constexpr int kBySourceThreads = 512;
+constexpr int kBySourceWaves = kBySourceThreads / kWave;
+constexpr int kBySourceMaxRanks = 1024;
+constexpr int kBySourceMaxLocalExperts = 1024;
+
+// Exclusive prefix of recv_counts (negative counts read as 0) over the ranks, by the whole workgroup:
+// records [prefix[s], prefix[s + 1]) belong to source s.  prefix has num_ranks + 1 entries.
+__device__ __forceinline__ void source_prefix(const int32_t* __restrict__ recv_counts, int num_ranks, int32_t* prefix,
+                                              int32_t* scan_tmp) {
+    for (int r = threadIdx.x; r < num_ranks; r += blockDim.x) {
+        const int c = recv_counts[r];
+        prefix[r] = c < 0 ? 0 : c;
+    }
+    lds_barrier();
+    block_exclusive_scan(prefix, num_ranks, scan_tmp);
+}
+
+// The records of source s that are looked at: [begin, end) exist, those from `live_end` on lie past the
+// source's slot of slot_rows rows (or past the records written) and are not copied.
+__device__ __forceinline__ void source_records(const int32_t* prefix, int s, int num_ranks, int slot_rows,
+                                               int64_t records, int64_t& begin, int64_t& end, int64_t& live_end) {
+    begin = prefix[s];
+    end = prefix[s + 1];
+    if (end > records) end = records;
+    if (begin > end) begin = end;
+    live_end = begin + slot_rows < end ? begin + slot_rows : end;
+}
+
+// Local expert of the row a record points at, or -1 when the record or the row's tail is out of range.
+__device__ __forceinline__ int record_expert(const uint8_t* __restrict__ recv_by_source, int64_t stride,
+                                             int64_t tail_off, uint32_t offset, int64_t buffer_rows,
+                                             int num_local_experts) {
+    if (int64_t(offset) >= buffer_rows) return -1;
+    const int e = *reinterpret_cast<const int32_t*>(recv_by_source + int64_t(offset) * stride + tail_off + 12);
+    return e >= 0 && e < num_local_experts ? e : -1;
+}
+
+// pair_counts[e_l * R + s] = records of source s whose row names local expert e_l.
+__global__ __launch_bounds__(kBySourceThreads) void ll_by_source_count_kernel(
+    const uint8_t* __restrict__ recv_by_source, int64_t stride, int64_t tail_off, int64_t buffer_rows, int slot_rows,
+    const int32_t* __restrict__ recv_counts, const uint32_t* __restrict__ source_offset,
+    const uint32_t* __restrict__ num_recv_tokens, int64_t row_capacity, int num_local_experts, int num_ranks,
+    int32_t* __restrict__ pair_counts) {
+    extern __shared__ int32_t lds[];  // prefix [R + 1] | hist [E_l]
+    __shared__ int32_t scan_tmp[kMaxBlockWaves];
+    int32_t* prefix = lds;
+    int32_t* hist = lds + num_ranks + 1;
+    const int s = blockIdx.x, tid = threadIdx.x;
+    source_prefix(recv_counts, num_ranks, prefix, scan_tmp);
+    for (int e = tid; e < num_local_experts; e += kBySourceThreads) hist[e] = 0;
+    lds_barrier();
+    int64_t records = num_recv_tokens[1];
+    if (records > row_capacity) records = row_capacity;
+    int64_t begin, end, live_end;
+    source_records(prefix, s, num_ranks, slot_rows, records, begin, end, live_end);
+    for (int64_t i = begin + tid; i < live_end; i += kBySourceThreads) {
+        const int e = record_expert(recv_by_source, stride, tail_off, source_offset[i], buffer_rows, num_local_experts);
+        if (e >= 0) atomicAdd(&hist[e], 1);
+    }
+    lds_barrier();
+    for (int e = tid; e < num_local_experts; e += kBySourceThreads) pair_counts[e * num_ranks + s] = hist[e];
+}
+
+// Ranges from the pair counts (every workgroup, the first one writes them), then for the records
+// of source blockIdx.x, in arrival order: packed row = range begin + rows of the same pair before it.
+__global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
+    const uint8_t* __restrict__ recv_by_source, int64_t stride, int64_t tail_off, int64_t buffer_rows, int slot_rows,
+    const int32_t* __restrict__ recv_counts, const uint32_t* __restrict__ source_offset,
+    const uint32_t* __restrict__ num_recv_tokens, int64_t row_capacity, int num_local_experts, int num_ranks,
+    int max_tokens, const int32_t* __restrict__ pair_counts, int64_t* __restrict__ layout_range,
+    int32_t* __restrict__ packed_count, int32_t* __restrict__ stats, uint32_t* __restrict__ tokens_per_expert,
+    int32_t* __restrict__ flat_total, RowDesc* __restrict__ desc) {
+    extern __shared__ int32_t lds[];  // prefix [R + 1] | pair_prefix [E_l * R + 1] | running [E_l] | wave_cnt [waves][E_l]
+    __shared__ int32_t scan_tmp[kMaxBlockWaves];
+    const int num_segments = num_local_experts * num_ranks;
+    int32_t* prefix = lds;
+    int32_t* pair_prefix = prefix + num_ranks + 1;
+    int32_t* running = pair_prefix + num_segments + 1;
+    int32_t* wave_cnt = running + num_local_experts;
+    const int s = blockIdx.x, tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
+    const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
+
+    source_prefix(recv_counts, num_ranks, prefix, scan_tmp);
+    for (int q = tid; q < num_segments; q += kBySourceThreads) {
+        const int c = pair_counts[q];
+        pair_prefix[q] = c < 0 ? 0 : c;
+    }
+    lds_barrier();
+    block_exclusive_scan(pair_prefix, num_segments, scan_tmp);
+    int64_t records = num_recv_tokens[1];
+    if (records > row_capacity) records = row_capacity;
+    if (s == 0) {
+        // csrc/kernels/efa_kernels.cu:991-1010: begin = rows of the lower source ranks, 0 where the count is 0
+        for (int q = tid; q < num_segments; q += kBySourceThreads) {
+            const int le = q / num_ranks;
+            const int64_t cnt = pair_prefix[q + 1] - pair_prefix[q];
+            const int64_t begin = pair_prefix[q] - pair_prefix[le * num_ranks];
+            layout_range[q] = cnt > 0 ? ((begin << 32) | cnt) : 0;
+        }
+        for (int le = tid; le < num_local_experts; le += kBySourceThreads) {
+            const int c = pair_prefix[(le + 1) * num_ranks] - pair_prefix[le * num_ranks];
+            packed_count[le] = c;
+            if (stats != nullptr) stats[le] += c;
+            if (tokens_per_expert != nullptr) tokens_per_expert[le] = uint32_t(c);
+        }
+        if (tid == 0) flat_total[0] = int32_t(records < prefix[num_ranks] ? records : prefix[num_ranks]);
+    }
+    for (int e = tid; e < num_local_experts; e += kBySourceThreads) running[e] = 0;
+
+    int64_t begin, end, live_end;
+    source_records(prefix, s, num_ranks, slot_rows, records, begin, end, live_end);
+    int expert_bits = 0;
+    while ((1 << expert_bits) < num_local_experts) ++expert_bits;
+    for (int64_t base = begin; base < end; base += kBySourceThreads) {  // batches of rows, in arrival order
+        for (int q = tid; q < kBySourceWaves * num_local_experts; q += kBySourceThreads) wave_cnt[q] = 0;
+        lds_barrier();
+        const int64_t i = base + tid;
+        uint32_t offset = 0;
+        int e = -1;
+        if (i < live_end) {
+            offset = source_offset[i];
+            e = record_expert(recv_by_source, stride, tail_off, offset, buffer_rows, num_local_experts);
+        }
+        // the lanes of this wave whose row names the same expert: one ballot per bit of the expert id
+        uint64_t same = __ballot(e >= 0);
+        for (int bit = 0; bit < expert_bits; ++bit) {
+            const uint64_t set = __ballot(e >= 0 && ((e >> bit) & 1) != 0);
+            same &= ((e >> bit) & 1) != 0 ? set : ~set;
+        }
+        const int before_in_wave = __popcll(same & lanes_below(lane));
+        if (e >= 0 && (same >> lane) >> 1 == 0) wave_cnt[w * num_local_experts + e] = __popcll(same);  // the group's last lane
+        lds_barrier();
+        if (i < end) {
+            RowDesc d;
+            d.src_row = -1, d.dst_row = 0;  // a row without a valid expert is not copied
+            if (e >= 0) {
+                int pos = running[e] + before_in_wave;
+                for (int w2 = 0; w2 < w; ++w2) pos += wave_cnt[w2 * num_local_experts + e];
+                const int64_t pair_begin = pair_prefix[e * num_ranks + s] - pair_prefix[e * num_ranks];
+                if (pair_begin + pos < slots_per_expert) {
+                    d.src_row = int32_t(offset);
+                    d.dst_row = int32_t(int64_t(e) * slots_per_expert + pair_begin + pos);
+                }
+            }
+            desc[i] = d;
+        }
+        lds_barrier();
+        for (int e2 = tid; e2 < num_local_experts; e2 += kBySourceThreads) {
+            int add = 0;
+            for (int w2 = 0; w2 < kBySourceWaves; ++w2) add += wave_cnt[w2 * num_local_experts + e2];
+            running[e2] += add;
+        }
+        lds_barrier();
+    }
+}
+
+}  // namespace deepep
+
+using namespace deepep;
+
+extern "C" {
+
+size_t deepep_ll_by_source_workspace_bytes(int num_experts, int64_t row_capacity) {
+    const int64_t head = ((int64_t(num_experts) + 64) * 4 + 255) & ~int64_t(255);  // pair counts, row total
+    return size_t(head + (row_capacity < 1 ? 1 : row_capacity) * int64_t(sizeof(RowDesc)));
+}
+
+int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_rows, const int32_t* recv_counts,
+                                      const uint32_t* source_offset, const uint32_t* num_recv_tokens,
+                                      int64_t row_capacity, int hidden, int num_experts, int num_ranks,
+                                      int num_max_dispatch_tokens_per_rank, int row_format, void* packed_recv_x,
+                                      void* packed_recv_scales, int32_t* packed_recv_src_info,
+                                      int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
+                                      int32_t* cumulative_local_expert_recv_stats, uint32_t* tokens_per_expert,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+    clear_error();
+    EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
+    EP_HOST_ASSERT(num_ranks > 0 && num_ranks <= kBySourceMaxRanks);
+    EP_HOST_ASSERT(num_experts > 0 && num_experts % num_ranks == 0);
+    const int num_local_experts = num_experts / num_ranks;
+    EP_HOST_ASSERT(num_local_experts <= kBySourceMaxLocalExperts && num_experts <= 4096);
+    EP_HOST_ASSERT(num_max_dispatch_tokens_per_rank > 0);
+    EP_HOST_ASSERT(row_format >= kRowBF16 && row_format <= kRowFP8UE8M0);
+    EP_HOST_ASSERT(row_format != kRowFP8UE8M0 || (hidden / 128) % 4 == 0);
+    EP_HOST_ASSERT(slot_rows > 0 && slot_rows * num_ranks < (int64_t(1) << 31));
+    EP_HOST_ASSERT(row_capacity >= 0 && row_capacity < (int64_t(1) << 31));
+    EP_HOST_ASSERT(int64_t(num_experts) * num_max_dispatch_tokens_per_rank < (int64_t(1) << 31));
+    EP_HOST_ASSERT(recv_by_source != nullptr && recv_counts != nullptr && num_recv_tokens != nullptr);
+    EP_HOST_ASSERT(row_capacity == 0 || source_offset != nullptr);
+    EP_HOST_ASSERT(packed_recv_x != nullptr && (row_format == kRowBF16 || packed_recv_scales != nullptr));
+    EP_HOST_ASSERT(packed_recv_src_info != nullptr && packed_recv_layout_range != nullptr &&
+                   packed_recv_count != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_by_source) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_x) & 15) == 0);
+    EP_HOST_ASSERT(workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
+    EP_HOST_ASSERT(workspace_bytes >= deepep_ll_by_source_workspace_bytes(num_experts, row_capacity));
+    // LDS of the index kernel: prefix, pair prefix, running counts, per-wave counts
+    const size_t index_lds = size_t(num_ranks + 1 + num_experts + 1 + num_local_experts +
+                                    kBySourceWaves * num_local_experts) * sizeof(int32_t);
+    EP_HOST_ASSERT(index_lds <= 64 * 1024);
+
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    const int64_t stride = row_stride_bytes(hidden, row_format);
+    const int64_t data_bytes = row_data_bytes(hidden, row_format);
+    const int64_t scale_bytes = row_scale_bytes(hidden, row_format);
+    const int64_t tail_off = align16(data_bytes) + align16(scale_bytes);
+    const int64_t buffer_rows = slot_rows * num_ranks;
+    int32_t* pair_counts = reinterpret_cast<int32_t*>(workspace);
+    int32_t* flat_total = pair_counts + num_experts;
+    const int64_t head = ((int64_t(num_experts) + 64) * 4 + 255) & ~int64_t(255);
+    RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) + head);
+
+    const size_t count_lds = size_t(num_ranks + 1 + num_local_experts) * sizeof(int32_t);
+    ll_by_source_count_kernel<<<num_ranks, kBySourceThreads, count_lds, hs>>>(
+        reinterpret_cast<const uint8_t*>(recv_by_source), stride, tail_off, buffer_rows, int(slot_rows), recv_counts,
+        source_offset, num_recv_tokens, row_capacity, num_local_experts, num_ranks, pair_counts);
+    EP_LAUNCH_CHECK();
+    ll_by_source_index_kernel<<<num_ranks, kBySourceThreads, index_lds, hs>>>(
+        reinterpret_cast<const uint8_t*>(recv_by_source), stride, tail_off, buffer_rows, int(slot_rows), recv_counts,
+        source_offset, num_recv_tokens, row_capacity, num_local_experts, num_ranks, num_max_dispatch_tokens_per_rank,
+        pair_counts, packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, tokens_per_expert,
+        flat_total, desc);
+    EP_LAUNCH_CHECK();
+    if (row_capacity == 0) return 0;
+    const int num_vec = int(data_bytes / 16);
+    int threads = ((num_vec + 63) / 64) * 64;
+    int extra = 64;  // one more wave for scales + source index
+    if (threads + extra > 1024) threads = 1024, extra = 0;
+    int64_t blocks = row_capacity;
+    if (blocks > 16384) blocks = blocks / 2 > 16384 ? blocks / 2 : 16384;
+    if (blocks > (int64_t(1) << 22)) blocks = int64_t(1) << 22;
+    ll_rows_flat_kernel<<<unsigned(blocks), threads + extra, 0, hs>>>(
+        flat_total, 0, desc, reinterpret_cast<const uint8_t*>(recv_by_source), stride, num_vec,
+        reinterpret_cast<uint8_t*>(packed_recv_x), nullptr, data_bytes, int(scale_bytes / 4), align16(data_bytes),
+        scale_bytes > 0 ? reinterpret_cast<uint8_t*>(packed_recv_scales) : nullptr, tail_off, packed_recv_src_info,
+        extra);
+    EP_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // extern "C"

@@ -181,7 +181,7 @@ inline int choose_row_parts_log2(int64_t estimated_rows, int64_t row_bytes) {
 // and writes a descriptor {source row, destination row} for each of its rows.
 // ---------------------------------------------------------------------
 struct RowDesc {
-    int32_t src_row;  // row index in the source buffer
+    int32_t src_row;  // row index in the source buffer; < 0: nothing to copy
     int32_t dst_row;  // >= 0: row index in the primary destination; < 0: -(1 + row) in the secondary one
 };
 
@@ -295,6 +295,7 @@ static __global__ __launch_bounds__(1024) void ll_rows_flat_kernel(
     const int total = flat[num_segments];
     for (int row = blockIdx.x; row < total; row += gridDim.x) {
         const RowDesc d = desc[row];
+        if (d.src_row < 0) continue;  // a record that names no row
         const uint8_t* s = src + int64_t(d.src_row) * src_stride;
         uint8_t* o;
         if (d.dst_row >= 0) {

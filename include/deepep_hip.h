@@ -62,7 +62,7 @@ size_t deepep_ll_row_data_bytes(int hidden, int row_format);
 /* Bytes of the scale part of a row (0 for bf16). */
 size_t deepep_ll_row_scale_bytes(int hidden, int row_format);
 /* Stride of one staged row: data and scales each padded to 16 B, plus a
- * 16 B tail {int32 src_token, int32 topk_slot, int32 src_rank, int32 0}.
+ * 16 B tail {int32 src_token, int32 topk_slot, int32 src_rank, int32 local expert}.
  * 7408 for fp8 at H = 7168 — the value the reference's cooperative send
  * uses (csrc/kernels/coop_dispatch_send.cu:73-75). */
 size_t deepep_ll_row_stride(int hidden, int row_format);
@@ -309,6 +309,39 @@ int deepep_ll_exchange_metadata(const int32_t* all_num_routed, int num_experts, 
                                 uint32_t* source_rank, uint32_t* source_offset, uint32_t* padded_index,
                                 uint32_t* combine_send_offset, uint32_t* num_recv_tokens,
                                 uint32_t* tokens_per_expert, void* stream);
+
+/* Bytes of scratch deepep_ll_dispatch_recv_by_source needs for `row_capacity` records. */
+size_t deepep_ll_by_source_workspace_bytes(int num_experts, int64_t row_capacity);
+
+/* deepep_ll_dispatch_recv for a transport that delivers rows grouped by source rank (what an
+ * all-to-all leaves behind): the rows of source s sit in slot s of `recv_by_source`, in the order
+ * they arrived, and the records of deepep_ll_exchange_metadata say where each expected row is.
+ * Same outputs as deepep_ll_dispatch_recv (ranges in ascending source order; inside an (expert,
+ * source) segment the rows keep their arrival order, which for a sender that emits in (token, k)
+ * order is the order of the staged form), plus the reference's tokens_per_expert.
+ *   recv_by_source  [R * slot_rows] rows of deepep_ll_row_stride bytes in the staged row format;
+ *                   the last int32 of a row's tail is its local expert id
+ *   slot_rows       rows one source's slot holds (the M the records were built with: record j of
+ *                   source s has source_offset = s * M + j); records past it are not copied
+ *   recv_counts     [R] int32 rows expected from each rank          } outputs of
+ *   source_offset   [row_capacity] uint32 row index of each record  } deepep_ll_exchange_metadata
+ *   num_recv_tokens [2] uint32: [1] = records present               }
+ *   tokens_per_expert [E_l] uint32 (out) = packed_recv_count, or NULL
+ *   workspace       deepep_ll_by_source_workspace_bytes(E, row_capacity) bytes
+ * Replaces ll_recv_unpack_v2 on its flat / slotted input (csrc/kernels/efa_kernels.cu:2121-2231,
+ * kernels :877-1052 and :1227-1389, slot addressing :906-913) and consumes the records
+ * a2a_dispatch_recv reads (csrc/kernels/coop_dispatch_recv.cuh:42, source_offset). */
+int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_rows,
+                                      const int32_t* recv_counts, const uint32_t* source_offset,
+                                      const uint32_t* num_recv_tokens, int64_t row_capacity,
+                                      int hidden, int num_experts, int num_ranks,
+                                      int num_max_dispatch_tokens_per_rank, int row_format,
+                                      void* packed_recv_x, void* packed_recv_scales,
+                                      int32_t* packed_recv_src_info, int64_t* packed_recv_layout_range,
+                                      int32_t* packed_recv_count,
+                                      int32_t* cumulative_local_expert_recv_stats,
+                                      uint32_t* tokens_per_expert,
+                                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Low-latency combine                                                */

@@ -406,9 +406,10 @@ def _serial_dispatch(all_x, all_topk_idx, rank: int, num_experts: int, max_token
 
 
 def staged_rows(x: torch.Tensor, topk_idx: torch.Tensor, src_rank: int, num_experts: int, max_tokens: int,
-                fmt: int):
+                fmt: int, num_ranks: int):
     """Rows one rank emits, keyed (expert, slot) -> stride-sized row bytes, as the
-    send side stages them: [data|pad][scales|pad][token, k, src_rank, 0]."""
+    send side stages them: [data|pad][scales|pad][token, k, src_rank, local expert] (the reference's
+    packed rows end in [token, local_eid], csrc/kernels/efa_kernels.cu:797-800)."""
     hidden = x.shape[1]
     db, sb = row_data_bytes(hidden, fmt), row_scale_bytes(hidden, fmt)
     dp, sp = align_up(db, 16), align_up(sb, 16)
@@ -420,8 +421,10 @@ def staged_rows(x: torch.Tensor, topk_idx: torch.Tensor, src_rank: int, num_expe
     rows[:, :db] = data[tok]
     if sb:
         rows[:, dp:dp + sb] = scales[tok]
+    experts_per_rank = num_experts // num_ranks
+    local = (topk_idx[tok, kk] % experts_per_rank).to(torch.int32)
     tail = torch.stack([tok.to(torch.int32), kk.to(torch.int32), torch.full_like(tok, src_rank, dtype=torch.int32),
-                        torch.zeros_like(tok, dtype=torch.int32)], 1).contiguous()
+                        local], 1).contiguous()
     rows[:, dp + sp:] = tail.view(torch.uint8).view(-1, 16)
     experts = topk_idx[tok, kk]
     slots = pair_slot[tok, kk].to(torch.int64)

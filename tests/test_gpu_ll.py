@@ -251,6 +251,104 @@ def test_exchange_metadata_hand_derived_world(rt):
             assert out[key][:n].cpu().tolist() == want[key], key
 
 
+def rows_by_source(x_all, topk_all, rank, e, m, fmt, slot_rows):
+    """What an all-to-all leaves on rank `rank`: for every source s, the rows it sends to this rank's experts,
+    in the sender's (token, k) order, at the start of slot s of one buffer (rows past the slot are lost)."""
+    r, _, h = x_all.shape
+    epr = e // r
+    stride = O.row_stride(h, fmt)
+    buf = torch.full((r * slot_rows, stride), 0xEE, dtype=torch.uint8)
+    for s in range(r):
+        _, _, experts, _, rows = O.staged_rows(x_all[s], topk_all[s], s, e, m, fmt, r)
+        mine = rows[(experts // epr) == rank][:slot_rows]
+        buf[s * slot_rows:s * slot_rows + mine.shape[0]] = mine
+    return buf
+
+
+def recv_by_source_on_gpu(rt, buf, routed, rank, e, m, h, fmt, slot_rows, capacity):
+    """The exchange-metadata records for `routed`, then the receive side fed from the per-source buffer."""
+    lib, capi = rt.capi.load(), rt.capi
+    r = routed.shape[0]
+    meta = rt.ll.exchange_metadata(routed.cuda(), rank, slot_rows, capacity)
+    shape = rt.ll.LLShape(num_ranks=r, rank=rank, num_experts=e, max_tokens=m, hidden=h, num_topk=1, fmt=fmt)
+    st = rt.ll.LowLatencyState(shape, keep_remote_rows=False)
+    poison_outputs(st)
+    ws = torch.empty(lib.deepep_ll_by_source_workspace_bytes(e, capacity), dtype=torch.uint8, device="cuda")
+    tokens_per_expert = torch.full((e // r,), 77, dtype=torch.int32, device="cuda")
+    dev = buf.cuda()
+    capi.check(lib.deepep_ll_dispatch_recv_by_source(
+        capi.ptr(dev), slot_rows, capi.ptr(meta["recv_counts"]), capi.ptr(meta["source_offset"]),
+        capi.ptr(meta["num_recv_tokens"]), capacity, h, e, r, m, fmt, capi.ptr(st.packed_recv_x),
+        capi.ptr(st.packed_recv_scales), capi.ptr(st.packed_recv_src_info), capi.ptr(st.packed_recv_layout_range),
+        capi.ptr(st.packed_recv_count), None, capi.ptr(tokens_per_expert), capi.ptr(ws), ws.numel(),
+        torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return st, tokens_per_expert, meta
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16, O.ROW_FP8_UE8M0])
+@pytest.mark.parametrize("r,rank,t,h,k,e", [
+    (4, 1, 8, 512, 3, 16), (8, 7, 33, 1024, 4, 64), (2, 0, 1, 512, 1, 2),
+    (32, 5, 128, 7168, 8, 256),   # the headline shape
+    (8, 3, 700, 512, 8, 256),     # sources with more rows than one batch of the index kernel: running counts
+    (1, 0, 16, 512, 2, 4),        # a world of one rank
+    (4, 2, 64, 512, 2, 4),        # one expert per rank
+    (2, 1, 40, 512, 6, 2048),     # 1024 local experts: ten bits of expert id
+])
+def test_dispatch_recv_by_source(rt, fmt, r, rank, t, h, k, e):
+    """Rows delivered grouped by source rank + the exchange-metadata records give the packed outputs of
+    the staged receive, i.e. the same oracle outputs (csrc/kernels/efa_kernels.cu:877-1052,1227-1389)."""
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=r * 31 + t, drop=min(5, t))
+    m = t
+    slot_rows = t * min(k, e // r)  # the most one source can send to one rank
+    buf = rows_by_source(x_all, topk_all, rank, e, m, fmt, slot_rows)
+    routed = torch.stack([O.route(topk_all[s], e, m)[0] for s in range(r)]).to(torch.int32)
+    capacity = int(routed[:, rank * (e // r):(rank + 1) * (e // r)].sum()) + 5
+    st, tokens_per_expert, meta = recv_by_source_on_gpu(rt, buf, routed, rank, e, m, h, fmt, slot_rows, capacity)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, fmt)
+    check_dispatch(st, want, fmt)
+    assert torch.equal(tokens_per_expert.cpu(), want["packed_recv_count"])
+    assert int(meta["num_recv_tokens"][0]) == int(want["packed_recv_count"].sum())
+
+
+def test_dispatch_recv_by_source_drops_what_does_not_fit(rt):
+    """A slot of M rows per source, as the reference sizes it (csrc/transport/ll_pipeline.cpp:1527): rows a
+    source sends beyond it are lost, the others land as if the lost ones had not been sent; and with fewer
+    record slots than rows, only the rows that have a record are received."""
+    r, rank, t, h, k, e, fmt = 2, 0, 24, 512, 4, 8, O.ROW_FP8
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=3, drop=0)
+    topk_all[1, :, :] = torch.tensor([0, 1, 2, 3])  # every token of source 1 names all of rank 0's experts
+    slot_rows = t  # source 1 sends 4 * t rows
+    buf = rows_by_source(x_all, topk_all, rank, e, t, fmt, slot_rows)
+    routed = torch.stack([O.route(topk_all[s], e, t)[0] for s in range(r)]).to(torch.int32)
+    for capacity in (4 * t * r, t // 2 + 3):
+        st, _, meta = recv_by_source_on_gpu(rt, buf, routed, rank, e, t, h, fmt, slot_rows, capacity)
+        recv_counts = meta["recv_counts"].cpu().tolist()
+        # expected: walk the records the way the kernel may use them
+        epr, n = e // r, 0
+        want_rows = [[[] for _ in range(r)] for _ in range(epr)]
+        tail = buf[:, -16:].contiguous().view(torch.int32)
+        for s in range(r):
+            for j in range(recv_counts[s]):
+                if n < capacity and j < slot_rows:
+                    row = s * slot_rows + j
+                    want_rows[int(tail[row, 3])][s].append(row)
+                n += 1
+        count = st.packed_recv_count.cpu().tolist()
+        layout = st.packed_recv_layout_range.cpu()
+        px = st.packed_recv_x.view(torch.uint8).cpu()
+        for le in range(epr):
+            begin = 0
+            for s in range(r):
+                rows = want_rows[le][s]
+                assert int(layout[le, s]) == (((begin << 32) | len(rows)) if rows else 0), (capacity, le, s)
+                for j, row in enumerate(rows):
+                    assert torch.equal(px[le, begin + j], buf[row, :h])
+                    assert int(st.packed_recv_src_info[le, begin + j]) == int(tail[row, 0])
+                begin += len(rows)
+            assert count[le] == begin
+
+
 def _random_shape(seed):
     g = np.random.default_rng(seed)
     r = int(g.choice([1, 2, 3, 4, 5, 6, 8, 12, 16, 24]))
@@ -313,7 +411,7 @@ def test_dispatch_send_staging_and_send_slots(rt):
     st.send_slots.fill_(0xCD)
     st.dispatch_send(x_all[rank].cuda(), topk_all[rank].cuda())
     torch.cuda.synchronize()
-    send_count, pair_slot, experts, slots, rows = O.staged_rows(x_all[rank], topk_all[rank], rank, e, m, O.ROW_FP8)
+    send_count, pair_slot, experts, slots, rows = O.staged_rows(x_all[rank], topk_all[rank], rank, e, m, O.ROW_FP8, r)
     assert torch.equal(st.send_count.cpu(), send_count)
     assert torch.equal(st.pair_slot[:t].cpu(), pair_slot)
     stride = st.stride

@@ -284,10 +284,10 @@ def test_route_slots_and_staged_rows():
             assert pair_slot[t, k] == seen.get(e, 0)
             seen[e] = seen.get(e, 0) + 1
     assert send_count.tolist() == [seen.get(e, 0) for e in range(8)]
-    sc, ps, experts, slots, rows = O.staged_rows(xs[0], tk[0], 1, 8, 10, O.ROW_FP8)
+    sc, ps, experts, slots, rows = O.staged_rows(xs[0], tk[0], 1, 8, 10, O.ROW_FP8, num_ranks=2)
     assert rows.shape[1] == O.row_stride(256, O.ROW_FP8) == 256 + 16 + 16
     tail = rows[:, -16:].contiguous().view(torch.int32)
-    assert (tail[:, 2] == 1).all() and (tail[:, 3] == 0).all()
+    assert (tail[:, 2] == 1).all() and torch.equal(tail[:, 3].long(), experts % 4)  # 8 experts on 2 ranks
     q, s = O.per_token_cast_to_fp8(xs[0])
     assert torch.equal(rows[:, :256], q.view(torch.uint8)[tail[:, 0].long()])
     assert torch.equal(rows[:, 256:264].contiguous().view(torch.float32), s[tail[:, 0].long()])
