@@ -10,7 +10,6 @@ produced in HBM by the loopback world (`loopback_set_world` /
 """
 import os
 import sys
-import time
 from collections import defaultdict
 from typing import Callable, Optional, Tuple
 
@@ -28,38 +27,42 @@ _PROFILE_WARMUP = int(os.environ.get("DEEPEP_PROFILE_WARMUP", "5"))
 
 
 class _LLProfiler:
-    """Wall-clock phase timing with a device sync at every mark (reference: deep_ep/buffer.py:27-77).
-    Enabled by DEEPEP_PROFILE=1; prints an average every DEEPEP_PROFILE_INTERVAL calls."""
+    """Per-phase timing of the low-latency calls, enabled by DEEPEP_PROFILE=1 (the reference's switch and
+    report line, deep_ep/buffer.py:20-77).  A mark is a HIP event recorded on the current stream, so marking
+    costs no device synchronisation; the events of DEEPEP_PROFILE_INTERVAL calls are resolved together, after
+    one synchronisation, when the report is due.  The first DEEPEP_PROFILE_WARMUP calls are not counted."""
 
     def __init__(self, name: str, rank: int):
         self.name, self.rank = name, rank
-        self.timestamps = {}
-        self.accum = defaultdict(float)
-        self.count = 0
-        self.warmup_remaining = _PROFILE_WARMUP
+        self.skip = _PROFILE_WARMUP
+        self.current = []   # (label, event) of the call in progress
+        self.finished = []  # one such list per counted call
 
     def mark(self, label: str) -> None:
-        torch.cuda.synchronize()
-        self.timestamps[label] = time.perf_counter_ns()
+        event = torch.cuda.Event(enable_timing=True)
+        event.record()
+        self.current.append((label, event))
 
     def finish_iter(self, extra_info: str = "") -> None:
-        if self.warmup_remaining > 0:
-            self.warmup_remaining -= 1
-            self.timestamps.clear()
+        marks, self.current = self.current, []
+        if self.skip > 0:
+            self.skip -= 1
             return
-        labels, times = list(self.timestamps), list(self.timestamps.values())
-        for i in range(1, len(labels)):
-            self.accum[f"{labels[i - 1]}->{labels[i]}"] += (times[i] - times[i - 1]) / 1000.0
-        if len(labels) >= 2:
-            self.accum["TOTAL"] += (times[-1] - times[0]) / 1000.0
-        self.count += 1
-        self.timestamps.clear()
-        if self.count >= _PROFILE_PRINT_EVERY:
-            parts = [f"{k}={v / self.count:.1f}us" for k, v in self.accum.items()]
-            msg = f"[LL_PROFILE rank={self.rank}] {self.name} (avg of {self.count}): {' | '.join(parts)}"
-            print(msg + (f" | {extra_info}" if extra_info else ""), file=sys.stderr, flush=True)
-            self.accum.clear()
-            self.count = 0
+        self.finished.append(marks)
+        if len(self.finished) < _PROFILE_PRINT_EVERY:
+            return
+        torch.cuda.synchronize()
+        sums = defaultdict(float)
+        for marks in self.finished:
+            for (a, ea), (b, eb) in zip(marks, marks[1:]):
+                sums[f"{a}->{b}"] += ea.elapsed_time(eb) * 1e3
+            if len(marks) >= 2:
+                sums["TOTAL"] += marks[0][1].elapsed_time(marks[-1][1]) * 1e3
+        n = len(self.finished)
+        self.finished = []
+        line = " | ".join(f"{phase}={total / n:.1f}us" for phase, total in sums.items())
+        tail = f" | {extra_info}" if extra_info else ""
+        print(f"[LL_PROFILE rank={self.rank}] {self.name} (avg of {n}): {line}{tail}", file=sys.stderr, flush=True)
 
 
 class Buffer:

@@ -233,6 +233,29 @@ def test_layout_calls_on_two_streams_in_flight_together(deep_ep):
     buffer.destroy()
 
 
+def test_profile_report_line(deep_ep, monkeypatch, capsys):
+    """DEEPEP_PROFILE=1 prints the reference's report line (deep_ep/buffer.py:67-76) every
+    DEEPEP_PROFILE_INTERVAL calls, after DEEPEP_PROFILE_WARMUP uncounted ones."""
+    import re
+    from deepep_efa_amd import buffer as buffer_module
+    monkeypatch.setattr(buffer_module, "_PROFILE_ENABLED", True)
+    monkeypatch.setattr(buffer_module, "_PROFILE_PRINT_EVERY", 2)
+    monkeypatch.setattr(buffer_module, "_PROFILE_WARMUP", 1)
+    buffer = deep_ep.Buffer(None, low_latency_mode=True, explicitly_destroy=True, sim_num_ranks=4, sim_rank=2)
+    x, topk_idx = buffer.loopback_synthesise(16, 512, 2, 16)
+    w = torch.ones((16, 2), dtype=torch.float32, device="cuda")
+    for call in range(5):  # 1 warm-up + 2 reports of 2 calls each
+        recv, _, handle, _, _ = buffer.low_latency_dispatch(x, topk_idx, 16, 16, use_fp8=False)
+        buffer.low_latency_combine(recv, topk_idx, w, handle)
+    torch.cuda.synchronize()
+    lines = [l for l in capsys.readouterr().err.splitlines() if l.startswith("[LL_PROFILE")]
+    assert len(lines) == 4
+    pattern = r"\[LL_PROFILE rank=2\] (DISPATCH|COMBINE) \(avg of 2\): start->end=\d+\.\d+us \| TOTAL=\d+\.\d+us"
+    assert all(re.fullmatch(pattern, l) for l in lines), lines
+    assert [l.split()[2] for l in lines] == ["DISPATCH", "COMBINE", "DISPATCH", "COMBINE"]
+    buffer.destroy()
+
+
 def test_get_dispatch_layout_api(deep_ep):
     """tests/test_intranode.py:35-66 recipe, plus the event plumbing of csrc/deep_ep.cpp:526-574."""
     for num_ranks, num_experts, num_tokens, num_topk in ((8, 256, 4096, 8), (16, 256, 128, 8), (64, 256, 333, 6)):
