@@ -375,12 +375,15 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a plain row copy of known size (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-profiler", action="store_true",
+                    help="skip the per-launch GPU timestamps taken with torch.profiler (for runs under rocprofv3)")
     ap.add_argument("--row-format", choices=["fp8", "bf16", "fp8_pow2", "fp8_ue8m0"], default="fp8",
                     help="dispatch payload (the headline workload is fp8); other formats skip the CPU baseline")
     ap.add_argument("--cold-trace", type=int, default=0, metavar="N",
                     help="only run N eager dispatch / combine pairs, each call after a 512 MiB flush of the caches "
                          "(writes, or reads with --cold-by-reads), for a rocprofv3 kernel trace")
     ap.add_argument("--cold-by-reads", action="store_true")
+    ap.add_argument("--no-skew-stress", action="store_true", help="skip the skewed 8192-token stress section")
     ap.add_argument("--only-ll-4096", action="store_true",
                     help="only time the LL entry points at 4096 tokens (8 ranks x 32 experts) and print that section")
     ap.add_argument("--skew-stress", action="store_true",
@@ -555,6 +558,8 @@ def main():
         — the clock rocprofv3's kernel trace reads.  HIP events cannot isolate a 10 us kernel that has to follow
         a flush: a pair of them around one launch costs ~7 us by itself (the *_two_trivial_launches_us lines).
         None when the profiler is unavailable."""
+        if args.no_profiler:
+            return None
         try:
             from torch.profiler import ProfilerActivity, profile
             for i in range(3):
@@ -687,7 +692,9 @@ def main():
         result["ll_4096_tokens"] = bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args)
         torch.cuda.empty_cache()
         free, _ = torch.cuda.mem_get_info()
-        if free >= 170 * 2 ** 30:
+        if args.no_skew_stress:
+            pass
+        elif free >= 170 * 2 ** 30:
             result["skew_stress"] = bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=True)
             torch.cuda.empty_cache()
         else:
