@@ -114,10 +114,33 @@ struct CombineRecvArgs {
     uint8_t* out;
 };
 
+// What lane k of a wave knows about selection k of its token once the index loads are back.
+struct CombineSelection {
+    int slot;
+    int64_t expert;
+    float weight;
+};
+
+// Issues the loads of selection `lane`'s (slot, expert, weight): one round of loads for the whole token.
+// Nothing here waits for them, so a caller can put other latency (the own-range lookup of the
+// single-launch combine) behind the same round trip.
+__device__ __forceinline__ CombineSelection combine_load_selection(const CombineRecvArgs& a, int64_t item) {
+    CombineSelection s = {-1, -1, 0.0f};
+    const int lane = lane_id();
+    if (item < int64_t(a.num_tokens) * a.pieces_per_row && lane < a.num_topk) {
+        const int64_t idx = (item / a.pieces_per_row) * a.num_topk + lane;
+        s.slot = a.pair_slot[idx];
+        s.expert = a.topk_idx[idx];
+        s.weight = a.topk_weights[idx];
+    }
+    return s;
+}
+
 template <bool kStream>
-__device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int64_t item, const uint8_t* own_x,
-                                                   const int32_t* own_begin, int own_first_expert,
-                                                   int num_local_experts, int64_t slots_per_expert) {
+__device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int64_t item, const CombineSelection& sel,
+                                                   const uint8_t* own_x, const int32_t* own_begin,
+                                                   int own_first_expert, int num_local_experts,
+                                                   int64_t slots_per_expert) {
     const int lane = lane_id();
     if (item >= int64_t(a.num_tokens) * a.pieces_per_row) return;
     const int t = int(item / a.pieces_per_row);
@@ -128,17 +151,14 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
     const int num_topk = a.num_topk;
 
     DEEPEP_PHASE(0);
-    // Lane k fetches selection k's (slot, expert, weight) and works out where its row is: one round
-    // of loads for the whole token instead of one per selection.  The loop below reads the results
-    // back lane by lane, as wave-uniform values.
+    // Lane k works out where selection k's row is; the loop below reads the results back lane by
+    // lane, as wave-uniform values.
     uint64_t my_row = 0;
-    float my_weight = 0.0f;
+    const float my_weight = sel.weight;
     bool my_live = false;
     if (lane < num_topk) {
-        const int64_t idx = int64_t(t) * num_topk + lane;
-        const int slot = a.pair_slot[idx];
-        const int64_t e = a.topk_idx[idx];
-        my_weight = a.topk_weights[idx];
+        const int slot = sel.slot;
+        const int64_t e = sel.expert;
         if (slot >= 0 && slot < a.max_tokens && e >= 0 && e < a.num_experts) {
             const uint8_t* row = a.combine_staging + (e * a.max_tokens + slot) * row_bytes;
             my_live = true;
@@ -207,6 +227,8 @@ __global__ __launch_bounds__(1024) void ll_combine_recv_kernel(CombineRecvArgs a
                                                                const int64_t* layout_range, int rank,
                                                                int num_local_experts, int num_ranks) {
     extern __shared__ int32_t own_begin[];  // [E_l], with own_x only
+    const int64_t item = int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_in_block();
+    const CombineSelection sel = combine_load_selection(a, item);  // in flight while the own ranges are fetched
     if (own_x != nullptr) {
         for (int le = threadIdx.x; le < num_local_experts; le += blockDim.x) {
             const int64_t lr = layout_range[le * num_ranks + rank];
@@ -214,9 +236,8 @@ __global__ __launch_bounds__(1024) void ll_combine_recv_kernel(CombineRecvArgs a
         }
         lds_barrier();
     }
-    combine_recv_piece<kStream>(a, int64_t(blockIdx.x) * (blockDim.x >> 6) + wave_in_block(), own_x,
-                                own_x != nullptr ? own_begin : nullptr, rank * num_local_experts, num_local_experts,
-                                int64_t(a.max_tokens) * num_ranks);
+    combine_recv_piece<kStream>(a, item, sel, own_x, own_x != nullptr ? own_begin : nullptr, rank * num_local_experts,
+                                num_local_experts, int64_t(a.max_tokens) * num_ranks);
 }
 
 // ---------------------------------------------------------------------
@@ -234,14 +255,17 @@ __global__ __launch_bounds__(256) void ll_combine_fused_kernel(CombineSendArgs s
     extern __shared__ int32_t dyn_lds[];  // reduce workgroups: own_begin[E_l]
     const int block = blockIdx.x;
     if (block < num_recv_blocks) {
+        // the token's index loads and the own-range loads go out together: one memory round trip
+        // before the row loads instead of two
+        const int64_t item = int64_t(block) * 4 + wave_in_block();
+        const CombineSelection sel = combine_load_selection(ra, item);
         for (int le = threadIdx.x; le < sa.num_local_experts; le += blockDim.x) {
             const int64_t lr = sa.layout_range[le * sa.num_ranks + sa.rank];
             dyn_lds[le] = (lr & 0xffffffffll) > 0 ? int(lr >> 32) : 0;
         }
         lds_barrier();
-        combine_recv_piece<kStream>(ra, int64_t(block) * 4 + wave_in_block(), sa.x, dyn_lds,
-                                    sa.rank * sa.num_local_experts, sa.num_local_experts,
-                                    int64_t(sa.max_tokens) * sa.num_ranks);
+        combine_recv_piece<kStream>(ra, item, sel, sa.x, dyn_lds, sa.rank * sa.num_local_experts,
+                                    sa.num_local_experts, int64_t(sa.max_tokens) * sa.num_ranks);
     } else {
         combine_send_rows<kStream>(sa, block - num_recv_blocks, int(gridDim.x) - num_recv_blocks, true);
     }
