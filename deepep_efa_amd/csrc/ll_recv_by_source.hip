@@ -11,9 +11,13 @@
 // reference claims that rank with an atomic; here it is the row's arrival order inside its source,
 // so the result does not depend on scheduling.
 //
-// Three launches: pair counts (one workgroup per source), ranges + one {source row, packed row}
-// descriptor per record (one workgroup per source), and the flat row copy the other large-batch
-// paths use.
+// Work is cut into chunks of 512 records that never straddle two sources (the records come grouped
+// by source, ascending).  Large batches, three launches: per-chunk expert histograms (one workgroup
+// per chunk); ranges + one {source row, packed row} descriptor per record (one workgroup per chunk:
+// it adds up the histograms into the (expert, source) counts, scans them into the ranges, and ranks
+// its own 512 rows on top of the histograms of its source's earlier chunks); and the flat row copy
+// the other large-batch paths use.  Small batches, two launches: no histograms, one workgroup per
+// source counts every record's expert itself and walks its source's chunks in order.
 #include "common.hpp"
 #include "segments.hpp"
 #include "../../include/deepep_hip.h"
@@ -57,61 +61,132 @@ __device__ __forceinline__ int record_expert(const uint8_t* __restrict__ recv_by
     return e >= 0 && e < num_local_experts ? e : -1;
 }
 
-// pair_counts[e_l * R + s] = records of source s whose row names local expert e_l.
+constexpr int kBySourceSmallRecords = 4096;  // up to here (record capacity) the two-launch form
+
+// Exclusive prefix over the sources of their chunk counts, ceil(records of the source / 512); chunk g
+// of the launch belongs to the source s with chunk_prefix[s] <= g < chunk_prefix[s + 1].
+__device__ __forceinline__ void source_chunk_prefix(const int32_t* prefix, int num_ranks, int64_t records,
+                                                    int32_t* chunk_prefix, int32_t* scan_tmp) {
+    for (int r = threadIdx.x; r < num_ranks; r += blockDim.x) {
+        int64_t begin = prefix[r], end = prefix[r + 1];
+        if (end > records) end = records;
+        if (begin > end) begin = end;
+        chunk_prefix[r] = int32_t((end - begin + kBySourceThreads - 1) / kBySourceThreads);
+    }
+    lds_barrier();
+    block_exclusive_scan(chunk_prefix, num_ranks, scan_tmp);
+}
+
+// Largest s with table[s] <= v, for an ascending table of n + 1 entries with table[0] <= v < table[n].
+__device__ __forceinline__ int upper_source(const int32_t* table, int n, int64_t v) {
+    int lo = 0, hi = n;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (table[mid] <= v) lo = mid;
+        else hi = mid;
+    }
+    return lo;
+}
+
+// Large batches, first launch: hist[g * E_l + e] = records of chunk g, inside their source's slot,
+// whose row names local expert e.
 __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_count_kernel(
     const uint8_t* __restrict__ recv_by_source, int64_t stride, int64_t tail_off, int64_t buffer_rows, int slot_rows,
     const int32_t* __restrict__ recv_counts, const uint32_t* __restrict__ source_offset,
     const uint32_t* __restrict__ num_recv_tokens, int64_t row_capacity, int num_local_experts, int num_ranks,
-    int32_t* __restrict__ pair_counts) {
-    extern __shared__ int32_t lds[];  // prefix [R + 1] | hist [E_l]
+    int32_t* __restrict__ hist) {
+    extern __shared__ int32_t lds[];  // prefix [R + 1] | chunk_prefix [R + 1] | counts [E_l]
     __shared__ int32_t scan_tmp[kMaxBlockWaves];
     int32_t* prefix = lds;
-    int32_t* hist = lds + num_ranks + 1;
-    const int s = blockIdx.x, tid = threadIdx.x;
+    int32_t* chunk_prefix = prefix + num_ranks + 1;
+    int32_t* counts = chunk_prefix + num_ranks + 1;
+    const int g = blockIdx.x, tid = threadIdx.x;
     source_prefix(recv_counts, num_ranks, prefix, scan_tmp);
-    for (int e = tid; e < num_local_experts; e += kBySourceThreads) hist[e] = 0;
-    lds_barrier();
     int64_t records = num_recv_tokens[1];
     if (records > row_capacity) records = row_capacity;
+    source_chunk_prefix(prefix, num_ranks, records, chunk_prefix, scan_tmp);
+    if (g >= chunk_prefix[num_ranks]) return;
+    for (int e = tid; e < num_local_experts; e += kBySourceThreads) counts[e] = 0;
+    lds_barrier();
+    const int s = upper_source(chunk_prefix, num_ranks, g);
     int64_t begin, end, live_end;
     source_records(prefix, s, num_ranks, slot_rows, records, begin, end, live_end);
-    for (int64_t i = begin + tid; i < live_end; i += kBySourceThreads) {
+    const int64_t i = begin + int64_t(g - chunk_prefix[s]) * kBySourceThreads + tid;
+    if (i < live_end) {
         const int e = record_expert(recv_by_source, stride, tail_off, source_offset[i], buffer_rows, num_local_experts);
-        if (e >= 0) atomicAdd(&hist[e], 1);
+        if (e >= 0) atomicAdd(&counts[e], 1);
     }
     lds_barrier();
-    for (int e = tid; e < num_local_experts; e += kBySourceThreads) pair_counts[e * num_ranks + s] = hist[e];
+    for (int e = tid; e < num_local_experts; e += kBySourceThreads) hist[int64_t(g) * num_local_experts + e] = counts[e];
 }
 
-// Ranges from the pair counts (every workgroup, the first one writes them), then for the records
-// of source blockIdx.x, in arrival order: packed row = range begin + rows of the same pair before it.
+// Ranges from the (expert, source) counts (every workgroup builds them, the first one writes them),
+// then for this workgroup's records, in arrival order: packed row = range begin + rows of the same
+// pair before it.  kChunked: the workgroup is chunk blockIdx.x and the counts come from the chunk
+// histograms; otherwise it is source blockIdx.x, counts the experts of all records itself and walks
+// the source's chunks one after the other.
+template <bool kChunked>
 __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
     const uint8_t* __restrict__ recv_by_source, int64_t stride, int64_t tail_off, int64_t buffer_rows, int slot_rows,
     const int32_t* __restrict__ recv_counts, const uint32_t* __restrict__ source_offset,
     const uint32_t* __restrict__ num_recv_tokens, int64_t row_capacity, int num_local_experts, int num_ranks,
-    int max_tokens, const int32_t* __restrict__ pair_counts, int64_t* __restrict__ layout_range,
+    int max_tokens, const int32_t* __restrict__ hist, int64_t* __restrict__ layout_range,
     int32_t* __restrict__ packed_count, int32_t* __restrict__ stats, uint32_t* __restrict__ tokens_per_expert,
     int32_t* __restrict__ flat_total, RowDesc* __restrict__ desc) {
-    extern __shared__ int32_t lds[];  // prefix [R + 1] | pair_prefix [E_l * R + 1] | running [E_l] | wave_cnt [waves][E_l]
+    // prefix [R + 1] | chunk_prefix [R + 1] | pair_prefix [E_l * R + 1] | running [E_l] | wave_cnt [waves][E_l]
+    extern __shared__ int32_t lds[];
     __shared__ int32_t scan_tmp[kMaxBlockWaves];
     const int num_segments = num_local_experts * num_ranks;
     int32_t* prefix = lds;
-    int32_t* pair_prefix = prefix + num_ranks + 1;
+    int32_t* chunk_prefix = prefix + num_ranks + 1;
+    int32_t* pair_prefix = chunk_prefix + num_ranks + 1;
     int32_t* running = pair_prefix + num_segments + 1;
     int32_t* wave_cnt = running + num_local_experts;
-    const int s = blockIdx.x, tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
+    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
     const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
 
     source_prefix(recv_counts, num_ranks, prefix, scan_tmp);
-    for (int q = tid; q < num_segments; q += kBySourceThreads) {
-        const int c = pair_counts[q];
-        pair_prefix[q] = c < 0 ? 0 : c;
+    int64_t records = num_recv_tokens[1];
+    if (records > row_capacity) records = row_capacity;
+    int s, first_chunk = 0, num_chunks;
+    if constexpr (kChunked) {
+        source_chunk_prefix(prefix, num_ranks, records, chunk_prefix, scan_tmp);
+        const int g = blockIdx.x;
+        if (g >= chunk_prefix[num_ranks] && g != 0) return;  // workgroup 0 writes the ranges even of an empty world
+        // (expert, source) counts: the column sums of the source's chunk histograms
+        for (int q = tid; q < num_segments; q += kBySourceThreads) {
+            const int e = q / num_ranks, src = q - e * num_ranks;
+            int sum = 0;
+            for (int c = chunk_prefix[src]; c < chunk_prefix[src + 1]; ++c) sum += hist[int64_t(c) * num_local_experts + e];
+            pair_prefix[q] = sum;
+        }
+        const bool has_rows = g < chunk_prefix[num_ranks];
+        s = has_rows ? upper_source(chunk_prefix, num_ranks, g) : 0;
+        first_chunk = has_rows ? g - chunk_prefix[s] : 0;
+        num_chunks = has_rows ? 1 : 0;
+        // rows of the same (expert, source) pair in the source's earlier chunks
+        for (int e = tid; e < num_local_experts; e += kBySourceThreads) {
+            int sum = 0;
+            for (int c = chunk_prefix[s]; c < chunk_prefix[s] + first_chunk; ++c) sum += hist[int64_t(c) * num_local_experts + e];
+            running[e] = sum;
+        }
+    } else {
+        s = blockIdx.x;
+        for (int q = tid; q < num_segments; q += kBySourceThreads) pair_prefix[q] = 0;
+        for (int e = tid; e < num_local_experts; e += kBySourceThreads) running[e] = 0;
+        lds_barrier();
+        const int64_t expected = records < prefix[num_ranks] ? records : prefix[num_ranks];
+        for (int64_t i = tid; i < expected; i += kBySourceThreads) {
+            const int src = upper_source(prefix, num_ranks, i);
+            if (i - prefix[src] >= slot_rows) continue;  // past the source's slot
+            const int e = record_expert(recv_by_source, stride, tail_off, source_offset[i], buffer_rows, num_local_experts);
+            if (e >= 0) atomicAdd(&pair_prefix[e * num_ranks + src], 1);
+        }
+        num_chunks = 1 << 30;  // until the source's records end
     }
     lds_barrier();
     block_exclusive_scan(pair_prefix, num_segments, scan_tmp);
-    int64_t records = num_recv_tokens[1];
-    if (records > row_capacity) records = row_capacity;
-    if (s == 0) {
+    if (blockIdx.x == 0) {
         // csrc/kernels/efa_kernels.cu:991-1010: begin = rows of the lower source ranks, 0 where the count is 0
         for (int q = tid; q < num_segments; q += kBySourceThreads) {
             const int le = q / num_ranks;
@@ -127,13 +202,13 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
         }
         if (tid == 0) flat_total[0] = int32_t(records < prefix[num_ranks] ? records : prefix[num_ranks]);
     }
-    for (int e = tid; e < num_local_experts; e += kBySourceThreads) running[e] = 0;
 
     int64_t begin, end, live_end;
     source_records(prefix, s, num_ranks, slot_rows, records, begin, end, live_end);
     int expert_bits = 0;
     while ((1 << expert_bits) < num_local_experts) ++expert_bits;
-    for (int64_t base = begin; base < end; base += kBySourceThreads) {  // batches of rows, in arrival order
+    int64_t base = begin + int64_t(first_chunk) * kBySourceThreads;
+    for (int chunk = 0; chunk < num_chunks && base < end; ++chunk, base += kBySourceThreads) {  // in arrival order
         for (int q = tid; q < kBySourceWaves * num_local_experts; q += kBySourceThreads) wave_cnt[q] = 0;
         lds_barrier();
         const int64_t i = base + tid;
@@ -166,6 +241,7 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
             }
             desc[i] = d;
         }
+        if constexpr (kChunked) break;  // one chunk per workgroup
         lds_barrier();
         for (int e2 = tid; e2 < num_local_experts; e2 += kBySourceThreads) {
             int add = 0;
@@ -182,9 +258,17 @@ using namespace deepep;
 
 extern "C" {
 
+// Workspace: [flat_total | pad] [chunk histograms: at most ceil(capacity / 512) + R chunks of E_l counts] [descriptors]
+static int64_t by_source_head_bytes() { return 256; }
+static int64_t by_source_hist_bytes(int num_experts, int64_t row_capacity) {
+    const int64_t chunks = (row_capacity + kBySourceThreads - 1) / kBySourceThreads + 1;  // E_l * (chunks + R) <= E * chunks
+    return (chunks * num_experts * 4 + 255) & ~int64_t(255);
+}
+
 size_t deepep_ll_by_source_workspace_bytes(int num_experts, int64_t row_capacity) {
-    const int64_t head = ((int64_t(num_experts) + 64) * 4 + 255) & ~int64_t(255);  // pair counts, row total
-    return size_t(head + (row_capacity < 1 ? 1 : row_capacity) * int64_t(sizeof(RowDesc)));
+    const int64_t capacity = row_capacity < 1 ? 1 : row_capacity;
+    return size_t(by_source_head_bytes() + by_source_hist_bytes(num_experts, capacity) +
+                  capacity * int64_t(sizeof(RowDesc)));
 }
 
 int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_rows, const int32_t* recv_counts,
@@ -216,8 +300,8 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_x) & 15) == 0);
     EP_HOST_ASSERT(workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
     EP_HOST_ASSERT(workspace_bytes >= deepep_ll_by_source_workspace_bytes(num_experts, row_capacity));
-    // LDS of the index kernel: prefix, pair prefix, running counts, per-wave counts
-    const size_t index_lds = size_t(num_ranks + 1 + num_experts + 1 + num_local_experts +
+    // LDS of the index kernel: source prefix, chunk prefix, pair prefix, running counts, per-wave counts
+    const size_t index_lds = size_t(2 * (num_ranks + 1) + num_experts + 1 + num_local_experts +
                                     kBySourceWaves * num_local_experts) * sizeof(int32_t);
     EP_HOST_ASSERT(index_lds <= 64 * 1024);
 
@@ -227,22 +311,35 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
     const int64_t scale_bytes = row_scale_bytes(hidden, row_format);
     const int64_t tail_off = align16(data_bytes) + align16(scale_bytes);
     const int64_t buffer_rows = slot_rows * num_ranks;
-    int32_t* pair_counts = reinterpret_cast<int32_t*>(workspace);
-    int32_t* flat_total = pair_counts + num_experts;
-    const int64_t head = ((int64_t(num_experts) + 64) * 4 + 255) & ~int64_t(255);
-    RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) + head);
+    const int64_t capacity = row_capacity < 1 ? 1 : row_capacity;
+    int32_t* flat_total = reinterpret_cast<int32_t*>(workspace);
+    int32_t* hist = reinterpret_cast<int32_t*>(reinterpret_cast<uint8_t*>(workspace) + by_source_head_bytes());
+    RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) + by_source_head_bytes() +
+                                               by_source_hist_bytes(num_experts, capacity));
+    const uint8_t* rows_in = reinterpret_cast<const uint8_t*>(recv_by_source);
 
-    const size_t count_lds = size_t(num_ranks + 1 + num_local_experts) * sizeof(int32_t);
-    ll_by_source_count_kernel<<<num_ranks, kBySourceThreads, count_lds, hs>>>(
-        reinterpret_cast<const uint8_t*>(recv_by_source), stride, tail_off, buffer_rows, int(slot_rows), recv_counts,
-        source_offset, num_recv_tokens, row_capacity, num_local_experts, num_ranks, pair_counts);
-    EP_LAUNCH_CHECK();
-    ll_by_source_index_kernel<<<num_ranks, kBySourceThreads, index_lds, hs>>>(
-        reinterpret_cast<const uint8_t*>(recv_by_source), stride, tail_off, buffer_rows, int(slot_rows), recv_counts,
-        source_offset, num_recv_tokens, row_capacity, num_local_experts, num_ranks, num_max_dispatch_tokens_per_rank,
-        pair_counts, packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, tokens_per_expert,
-        flat_total, desc);
-    EP_LAUNCH_CHECK();
+    if (row_capacity <= kBySourceSmallRecords) {
+        ll_by_source_index_kernel<false><<<num_ranks, kBySourceThreads, index_lds, hs>>>(
+            rows_in, stride, tail_off, buffer_rows, int(slot_rows), recv_counts, source_offset, num_recv_tokens,
+            row_capacity, num_local_experts, num_ranks, num_max_dispatch_tokens_per_rank, nullptr,
+            packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, tokens_per_expert,
+            flat_total, desc);
+        EP_LAUNCH_CHECK();
+    } else {
+        // every source's records round up to whole chunks: at most ceil(capacity / 512) + R of them
+        const int64_t chunks = (row_capacity + kBySourceThreads - 1) / kBySourceThreads + num_ranks;
+        const size_t count_lds = size_t(2 * (num_ranks + 1) + num_local_experts) * sizeof(int32_t);
+        ll_by_source_count_kernel<<<unsigned(chunks), kBySourceThreads, count_lds, hs>>>(
+            rows_in, stride, tail_off, buffer_rows, int(slot_rows), recv_counts, source_offset, num_recv_tokens,
+            row_capacity, num_local_experts, num_ranks, hist);
+        EP_LAUNCH_CHECK();
+        ll_by_source_index_kernel<true><<<unsigned(chunks), kBySourceThreads, index_lds, hs>>>(
+            rows_in, stride, tail_off, buffer_rows, int(slot_rows), recv_counts, source_offset, num_recv_tokens,
+            row_capacity, num_local_experts, num_ranks, num_max_dispatch_tokens_per_rank, hist,
+            packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, tokens_per_expert,
+            flat_total, desc);
+        EP_LAUNCH_CHECK();
+    }
     if (row_capacity == 0) return 0;
     const int num_vec = int(data_bytes / 16);
     int threads = ((num_vec + 63) / 64) * 64;
@@ -252,7 +349,7 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
     if (blocks > 16384) blocks = blocks / 2 > 16384 ? blocks / 2 : 16384;
     if (blocks > (int64_t(1) << 22)) blocks = int64_t(1) << 22;
     ll_rows_flat_kernel<<<unsigned(blocks), threads + extra, 0, hs>>>(
-        flat_total, 0, desc, reinterpret_cast<const uint8_t*>(recv_by_source), stride, num_vec,
+        flat_total, 0, desc, rows_in, stride, num_vec,
         reinterpret_cast<uint8_t*>(packed_recv_x), nullptr, data_bytes, int(scale_bytes / 4), align16(data_bytes),
         scale_bytes > 0 ? reinterpret_cast<uint8_t*>(packed_recv_scales) : nullptr, tail_off, packed_recv_src_info,
         extra);

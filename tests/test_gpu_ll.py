@@ -290,7 +290,9 @@ def recv_by_source_on_gpu(rt, buf, routed, rank, e, m, h, fmt, slot_rows, capaci
 @pytest.mark.parametrize("r,rank,t,h,k,e", [
     (4, 1, 8, 512, 3, 16), (8, 7, 33, 1024, 4, 64), (2, 0, 1, 512, 1, 2),
     (32, 5, 128, 7168, 8, 256),   # the headline shape
-    (8, 3, 700, 512, 8, 256),     # sources with more rows than one batch of the index kernel: running counts
+    (8, 3, 700, 512, 8, 256),     # past 4096 records: chunk histograms, sources of two chunks each
+    (4, 1, 900, 512, 4, 16),      # up to 4096 records: one workgroup per source walks its two chunks, running counts
+    (16, 2, 1200, 512, 8, 64),    # 9600 records in chunks of 512, about 600 per source
     (1, 0, 16, 512, 2, 4),        # a world of one rank
     (4, 2, 64, 512, 2, 4),        # one expert per rank
     (2, 1, 40, 512, 6, 2048),     # 1024 local experts: ten bits of expert id
