@@ -267,7 +267,7 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
     p = int((st.pair_slot[:t] >= 0).sum())
     rv = int(st.packed_recv_count.sum())
     own = int((st.packed_recv_layout_range[:, rank] & 0xFFFFFFFF).sum())
-    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r, own)
+    nbytes = algorithmic_bytes(t, h, k, p, rv, st.payload_bytes, e, r, own)
     calls = {
         "dispatch_send": lambda: st.dispatch_send(x, topk),
         "dispatch_recv": lambda: st.dispatch_recv(),
@@ -609,7 +609,7 @@ def main():
     us_per_step = graph_us if graph_us is not None else eager_us
     us_per_phase_step = graph_phase_us if graph_phase_us is not None else eager_phase_us
 
-    nbytes = algorithmic_bytes(t, h, k, p, rv, st.stride, e, r, own, packed=st.data_bytes + st.scale_bytes + 4)
+    nbytes = algorithmic_bytes(t, h, k, p, rv, st.payload_bytes, e, r, own, packed=st.data_bytes + st.scale_bytes + 4)
     kernels = {n: {"us": round(per_call[n], 2), "bytes": nbytes[n],
                    "GBps": round(nbytes[n] / per_call[n] / 1e3, 1)} for n in calls}
     dom = max(step_calls, key=per_call.get)

@@ -19,6 +19,7 @@ PROTOTYPES = {
     "deepep_ll_row_data_bytes": (_SZ, [_I, _I]),
     "deepep_ll_row_scale_bytes": (_SZ, [_I, _I]),
     "deepep_ll_row_stride": (_SZ, [_I, _I]),
+    "deepep_ll_row_payload_bytes": (_SZ, [_I, _I]),
     "deepep_get_low_latency_rdma_size_hint": (_SZ, [_I, _I, _I, _I]),
     "deepep_layout_workspace_bytes": (_SZ, [_I, _I, _I]),
     "deepep_get_dispatch_layout": (_I, [_VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),

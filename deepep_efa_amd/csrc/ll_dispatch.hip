@@ -812,6 +812,7 @@ extern "C" {
 size_t deepep_ll_row_data_bytes(int hidden, int row_format) { return size_t(row_data_bytes(hidden, row_format)); }
 size_t deepep_ll_row_scale_bytes(int hidden, int row_format) { return size_t(row_scale_bytes(hidden, row_format)); }
 size_t deepep_ll_row_stride(int hidden, int row_format) { return size_t(row_stride_bytes(hidden, row_format)); }
+size_t deepep_ll_row_payload_bytes(int hidden, int row_format) { return size_t(row_payload_bytes(hidden, row_format)); }
 
 size_t deepep_ll_segment_workspace_bytes(int num_experts, int num_max_dispatch_tokens_per_rank) {
     return size_t(segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank));

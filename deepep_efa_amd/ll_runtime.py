@@ -58,6 +58,7 @@ class LowLatencyState:
         assert s.num_experts % s.num_ranks == 0 and 0 <= s.rank < s.num_ranks
         assert s.hidden % 128 == 0
         self.stride = lib.deepep_ll_row_stride(s.hidden, s.fmt)
+        self.payload_bytes = lib.deepep_ll_row_payload_bytes(s.hidden, s.fmt)  # what a staged row carries
         self.data_bytes = lib.deepep_ll_row_data_bytes(s.hidden, s.fmt)
         self.scale_bytes = lib.deepep_ll_row_scale_bytes(s.hidden, s.fmt)
         el, r, m, e, h = s.num_local_experts, s.num_ranks, s.max_tokens, s.num_experts, s.hidden

@@ -61,10 +61,13 @@ enum {
 size_t deepep_ll_row_data_bytes(int hidden, int row_format);
 /* Bytes of the scale part of a row (0 for bf16). */
 size_t deepep_ll_row_scale_bytes(int hidden, int row_format);
-/* Stride of one staged row: data and scales each padded to 16 B, plus a
+/* Payload of one staged row: data and scales each padded to 16 B, plus a
  * 16 B tail {int32 src_token, int32 topk_slot, int32 src_rank, int32 local expert}.
- * 7408 for fp8 at H = 7168 — the value the reference's cooperative send
- * uses (csrc/kernels/coop_dispatch_send.cu:73-75). */
+ * 7408 for fp8 at H = 7168 — the stride of the reference's cooperative send
+ * (csrc/kernels/coop_dispatch_send.cu:73-75). */
+size_t deepep_ll_row_payload_bytes(int hidden, int row_format);
+/* Distance between staged rows: the payload rounded up to whole 128-byte cache
+ * lines (7424 for fp8 at H = 7168); the bytes behind the tail are never written. */
 size_t deepep_ll_row_stride(int hidden, int row_format);
 
 /* Arithmetic of the reference's buffer sizing, kept for API parity.

@@ -56,7 +56,8 @@ class CpuRankStep:
             rows = self.staged[le, sr, :c]
             self.px[le, b:b + c] = rows[:, :h]
             self.ps[le, b:b + c] = rows[:, h:h + h // 32]
-            self.src_info[le, b:b + c] = rows[:, -16:-12].contiguous().view(torch.int32).view(-1)
+            tail = O.row_payload(h, O.ROW_FP8) - 16
+            self.src_info[le, b:b + c] = rows[:, tail:tail + 4].contiguous().view(torch.int32).view(-1)
         # ---- combine send (own pairs only come back locally; peers' rows are already staged)
         for le in range(epr):
             c, b = int(cnt[le, self.rank]), int(begin[le, self.rank])

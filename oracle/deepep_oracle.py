@@ -88,9 +88,15 @@ def row_scale_bytes(hidden: int, fmt: int) -> int:
     return g if fmt == ROW_FP8_UE8M0 else 4 * g
 
 
-def row_stride(hidden: int, fmt: int) -> int:
+def row_payload(hidden: int, fmt: int) -> int:
     """data and scales padded to 16 B + 16 B tail (csrc/kernels/coop_dispatch_send.cu:73-75)."""
     return align_up(row_data_bytes(hidden, fmt), 16) + align_up(row_scale_bytes(hidden, fmt), 16) + 16
+
+
+def row_stride(hidden: int, fmt: int) -> int:
+    """Distance between staged rows: the payload rounded up to whole 128-byte cache lines (this build's
+    choice; the bytes behind the tail are never written)."""
+    return align_up(row_payload(hidden, fmt), 128)
 
 
 # ----------------------------------------------------------------------------
@@ -413,7 +419,7 @@ def staged_rows(x: torch.Tensor, topk_idx: torch.Tensor, src_rank: int, num_expe
     hidden = x.shape[1]
     db, sb = row_data_bytes(hidden, fmt), row_scale_bytes(hidden, fmt)
     dp, sp = align_up(db, 16), align_up(sb, 16)
-    stride = dp + sp + 16
+    stride = row_stride(hidden, fmt)
     send_count, pair_slot = route(topk_idx, num_experts, max_tokens)
     data, scales = quantise_rows(x, fmt)
     tok, kk = torch.nonzero(pair_slot >= 0, as_tuple=True)
@@ -425,7 +431,7 @@ def staged_rows(x: torch.Tensor, topk_idx: torch.Tensor, src_rank: int, num_expe
     local = (topk_idx[tok, kk] % experts_per_rank).to(torch.int32)
     tail = torch.stack([tok.to(torch.int32), kk.to(torch.int32), torch.full_like(tok, src_rank, dtype=torch.int32),
                         local], 1).contiguous()
-    rows[:, dp + sp:] = tail.view(torch.uint8).view(-1, 16)
+    rows[:, dp + sp:dp + sp + 16] = tail.view(torch.uint8).view(-1, 16)
     experts = topk_idx[tok, kk]
     slots = pair_slot[tok, kk].to(torch.int64)
     return send_count, pair_slot, experts, slots, rows

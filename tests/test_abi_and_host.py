@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in include/deepep_hip.h but not exported"
         assert name in _capi.PROTOTYPES, f"{name} has no ctypes prototype"
     assert sorted(_capi.PROTOTYPES) == declared
-    assert lib.deepep_abi_version() == 8
+    assert lib.deepep_abi_version() == 9
 
 
 @pytest.mark.parametrize("hidden", [128, 512, 2048, 7168])

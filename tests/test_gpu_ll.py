@@ -329,7 +329,8 @@ def test_dispatch_recv_by_source_drops_what_does_not_fit(rt):
         # expected: walk the records the way the kernel may use them
         epr, n = e // r, 0
         want_rows = [[[] for _ in range(r)] for _ in range(epr)]
-        tail = buf[:, -16:].contiguous().view(torch.int32)
+        tail_at = O.row_payload(h, fmt) - 16
+        tail = buf[:, tail_at:tail_at + 16].contiguous().view(torch.int32)
         for s in range(r):
             for j in range(recv_counts[s]):
                 if n < capacity and j < slot_rows:
@@ -422,14 +423,18 @@ def test_dispatch_send_staging_and_send_slots(rt):
     epr = e // r
     touched_stage = torch.zeros((epr, r, m), dtype=torch.bool)
     touched_send = torch.zeros((e, m), dtype=torch.bool)
+    payload = O.row_payload(h, O.ROW_FP8)
+    assert stride == O.row_stride(h, O.ROW_FP8) == 640 and payload == 544  # a row takes whole 128-byte lines
     for i in range(rows.shape[0]):
         ex, sl = int(experts[i]), int(slots[i])
         if ex // epr == rank:
-            assert torch.equal(staging[ex % epr, rank, sl], rows[i])
+            got, fill = staging[ex % epr, rank, sl], 0xAB
             touched_stage[ex % epr, rank, sl] = True
         else:
-            assert torch.equal(sendbuf[ex, sl], rows[i])
+            got, fill = sendbuf[ex, sl], 0xCD
             touched_send[ex, sl] = True
+        assert torch.equal(got[:payload], rows[i, :payload])
+        assert (got[payload:] == fill).all()  # nothing is written behind the tail
     assert (staging[~touched_stage] == 0xAB).all() and (sendbuf[~touched_send] == 0xCD).all()
     rc = st.recv_count.cpu().view(epr, r)
     assert torch.equal(rc[:, rank], send_count[rank * epr:(rank + 1) * epr])

@@ -285,8 +285,10 @@ def test_route_slots_and_staged_rows():
             seen[e] = seen.get(e, 0) + 1
     assert send_count.tolist() == [seen.get(e, 0) for e in range(8)]
     sc, ps, experts, slots, rows = O.staged_rows(xs[0], tk[0], 1, 8, 10, O.ROW_FP8, num_ranks=2)
-    assert rows.shape[1] == O.row_stride(256, O.ROW_FP8) == 256 + 16 + 16
-    tail = rows[:, -16:].contiguous().view(torch.int32)
+    assert O.row_payload(256, O.ROW_FP8) == 256 + 16 + 16
+    assert rows.shape[1] == O.row_stride(256, O.ROW_FP8) == 384  # whole 128-byte lines
+    assert (rows[:, 288:] == 0).all()
+    tail = rows[:, 272:288].contiguous().view(torch.int32)
     assert (tail[:, 2] == 1).all() and torch.equal(tail[:, 3].long(), experts % 4)  # 8 experts on 2 ranks
     q, s = O.per_token_cast_to_fp8(xs[0])
     assert torch.equal(rows[:, :256], q.view(torch.uint8)[tail[:, 0].long()])
@@ -331,8 +333,11 @@ def test_size_hint_hand_values():
     # tiny case by hand: M=1,H=128,E=2: dmsg=16+256=272, cmsg=4+256=260; send=max(272,520)=520; recv=max(544,520)=544
     # sig=128 -> total = 1040+1088+256 = 2384 -> (2384+128)//128*128 = 2432
     assert O.get_low_latency_rdma_size_hint(1, 128, 2, 2) == 2432
-    assert O.row_stride(7168, O.ROW_FP8) == 7408 and O.row_stride(7168, O.ROW_BF16) == 14352
-    assert O.row_stride(7168, O.ROW_FP8_UE8M0) == 7168 + 64 + 16
+    # the reference's cooperative send stride (csrc/kernels/coop_dispatch_send.cu:73-75) is this build's row payload
+    assert O.row_payload(7168, O.ROW_FP8) == 7408 and O.row_payload(7168, O.ROW_BF16) == 14352
+    assert O.row_payload(7168, O.ROW_FP8_UE8M0) == 7168 + 64 + 16
+    assert O.row_stride(7168, O.ROW_FP8) == 7424 and O.row_stride(7168, O.ROW_BF16) == 14464
+    assert O.row_stride(7168, O.ROW_FP8_UE8M0) == 7296 and O.row_stride(512, O.ROW_FP8) == 640
 
 
 # --------------------------------------------------------------------------
