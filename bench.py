@@ -63,6 +63,18 @@ def time_calls(torch, fn, n):
     return e0.elapsed_time(e1) * 1e3 / n
 
 
+def rotating(fns):
+    """One callable that runs the given callables in turn.  Each works on its own set of buffers, so that a call
+    finds none of its bytes in the 256 MB memory-side cache where the call before left them: calls on one set
+    of buffers, back to back, measure that cache and not HBM unless a single call moves far more than it holds."""
+    turn = [0]
+
+    def call():
+        turn[0] = (turn[0] + 1) % len(fns)
+        fns[turn[0]]()
+    return call
+
+
 def calibrate_copy(torch, _capi, lib):
     """A plain copy through the pack kernel with identity row ids: 32768 rows x 14336 B read and written once.
     Under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` the counters of pack_rows_kernel divided into the
@@ -179,23 +191,37 @@ def bench_pack(torch, _capi, lib, loopback, args):
     torch.cuda.synchronize()
     s = int(cumsum[r])
     total_dev = cumsum[r:]
-    q = torch.empty((t, h), dtype=torch.uint8, device="cuda")
-    sc = torch.empty((t, h // 128), dtype=torch.float32, device="cuda")
-    _capi.check(lib.deepep_per_token_cast_to_fp8(_capi.ptr(x), t, h, 1, _capi.ptr(q), _capi.ptr(sc), stream))
-    out16 = torch.empty((s, h), dtype=torch.bfloat16, device="cuda")
-    out8 = torch.empty((s, h), dtype=torch.uint8, device="cuda")
-    outs = torch.empty((s, h // 128), dtype=torch.float32, device="cuda")
+    # The HBM-bound entries rotate over several sets of buffers (see `rotating`): seven for the cast (89 MB a
+    # call), two for the packs and the reduce (321 to 622 MB a call).
+    sets = 7
+    xs = [x] + [x.clone() for _ in range(sets - 1)]
+    qs = [torch.empty((t, h), dtype=torch.uint8, device="cuda") for _ in range(sets)]
+    scs = [torch.empty((t, h // 128), dtype=torch.float32, device="cuda") for _ in range(sets)]
+    q, sc = qs[0], scs[0]
+    for i in range(sets):
+        _capi.check(lib.deepep_per_token_cast_to_fp8(_capi.ptr(xs[i]), t, h, 1, _capi.ptr(qs[i]), _capi.ptr(scs[i]),
+                                                     stream))
+    out16s = [torch.empty((s, h), dtype=torch.bfloat16, device="cuda") for _ in range(2)]
+    out8s = [torch.empty((s, h), dtype=torch.uint8, device="cuda") for _ in range(2)]
+    outss = [torch.empty((s, h // 128), dtype=torch.float32, device="cuda") for _ in range(2)]
+    out16 = out16s[0]
 
-    def pack_bf16():
-        _capi.check(lib.deepep_pack_rows(_capi.ptr(x), None, _capi.ptr(ids), _capi.ptr(total_dev), s, t, 2 * h, 0,
-                                         _capi.ptr(out16), None, stream))
+    def pack_bf16_on(i):
+        return lambda: _capi.check(lib.deepep_pack_rows(_capi.ptr(xs[i]), None, _capi.ptr(ids), _capi.ptr(total_dev), s,
+                                                        t, 2 * h, 0, _capi.ptr(out16s[i]), None, stream))
 
-    def pack_fp8():
-        _capi.check(lib.deepep_pack_rows(_capi.ptr(q), _capi.ptr(sc), _capi.ptr(ids), _capi.ptr(total_dev), s, t, h,
-                                         h // 32, _capi.ptr(out8), _capi.ptr(outs), stream))
+    def pack_fp8_on(i):
+        return lambda: _capi.check(lib.deepep_pack_rows(_capi.ptr(qs[i]), _capi.ptr(scs[i]), _capi.ptr(ids),
+                                                        _capi.ptr(total_dev), s, t, h, h // 32, _capi.ptr(out8s[i]),
+                                                        _capi.ptr(outss[i]), stream))
 
-    def cast():
-        _capi.check(lib.deepep_per_token_cast_to_fp8(_capi.ptr(x), t, h, 1, _capi.ptr(q), _capi.ptr(sc), stream))
+    def cast_on(i):
+        return lambda: _capi.check(lib.deepep_per_token_cast_to_fp8(_capi.ptr(xs[i]), t, h, 1, _capi.ptr(qs[i]),
+                                                                    _capi.ptr(scs[i]), stream))
+
+    pack_bf16 = rotating([pack_bf16_on(i) for i in range(2)])
+    pack_fp8 = rotating([pack_fp8_on(i) for i in range(2)])
+    cast = rotating([cast_on(i) for i in range(sets)])
 
     # the steps either side of the pack: top-k remap of the send rows, source metadata of the rows
     # received (here: as many as were sent), and the per-token reduce of the rows that come back
@@ -204,10 +230,10 @@ def bench_pack(torch, _capi, lib, loopback, args):
     remap_e = torch.empty((s, k), dtype=torch.int64, device="cuda")
     remap_w = torch.empty((s, k), dtype=torch.float32, device="cuda")
     meta = torch.empty((s, 8), dtype=torch.uint8, device="cuda")
-    comb_x = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    comb_xs = [torch.empty((t, h), dtype=torch.bfloat16, device="cuda") for _ in range(2)]
     comb_w = torch.empty((t, k), dtype=torch.float32, device="cuda")
     ws3 = torch.empty(max(256, lib.deepep_combine_reduce_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
-    pack_bf16()
+    pack_bf16(), pack_bf16()
 
     def remap():
         _capi.check(lib.deepep_topk_remap(_capi.ptr(topk), _capi.ptr(weights), _capi.ptr(ids), _capi.ptr(cumsum), t, k, r,
@@ -218,13 +244,17 @@ def bench_pack(torch, _capi, lib, loopback, args):
 
     remap()
 
-    def reduce():
-        _capi.check(lib.deepep_combine_reduce(_capi.ptr(out16), _capi.ptr(remap_w), _capi.ptr(ids), _capi.ptr(cumsum),
-                                              _capi.ptr(is_in), None, None, t, h, k, r, s, _capi.ptr(comb_x),
-                                              _capi.ptr(comb_w), _capi.ptr(ws3), ws3.numel(), stream))
+    def reduce_on(i):
+        return lambda: _capi.check(lib.deepep_combine_reduce(
+            _capi.ptr(out16s[i]), _capi.ptr(remap_w), _capi.ptr(ids), _capi.ptr(cumsum), _capi.ptr(is_in), None, None,
+            t, h, k, r, s, _capi.ptr(comb_xs[i]), _capi.ptr(comb_w), _capi.ptr(ws3), ws3.numel(), stream))
+
+    reduce = rotating([reduce_on(i) for i in range(2)])
 
     n = max(10, args.steps // 4)
-    res = {"workload": "4096 tokens x 7168 bf16, top-8 of 256 experts, 8 ranks x 32 experts", "rows_packed": s}
+    res = {"workload": "4096 tokens x 7168 bf16, top-8 of 256 experts, 8 ranks x 32 experts", "rows_packed": s,
+           "buffers": "cast, packs and reduce rotate over 7 / 2 / 2 sets of buffers, so no call finds its bytes in "
+                      "the memory-side cache"}
     for name, fn, nbytes in (("layout", layout, t * k * 8 + t * r + 4 * (r + e)),
                              ("routing_sort", sort, 2 * t * r + s * 8),
                              ("channel_prefix", prefix, t * r + r * 10 * 4),
@@ -259,29 +289,39 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
     y = torch.empty((epr, n_slots, h), dtype=torch.bfloat16, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
     _capi.check(lib.deepep_synth_bf16_rows(_capi.ptr(y), epr * n_slots, h, h * 2, None, 0, 5, 0, stream))
-    st.dispatch_send(x, topk)
-    world.dispatch_from_peers(st)
-    st.dispatch_recv()
-    world.combine_from_peers(st, mode=1, seed=9)
+    # 4096 tokens: two sets of buffers taken in turn (see `rotating`; a send moves 302 MB, little more than the
+    # memory-side cache holds).  The skewed size moves gigabytes per call and keeps one set.
+    states = [st] if skewed else [st, ll_runtime.LowLatencyState(shape)]
+    xs = [x] + [x.clone() for _ in states[1:]]
+    for s_, x_ in zip(states, xs):
+        s_.dispatch_send(x_, topk)
+        world.dispatch_from_peers(s_)
+        s_.dispatch_recv()
+        world.combine_from_peers(s_, mode=1, seed=9)
     torch.cuda.synchronize()
     p = int((st.pair_slot[:t] >= 0).sum())
     rv = int(st.packed_recv_count.sum())
     own = int((st.packed_recv_layout_range[:, rank] & 0xFFFFFFFF).sum())
     nbytes = algorithmic_bytes(t, h, k, p, rv, st.payload_bytes, e, r, own)
+    def on_every_state(make):
+        return rotating([make(s_, x_) for s_, x_ in zip(states, xs)])
+
     calls = {
-        "dispatch_send": lambda: st.dispatch_send(x, topk),
-        "dispatch_recv": lambda: st.dispatch_recv(),
-        "combine_send": lambda: st.combine_send(y),
-        "combine_recv": lambda: st.combine_recv(topk, weights, out),
+        "dispatch_send": on_every_state(lambda s_, x_: lambda: s_.dispatch_send(x_, topk)),
+        "dispatch_recv": on_every_state(lambda s_, x_: lambda: s_.dispatch_recv()),
+        "combine_send": on_every_state(lambda s_, x_: lambda: s_.combine_send(y)),
+        "combine_recv": on_every_state(lambda s_, x_: lambda: s_.combine_recv(topk, weights, out)),
         # the one-call entries (what deep_ep.Buffer launches): the rank's own rows are written / read in place
-        "dispatch": lambda: st.dispatch(x, topk),
-        "combine": lambda: st.combine(y, topk, weights, out),
+        "dispatch": on_every_state(lambda s_, x_: lambda: s_.dispatch(x_, topk)),
+        "combine": on_every_state(lambda s_, x_: lambda: s_.combine(y, topk, weights, out)),
     }
     if not skewed:  # the receive side fed by a source-grouped transport (same bytes as dispatch_recv)
-        calls["dispatch_recv_by_source"], _ = by_source_receive(torch, _capi, lib, ll_runtime, st, world)
+        calls["dispatch_recv_by_source"] = on_every_state(
+            lambda s_, x_: by_source_receive(torch, _capi, lib, ll_runtime, s_, world)[0])
     res = {"workload": f"LL dispatch+combine at {t} tokens x {h}, top-{k} of {e} experts, {r} ranks x {epr} experts"
                        + (", Zipf(1.2) expert popularity, 1 % outlier rows" if skewed else ""),
-           "pairs_sent": p, "rows_received": rv, "rows_to_own_experts": own}
+           "pairs_sent": p, "rows_received": rv, "rows_to_own_experts": own,
+           "buffers": "one set" if skewed else "two sets taken in turn, so no call finds its bytes in the memory-side cache"}
     for name, fn in calls.items():
         if skewed:  # millisecond kernels: every call between its own events, so the spread shows
             samples = sorted(time_calls(torch, fn, 1) for _ in range(6))
@@ -292,6 +332,30 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
                      "frac_of_8TBps": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBS, 4)}
         if skewed:
             res[name]["us_min_max"] = [round(samples[0], 2), round(samples[-1], 2)]
+    if not skewed:  # what the same send measures when every call goes to the same buffers
+        us = time_calls(torch, lambda: st.dispatch_send(x, topk), max(10, args.steps // 10))
+        res["dispatch_send"]["us_on_one_set_of_buffers"] = round(us, 2)
+    # The send's memory traffic without the send: a bare kernel that reads every token row and stores one
+    # byte per element to the rows the send writes (remote experts' slots; the rows for this rank's own
+    # experts go to the same buffer at the expert's slots too).  What it reaches is what this access
+    # pattern gets from HBM on this GPU.
+    slot = st.pair_slot[:t].long()
+    dst_rows = torch.where(slot >= 0, topk.clamp(min=0) * st.shape.max_tokens + slot, torch.full_like(slot, -1))
+    dst_rows = dst_rows.to(torch.int32).contiguous()
+    probe = on_every_state(lambda s_, x_: lambda: _capi.check(lib.deepep_probe_row_scatter(
+        _capi.ptr(x_), t, h, _capi.ptr(dst_rows), k, _capi.ptr(s_.send_slots), s_.stride, stream)))
+    if skewed:
+        samples = sorted(time_calls(torch, probe, 1) for _ in range(6))
+        us = samples[len(samples) // 2]
+    else:
+        us = time_calls(torch, probe, max(10, args.steps // 10))
+    probe_bytes = t * 2 * h + p * h
+    res["bare_row_scatter"] = {"us": round(us, 2), "bytes": probe_bytes, "GBps": round(probe_bytes / us / 1e3, 1),
+                               "frac_of_8TBps": round(probe_bytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                               "what": "reads the token rows and stores hidden bytes to each row the send writes: "
+                                       "the send's traffic pattern without routing, quantisation or scales"}
+    res["dispatch_send"]["us_per_byte_against_bare_row_scatter"] = round(
+        (res["dispatch_send"]["us"] / nbytes["dispatch_send"]) / (us / probe_bytes), 3)
     return res
 
 

@@ -50,6 +50,7 @@ PROTOTYPES = {
     "deepep_combine_reduce": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP, _SZ, _VP]),
     "deepep_synth_topk_idx": (_I, [_VP, _VP, _I, _I, _I, _I, _U32, _VP, _VP]),
     "deepep_synth_bf16_rows": (_I, [_VP, _I64, _I, _I64, _VP, _U32, _U32, _I, _VP]),
+    "deepep_probe_row_scatter": (_I, [_VP, _I, _I, _VP, _I, _VP, _I64, _VP]),
     "deepep_loopback_dispatch_from_peers": (_I, [_VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _SZ,
                                                _VP]),
     "deepep_loopback_combine_from_peers": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _U32, _VP, _VP]),

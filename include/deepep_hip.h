@@ -478,6 +478,16 @@ int deepep_loopback_dispatch_from_peers(const void* x, const int64_t* topk_idx,
                                         void* recv_staging, int32_t* recv_count,
                                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* A measuring stick, not part of the path (no counterpart in the reference): reads T rows of
+ * 2 * hidden bytes and writes, for every token, `hidden` bytes (the two halves of each 32 bytes
+ * folded together) to each of its K destination rows — the memory traffic of the dispatch send side
+ * at one byte per element, with no routing, quantisation or scales.  bench.py times it beside the
+ * send kernel on the same destinations: what it reaches is what this access pattern gets from HBM.
+ *   x         [T, hidden] 2-byte elements       dst_rows  [T, K] int32 row index, -1 = none
+ *   dst       rows of dst_stride_bytes, the first `hidden` bytes of each named row written */
+int deepep_probe_row_scatter(const void* x, int num_tokens, int hidden, const int32_t* dst_rows, int num_topk,
+                             void* dst, int64_t dst_stride_bytes, void* stream);
+
 /* Plays the remote experts for this rank's own pairs: for every remote
  * expert e and slot j < send_count[e] writes combine_staging[e, j, :].
  *   mode 0: the dequantised send_slots row (f32(q) * scale -> bf16), i.e. an

@@ -364,3 +364,27 @@ def test_normal_mode_steps_through_the_host_module():
     assert torch.equal(cx.cpu().view(torch.int16), chain_x.view(torch.int16))
     with pytest.raises(RuntimeError, match="Assertion"):
         normal.topk_remap(topk.cuda(), w.cuda(), ids_d, cumsum_d, total_d + 10 ** 6, r, e // r)
+
+
+def test_row_scatter_probe(capi):
+    """The bare read-rows / store-K-copies kernel bench.py times beside the send side: every named row gets
+    the fold of its token's row, every other byte is left alone."""
+    lib = capi.load()
+    t, h, k, rows, stride = 37, 512, 3, 200, 640
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(0, 2 ** 16, (t, h), generator=g, dtype=torch.int32).to(torch.uint16)
+    dst_rows = torch.randperm(rows, generator=g)[:t * k].view(t, k).to(torch.int32)
+    dst_rows[::5, 1] = -1
+    dst = torch.full((rows, stride), 0xEE, dtype=torch.uint8, device="cuda")
+    x_dev, rows_dev = x.cuda(), dst_rows.cuda()
+    capi.check(lib.deepep_probe_row_scatter(capi.ptr(x_dev), t, h, capi.ptr(rows_dev), k, capi.ptr(dst), stride,
+                                            stream()))
+    torch.cuda.synchronize()
+    words = x.view(torch.uint8).view(t, h // 16, 2, 16)          # 32 bytes per thread: two 16-byte vectors
+    fold = (words[:, :, 0] ^ words[:, :, 1]).reshape(t, h)       # one vector out
+    want = torch.full((rows, stride), 0xEE, dtype=torch.uint8)
+    for i in range(t):
+        for j in range(k):
+            if dst_rows[i, j] >= 0:
+                want[int(dst_rows[i, j]), :h] = fold[i]
+    assert torch.equal(dst.cpu(), want)
