@@ -161,7 +161,7 @@ __global__ __launch_bounds__(1024) void row_scatter_probe_kernel(const uint8_t* 
     }
     for (int k = 0; k < num_topk; ++k) {
         const int row = dst_rows[int64_t(t) * num_topk + k];
-        if (row >= 0 && tid < vecs) *reinterpret_cast<u32x4*>(dst + int64_t(row) * dst_stride + int64_t(tid) * 16) = v;
+        if (row >= 0 && tid < vecs) store_u32x4<true>(dst + int64_t(row) * dst_stride + int64_t(tid) * 16, v);  // streaming
     }
 }
 
