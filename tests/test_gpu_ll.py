@@ -855,3 +855,27 @@ def test_tokens_naming_an_expert_more_than_once(rt, fmt, one_call):
     back = x_all[rank] if fmt == O.ROW_BF16 else O.per_token_cast_back(*O.per_token_cast_to_fp8(x_all[rank]))
     chain = O.ll_combine_f32_chain(back.unsqueeze(1).expand(-1, k, -1).contiguous(), w_all[rank], live)
     assert torch.equal(out.cpu().view(torch.int16), chain.view(torch.int16))
+
+
+@ONE_CALL
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
+def test_send_past_the_streaming_bound(rt, one_call, fmt):
+    """2800 tokens x 7168, top-8: the send moves more than 192 MB, so its payload stores carry the
+    non-temporal hint (a different kernel instantiation); every output must be what the oracle says."""
+    r, rank, t, h, k, e = 2, 1, 2800, 7168, 8, 16
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=2800, drop=10)
+    assert t * (2 * h + k * O.row_payload(h, fmt)) > 192 * 2 ** 20
+    st, _ = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt, one_call=one_call)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
+    check_dispatch(st, want, fmt)
+    send_count, pair_slot = O.route(topk_all[rank], e, t)
+    assert torch.equal(st.send_count.cpu(), send_count)
+    assert torch.equal(st.pair_slot.cpu(), pair_slot)
+    # the rows for the other rank's experts, byte for byte, on a sample of pairs
+    _, _, experts, slots, rows = O.staged_rows(x_all[rank][:64], topk_all[rank][:64], rank, e, t, fmt, r)
+    payload = O.row_payload(h, fmt)
+    sendbuf = st.send_slots.view(e, t, st.stride)
+    for i in range(0, rows.shape[0], 7):
+        ex, sl = int(experts[i]), int(slots[i])
+        if ex // (e // r) != rank:
+            assert torch.equal(sendbuf[ex, sl, :payload].cpu(), rows[i, :payload]), (ex, sl)
