@@ -293,6 +293,7 @@ def recv_by_source_on_gpu(rt, buf, routed, rank, e, m, h, fmt, slot_rows, capaci
     (8, 3, 700, 512, 8, 256),     # past 4096 records: chunk histograms, sources of two chunks each
     (4, 1, 900, 512, 4, 16),      # up to 4096 records: one workgroup per source walks its two chunks, running counts
     (16, 2, 1200, 512, 8, 64),    # 9600 records in chunks of 512, about 600 per source
+    (16, 5, 4096, 512, 8, 64),    # 32768 records: four chunks per source, 80 chunk workgroups
     (1, 0, 16, 512, 2, 4),        # a world of one rank
     (4, 2, 64, 512, 2, 4),        # one expert per rank
     (2, 1, 40, 512, 6, 2048),     # 1024 local experts: ten bits of expert id
@@ -879,3 +880,54 @@ def test_send_past_the_streaming_bound(rt, one_call, fmt):
         ex, sl = int(experts[i]), int(slots[i])
         if ex // (e // r) != rank:
             assert torch.equal(sendbuf[ex, sl, :payload].cpu(), rows[i, :payload]), (ex, sl)
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
+def test_every_rank_on_one_gpu_through_an_all_to_all(rt, fmt):
+    """The data flow of the all_to_all_single fallback (deep_ep/buffer.py:2268,2297) with all R ranks on the
+    one GPU: every rank's send side fills its per-expert slots; the "all-gather" of the route counts is the
+    stack of the ranks' send_count; each rank's message to rank d is its rows for d's experts, expert by
+    expert, copied into slot `source` of d's receive buffer; deepep_ll_exchange_metadata turns the gathered
+    counts into the records and deepep_ll_dispatch_recv_by_source unpacks.  The packed outputs must be the
+    oracle's (csrc/kernels/efa_kernels.cu:877-1052,1227-1389; csrc/transport/ll_pipeline.cpp:1204-1361)."""
+    r, t, h, k, e = 4, 40, 512, 3, 16
+    epr = e // r
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=321, drop=6)
+    lib, capi = rt.capi.load(), rt.capi
+    states = []
+    for rank in range(r):
+        st = rt.ll.LowLatencyState(rt.ll.LLShape(r, rank, e, t, h, k, fmt))
+        st.dispatch_send(x_all[rank].cuda(), topk_all[rank].cuda())
+        states.append(st)
+    torch.cuda.synchronize()
+    routed = torch.stack([st.send_count for st in states])  # [R, E]: what an all-gather of the counts leaves everywhere
+    slot_rows = t * min(k, epr)
+    stride = states[0].stride
+    for rank in range(r):
+        # the messages: source s -> this rank, rows in expert-major order (inside an expert, slot order)
+        buf = torch.full((r * slot_rows, stride), 0xEE, dtype=torch.uint8, device="cuda")
+        for s in range(r):
+            src = states[s]
+            counts = src.send_count.cpu()
+            if s == rank:  # a rank's rows for its own experts were staged, not put into send slots
+                own = src.recv_staging.view(epr, r, t, stride)
+                parts = [own[le, rank, :int(counts[rank * epr + le])] for le in range(epr)]
+            else:
+                slots = src.send_slots.view(e, t, stride)
+                parts = [slots[ex, :int(counts[ex])] for ex in range(rank * epr, (rank + 1) * epr)]
+            msg = torch.cat(parts)
+            buf[s * slot_rows:s * slot_rows + msg.shape[0]] = msg
+        capacity = int(routed[:, rank * epr:(rank + 1) * epr].sum())
+        meta = rt.ll.exchange_metadata(routed, rank, slot_rows, capacity)
+        st = states[rank]
+        poison_outputs_keep_pair_slot(st)
+        ws = torch.empty(lib.deepep_ll_by_source_workspace_bytes(e, capacity), dtype=torch.uint8, device="cuda")
+        capi.check(lib.deepep_ll_dispatch_recv_by_source(
+            capi.ptr(buf), slot_rows, capi.ptr(meta["recv_counts"]), capi.ptr(meta["source_offset"]),
+            capi.ptr(meta["num_recv_tokens"]), capacity, h, e, r, t, fmt, capi.ptr(st.packed_recv_x),
+            capi.ptr(st.packed_recv_scales), capi.ptr(st.packed_recv_src_info), capi.ptr(st.packed_recv_layout_range),
+            capi.ptr(st.packed_recv_count), None, None, capi.ptr(ws), ws.numel(), torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
+        check_dispatch(st, want, fmt)
+        assert int(meta["num_recv_tokens"][0]) == int(want["packed_recv_count"].sum())
