@@ -88,6 +88,20 @@ __device__ __forceinline__ int upper_source(const int32_t* table, int n, int64_t
     return lo;
 }
 
+// Sum of hist[c * E_l + e] over the chunks [c_begin, c_end), eight loads in flight at a time.
+__device__ __forceinline__ int sum_chunk_counts(const int32_t* __restrict__ hist, int num_local_experts, int e,
+                                                int c_begin, int c_end) {
+    int sum = 0;
+    for (int c0 = c_begin; c0 < c_end; c0 += 8) {
+        int v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = c0 + u < c_end ? hist[int64_t(c0 + u) * num_local_experts + e] : 0;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += v[u];
+    }
+    return sum;
+}
+
 // Large batches, first launch: hist[g * E_l + e] = records of chunk g, inside their source's slot,
 // whose row names local expert e.
 __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_count_kernel(
@@ -156,20 +170,15 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
         // (expert, source) counts: the column sums of the source's chunk histograms
         for (int q = tid; q < num_segments; q += kBySourceThreads) {
             const int e = q / num_ranks, src = q - e * num_ranks;
-            int sum = 0;
-            for (int c = chunk_prefix[src]; c < chunk_prefix[src + 1]; ++c) sum += hist[int64_t(c) * num_local_experts + e];
-            pair_prefix[q] = sum;
+            pair_prefix[q] = sum_chunk_counts(hist, num_local_experts, e, chunk_prefix[src], chunk_prefix[src + 1]);
         }
         const bool has_rows = g < chunk_prefix[num_ranks];
         s = has_rows ? upper_source(chunk_prefix, num_ranks, g) : 0;
         first_chunk = has_rows ? g - chunk_prefix[s] : 0;
         num_chunks = has_rows ? 1 : 0;
         // rows of the same (expert, source) pair in the source's earlier chunks
-        for (int e = tid; e < num_local_experts; e += kBySourceThreads) {
-            int sum = 0;
-            for (int c = chunk_prefix[s]; c < chunk_prefix[s] + first_chunk; ++c) sum += hist[int64_t(c) * num_local_experts + e];
-            running[e] = sum;
-        }
+        for (int e = tid; e < num_local_experts; e += kBySourceThreads)
+            running[e] = sum_chunk_counts(hist, num_local_experts, e, chunk_prefix[s], chunk_prefix[s] + first_chunk);
     } else {
         s = blockIdx.x;
         for (int q = tid; q < num_segments; q += kBySourceThreads) pair_prefix[q] = 0;
@@ -200,7 +209,7 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
             if (stats != nullptr) stats[le] += c;
             if (tokens_per_expert != nullptr) tokens_per_expert[le] = uint32_t(c);
         }
-        if (tid == 0) flat_total[0] = int32_t(records < prefix[num_ranks] ? records : prefix[num_ranks]);
+        if (tid == 0) flat_total[0] = pair_prefix[num_segments];  // one descriptor per row that names an expert
     }
 
     int64_t begin, end, live_end;
@@ -227,19 +236,19 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
         const int before_in_wave = __popcll(same & lanes_below(lane));
         if (e >= 0 && (same >> lane) >> 1 == 0) wave_cnt[w * num_local_experts + e] = __popcll(same);  // the group's last lane
         lds_barrier();
-        if (i < end) {
+        if (e >= 0) {
+            // The descriptors are laid out in the order of the packed rows (expert, source, arrival), not of
+            // the records: the copy then writes consecutive rows from consecutive workgroups.
+            int pos = running[e] + before_in_wave;
+            for (int w2 = 0; w2 < w; ++w2) pos += wave_cnt[w2 * num_local_experts + e];
+            const int64_t pair_begin = pair_prefix[e * num_ranks + s] - pair_prefix[e * num_ranks];
             RowDesc d;
-            d.src_row = -1, d.dst_row = 0;  // a row without a valid expert is not copied
-            if (e >= 0) {
-                int pos = running[e] + before_in_wave;
-                for (int w2 = 0; w2 < w; ++w2) pos += wave_cnt[w2 * num_local_experts + e];
-                const int64_t pair_begin = pair_prefix[e * num_ranks + s] - pair_prefix[e * num_ranks];
-                if (pair_begin + pos < slots_per_expert) {
-                    d.src_row = int32_t(offset);
-                    d.dst_row = int32_t(int64_t(e) * slots_per_expert + pair_begin + pos);
-                }
+            d.src_row = -1, d.dst_row = 0;  // a row past its expert's slots is not copied
+            if (pair_begin + pos < slots_per_expert) {
+                d.src_row = int32_t(offset);
+                d.dst_row = int32_t(int64_t(e) * slots_per_expert + pair_begin + pos);
             }
-            desc[i] = d;
+            desc[pair_prefix[e * num_ranks + s] + pos] = d;
         }
         if constexpr (kChunked) break;  // one chunk per workgroup
         lds_barrier();
