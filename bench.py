@@ -12,7 +12,11 @@ Prints ONE JSON line.  `value` is microseconds of stream time per step over K
 steps: the steps are enqueued by HIP-graph replays so the GPU never waits for
 the host (launching call by call from Python costs more than the kernels take;
 that figure is reported beside it).  Per-entry durations are measured the same
-way; the roofline of the slower of the two step kernels is in the same line.
+way; the roofline of the slower of the two step kernels is in the same line,
+quoted with every launch after a flush of the caches (replayed back to back the
+step's 66 MB never leave the 256 MB memory-side cache).  The sections at 4096
+tokens take two or more sets of buffers in turn for the same reason: a call
+must not find its bytes where the call before left them.
 """
 import argparse
 import json
