@@ -178,8 +178,8 @@ __device__ __forceinline__ void send_count_block(const SendArgs& a, int b, int32
                           a.send_count);
 }
 
-// One workgroup's share of token t of source b.  kStream: the call moves more than the caches hold,
-// so the payload of the rows is stored with the non-temporal hint; at 4096 tokens, with the
+// One workgroup's share of token t of source b.  kStream (64 MB of traffic and more): the payload of
+// the rows is stored with the non-temporal hint; at 4096 tokens, with the
 // destinations in HBM, that takes the send from 73 to 53 us (a row stored the ordinary way is first
 // allocated in the memory-side cache and written back later).  The token rows are read, and the
 // scales and tails stored, the ordinary way: the hint measured slower on those (63 and 56 us).
@@ -798,7 +798,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     // rows read once and written K times (about that many: a dropped selection writes nothing)
     const int64_t traffic = int64_t(num_src) * num_tokens *
                             (int64_t(hidden) * 2 + int64_t(num_topk) * row_payload_bytes(hidden, row_format));
-    const bool streams = traffic > stream_bytes();
+    const bool streams = traffic > send_stream_bytes();
 #define DEEPEP_LAUNCH_SEND(FMT)                                                           \
     do {                                                                                  \
         if (streams) ll_send_kernel<FMT, true><<<grid, waves * kWave, lds, stream>>>(sa, direct);  \
