@@ -39,11 +39,14 @@ generative on CUDA RNG streams that cannot be replayed here):
   hand-derived two-rank world (``tests/golden/ll_tiny_world.json``) and by the identities that tie it to
   the dispatch (recv_counts = row sums of the receiver's ``recv_count``; records = a running index).
 * ``get_low_latency_rdma_size_hint`` — hand-computed values.
-* ``round_scale`` scales: **parity unpinned at ulp boundaries** — the reference
-  computes ``exp2(ceil(log2(s)))`` in float32 (``deep_ep/buffer.py:1601``,
-  ``csrc/kernels/efa_kernels.cu:158``), whose result for s within one ulp above
-  a power of two depends on the libm in use; this oracle (and the kernel) take
-  the mathematical value, the smallest power of two >= s.
+* ``round_scale`` scales — the reference computes ``exp2(ceil(log2(s)))`` in float32
+  (``deep_ep/buffer.py:1601``, ``csrc/kernels/efa_kernels.cu:158``); this oracle (and the kernel)
+  take the smallest power of two >= s from the bit pattern.  The two could differ only for s
+  within a few ulps above a power of two, where log2f's rounding decides the ceiling; on this
+  path s = amax / 448 with amax a bf16 value or the 1e-4 clamp, and over every such amax log2(s) is
+  an integer exactly or at least 0.006 away from one, so every libm gives the same answer.
+  Pinned by that enumeration and by torch's float32 log2 / ceil / exp2 on the CPU agreeing on all of
+  them (``tests/test_oracle.py::test_round_scale_has_one_answer_for_every_bf16_amax``).
 """
 from __future__ import annotations
 

@@ -543,3 +543,27 @@ def test_oracle_exchange_metadata_identities_and_corrupt_counts():
     bad = O.ll_exchange_metadata(routed, rank, m)
     assert bad["corrupt"] and bad["total_send"] == 0 and bad["total_recv"] == 0
     assert bad["send_counts"].sum() == 0 and bad["recv_counts"].sum() == 0 and bad["source_rank"].numel() == 0
+
+
+def test_round_scale_has_one_answer_for_every_bf16_amax():
+    """The reference rounds a scale up to a power of two as exp2(ceil(log2(s))) in float32
+    (csrc/kernels/efa_kernels.cu:158, deep_ep/buffer.py:1601); oracle and kernel take the smallest power of
+    two >= s from the bit pattern.  The two can only differ where log2f's rounding error carries ceil over an
+    integer, i.e. for s a hair above a power of two.  On this path s = amax / 448 with amax a bf16 value (or the
+    1e-4 clamp), and that never happens: over every positive finite bf16 amax, log2(s) is either an integer
+    exactly (amax = 1.75 * 2^j) or at least 0.006 away from one — four hundred times the spacing of float32
+    near the largest |log2(s)| — so any log2f good to a few ulps gives the same ceiling.  torch's own
+    float32 log2 / ceil / exp2 on the CPU, the form the reference's Python writes, agrees on every one."""
+    bits = torch.arange(1, 0x7F80, dtype=torch.int32)  # every positive finite bf16, subnormals included
+    amax = (bits << 16).view(torch.float32).clamp(min=1e-4)
+    amax = torch.cat([amax, torch.tensor([1e-4])])
+    s = amax / 448.0
+    exact = np.log2(s.numpy().astype(np.float64))
+    off = np.abs(exact - np.round(exact))
+    is_pow2 = (s.view(torch.int32) & 0x7FFFFF).numpy() == 0
+    assert (off[is_pow2] == 0).all() and is_pow2.sum() > 100
+    assert off[~is_pow2].min() > 0.006
+    assert np.abs(exact).max() < 128 and np.spacing(np.float32(127.0)) < 0.006 / 400
+    want = np.exp2(np.ceil(exact)).astype(np.float32)
+    assert np.array_equal(O.pow2_ceil(s).numpy(), want)
+    assert torch.equal(torch.exp2(torch.ceil(torch.log2(s))), O.pow2_ceil(s))
