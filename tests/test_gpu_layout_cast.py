@@ -240,6 +240,18 @@ def test_cast_every_bf16_value_under_many_amax(capi, fmt):
 
 
 @pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_FP8_POW2, O.ROW_FP8_UE8M0])
+def test_cast_every_bf16_value_as_the_amax_of_a_group(capi, fmt):
+    """One group per positive finite bf16 value (and its negative), that value its only non-zero element: the
+    scale of every possible amax, power-of-two rounding included, against the oracle."""
+    bits = torch.arange(1, 0x7F80, dtype=torch.int32)
+    vals = torch.cat([bits, bits | 0x8000]).to(torch.int16).view(torch.bfloat16)
+    pad = (-vals.numel()) % 4
+    x = torch.zeros((vals.numel() + pad, 128), dtype=torch.bfloat16)
+    x[:vals.numel(), 77] = vals
+    _check_cast(capi, x.view(-1, 512).contiguous(), fmt)
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_FP8_POW2, O.ROW_FP8_UE8M0])
 @pytest.mark.parametrize("m,n", [(128, 7168), (1, 512), (33, 1536), (7, 4096)])
 def test_cast_random_and_outliers(capi, fmt, m, n):
     if fmt == O.ROW_FP8_UE8M0 and (n // 128) % 4:
