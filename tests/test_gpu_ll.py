@@ -314,11 +314,12 @@ def test_dispatch_recv_by_source(rt, fmt, r, rank, t, h, k, e):
     assert int(meta["num_recv_tokens"][0]) == int(want["packed_recv_count"].sum())
 
 
-def test_dispatch_recv_by_source_drops_what_does_not_fit(rt):
+@pytest.mark.parametrize("t", [24, 1500], ids=["one_workgroup_per_source", "chunked"])
+def test_dispatch_recv_by_source_drops_what_does_not_fit(rt, t):
     """A slot of M rows per source, as the reference sizes it (csrc/transport/ll_pipeline.cpp:1527): rows a
     source sends beyond it are lost, the others land as if the lost ones had not been sent; and with fewer
     record slots than rows, only the rows that have a record are received."""
-    r, rank, t, h, k, e, fmt = 2, 0, 24, 512, 4, 8, O.ROW_FP8
+    r, rank, h, k, e, fmt = 2, 0, 512, 4, 8, O.ROW_FP8
     x_all, topk_all, _ = make_world(r, t, h, k, e, seed=3, drop=0)
     topk_all[1, :, :] = torch.tensor([0, 1, 2, 3])  # every token of source 1 names all of rank 0's experts
     slot_rows = t  # source 1 sends 4 * t rows
@@ -346,9 +347,10 @@ def test_dispatch_recv_by_source_drops_what_does_not_fit(rt):
             for s in range(r):
                 rows = want_rows[le][s]
                 assert int(layout[le, s]) == (((begin << 32) | len(rows)) if rows else 0), (capacity, le, s)
-                for j, row in enumerate(rows):
-                    assert torch.equal(px[le, begin + j], buf[row, :h])
-                    assert int(st.packed_recv_src_info[le, begin + j]) == int(tail[row, 0])
+                if rows:
+                    idx = torch.tensor(rows)
+                    assert torch.equal(px[le, begin:begin + len(rows)], buf[idx, :h])
+                    assert torch.equal(st.packed_recv_src_info[le, begin:begin + len(rows)].cpu(), tail[idx, 0])
                 begin += len(rows)
             assert count[le] == begin
 
