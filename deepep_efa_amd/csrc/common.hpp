@@ -109,9 +109,11 @@ __device__ __forceinline__ void store_u32x4(uint8_t* p, u32x4 v) {
 }
 // Traffic above which a kernel streams (the memory-side cache holds 256 MB).
 inline int64_t stream_bytes() { return int64_t(192) << 20; }
-// The send side's payload stores stream from 64 MB of traffic on (every batch that does not go through
-// the single-launch dispatch): with clean caches the hint makes no difference from 1024 to 2560 tokens,
-// with the caches full of another call's dirty lines the send is 18 to 24 % faster with it.
+// The dispatch streams from 64 MB of traffic on (the send side's payload stores; in the single launch
+// the receive side's row copies too): with clean caches the hint makes no difference from 512 to 2560
+// tokens, with the caches full of another call's dirty lines the send is 18 to 24 % faster with it and
+// the single launch 11 to 16 %.  (The single-launch combine measured the other way: slower at 256 and
+// 512 tokens with the lower bound, so it keeps the 192 MB.)
 inline int64_t send_stream_bytes() { return int64_t(64) << 20; }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every

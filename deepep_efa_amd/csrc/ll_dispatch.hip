@@ -515,7 +515,7 @@ constexpr int kRecvDepth = 4;  // 16-byte loads in flight per lane
 // expert, where it comes from does not: a wave issues the loads of its first item before the
 // workgroup settles the own counts.
 // lds: [num_segments + 1 + num_local_experts] ints; wave_totals: 16 ints.
-template <int kPer>
+template <int kPer, bool kStream>
 __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int num_copy_blocks,
                                                const int64_t* own_topk, int own_entries, int own_rank, int32_t* lds,
                                                int32_t* wave_totals) {
@@ -599,7 +599,7 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
 #pragma unroll
         for (int u = 0; u < kRecvDepth; ++u) {
             const int v = it.v_begin + u * kWave + lane;
-            if (v < it.v_end) r[u] = load_u32x4<false>(it.src + int64_t(v) * 16);
+            if (v < it.v_end) r[u] = load_u32x4<kStream>(it.src + int64_t(v) * 16);
         }
     };
     auto finish = [&](const RecvItem& it, const u32x4 (&r)[kRecvDepth]) {
@@ -610,9 +610,9 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
 #pragma unroll
         for (int u = 0; u < kRecvDepth; ++u) {
             const int v = it.v_begin + u * kWave + lane;
-            if (v < it.v_end) store_u32x4<false>(dst + int64_t(v) * 16, r[u]);
+            if (v < it.v_end) store_u32x4<kStream>(dst + int64_t(v) * 16, r[u]);
         }
-        wave_copy_vec16<kRecvDepth>(it.src, dst, it.v_begin + kRecvDepth * kWave, it.v_end, lane);
+        wave_copy_vec16<kRecvDepth, kStream>(it.src, dst, it.v_begin + kRecvDepth * kWave, it.v_end, lane);
         if (!it.carries_tail) return;
         if (a.packed_scales != nullptr && scale_bytes > 0) {
             const uint32_t* s32 = reinterpret_cast<const uint32_t*>(it.src + data_pad);
@@ -646,12 +646,13 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
     }
 }
 
+template <bool kStream>
 __device__ __forceinline__ void recv_rows(const RecvArgs& a, int block, int num_copy_blocks, const int64_t* own_topk,
                                           int own_entries, int own_rank, int32_t* lds, int32_t* wave_totals) {
     if (a.num_local_experts * a.num_ranks <= 4 * kWave)
-        recv_rows_impl<4>(a, block, num_copy_blocks, own_topk, own_entries, own_rank, lds, wave_totals);
+        recv_rows_impl<4, kStream>(a, block, num_copy_blocks, own_topk, own_entries, own_rank, lds, wave_totals);
     else
-        recv_rows_impl<16>(a, block, num_copy_blocks, own_topk, own_entries, own_rank, lds, wave_totals);
+        recv_rows_impl<16, kStream>(a, block, num_copy_blocks, own_topk, own_entries, own_rank, lds, wave_totals);
 }
 
 // own_rank >= 0: the send side has already put this rank's own rows at their packed position.
@@ -659,7 +660,7 @@ __global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a, const int64_t*
                                                       int own_rank) {
     extern __shared__ int32_t flat[];  // [num_segments + 1 + E_l]
     __shared__ int32_t wave_totals[kMaxBlockWaves];
-    recv_rows(a, blockIdx.x, int(gridDim.x) - 1, own_topk, own_entries, own_rank, flat, wave_totals);
+    recv_rows<false>(a, blockIdx.x, int(gridDim.x) - 1, own_topk, own_entries, own_rank, flat, wave_totals);
 }
 
 // ---------------------------------------------------------------------
@@ -675,7 +676,7 @@ __global__ __launch_bounds__(256) void ll_recv_kernel(RecvArgs a, const int64_t*
 // (The reference's dispatch is one kernel with a send and a receive phase as
 // well: csrc/kernels/coop_dispatch_send.cuh:304, coop_dispatch_recv.cuh:42.)
 // ---------------------------------------------------------------------
-template <int kFmt>
+template <int kFmt, bool kStream>
 __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_dispatch_fused_kernel(SendArgs sa, RecvArgs ra, int blocks_per_token,
                                                                                  int num_send_blocks) {
     extern __shared__ int32_t dyn_lds[];  // counting: [E]; receive: [segments + 1 + E_l]
@@ -684,11 +685,11 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_dispatch_fused_kernel
     const int block = blockIdx.x;
     if (block < num_send_blocks) {
         const DirectOut direct = {ra.packed_x, ra.packed_scales, ra.src_info};
-        send_token_block<kFmt, false>(sa, direct, 0, block / blocks_per_token, block % blocks_per_token, lds);
+        send_token_block<kFmt, kStream>(sa, direct, 0, block / blocks_per_token, block % blocks_per_token, lds);
     } else if (block == num_send_blocks) {
         send_count_block(sa, 0, dyn_lds);
     } else {
-        recv_rows(ra, block - num_send_blocks - 1, int(gridDim.x) - num_send_blocks - 2, sa.topk_idx,
+        recv_rows<kStream>(ra, block - num_send_blocks - 1, int(gridDim.x) - num_send_blocks - 2, sa.topk_idx,
                   sa.num_tokens * sa.num_topk, sa.rank, dyn_lds, wave_totals);
     }
 }
@@ -775,9 +776,21 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
         const size_t need_count = size_t(num_experts) * sizeof(int32_t);
         const size_t lds = need_recv > need_count ? need_recv : need_count;
         const RecvArgs ra = *fused_recv;
+        // Token rows read and K copies written by the send workgroups, staged rows read and packed rows
+        // written by the receive workgroups.  From 64 MB on (about 350 tokens at hidden 7168, top-8) the
+        // launch streams: at 512 to 1024 tokens that changes nothing when the caches are clean and takes
+        // 11 to 16 % off when they are full of another call's dirty lines (44 against 50 us at 1024 tokens).
+        const int64_t payload = row_payload_bytes(hidden, row_format);
+        const int64_t fused_traffic = int64_t(num_tokens) * (int64_t(hidden) * 2 + int64_t(num_topk) * payload) +
+                                      2 * (fused_recv_wave_items >> ra.parts_log2) * payload;
+        const bool fused_streams = fused_traffic > send_stream_bytes();
 #define DEEPEP_LAUNCH_FUSED(FMT)                                                                        \
-    ll_dispatch_fused_kernel<FMT><<<dim3(unsigned(total)), waves * kWave, lds, stream>>>(sa, ra, blocks_per_token, \
-                                                                                         num_send_blocks)
+    do {                                                                                                \
+        if (fused_streams)                                                                              \
+            ll_dispatch_fused_kernel<FMT, true><<<dim3(unsigned(total)), waves * kWave, lds, stream>>>(sa, ra, blocks_per_token, num_send_blocks); \
+        else                                                                                            \
+            ll_dispatch_fused_kernel<FMT, false><<<dim3(unsigned(total)), waves * kWave, lds, stream>>>(sa, ra, blocks_per_token, num_send_blocks); \
+    } while (0)
         switch (row_format) {
             case kRowBF16: DEEPEP_LAUNCH_FUSED(kRowBF16); break;
             case kRowFP8: DEEPEP_LAUNCH_FUSED(kRowFP8); break;

@@ -933,3 +933,22 @@ def test_every_rank_on_one_gpu_through_an_all_to_all(rt, fmt):
         want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
         check_dispatch(st, want, fmt)
         assert int(meta["num_recv_tokens"][0]) == int(want["packed_recv_count"].sum())
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
+def test_single_launch_dispatch_past_the_streaming_bound(rt, fmt):
+    """700 tokens x 7168, top-8 on two ranks: 5600 entries, so the dispatch is one launch, and more than
+    64 MB of traffic, so that launch is the streaming instantiation."""
+    r, rank, t, h, k, e = 2, 0, 700, 7168, 8, 16
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=700, drop=10)
+    lib = rt.capi.load()
+    assert lib.deepep_ll_dispatch_is_single_launch(t, k, e, t, t * k) == 1
+    e_l = e // r
+    received = sum(int(((tk >= rank * e_l) & (tk < (rank + 1) * e_l)).sum()) for tk in topk_all)
+    assert t * (2 * h + k * O.row_payload(h, fmt)) + 2 * received * O.row_payload(h, fmt) > 64 * 2 ** 20
+    st, _ = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, fmt, one_call=True)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
+    check_dispatch(st, want, fmt)
+    send_count, pair_slot = O.route(topk_all[rank], e, t)
+    assert torch.equal(st.send_count.cpu(), send_count)
+    assert torch.equal(st.pair_slot.cpu(), pair_slot)
