@@ -314,6 +314,24 @@ def test_dispatch_recv_by_source(rt, fmt, r, rank, t, h, k, e):
     assert int(meta["num_recv_tokens"][0]) == int(want["packed_recv_count"].sum())
 
 
+@pytest.mark.parametrize("seed", range(int(os.environ.get("DEEPEP_TEST_RANDOM_SHAPES", "24"))))
+def test_dispatch_recv_by_source_seeded_random_shapes(rt, seed):
+    """The by-source receive on shapes nobody picked by hand, on both sides of its 4096-record bound."""
+    r, rank, t, _, h, k, e, fmt, drop = _random_shape(seed)
+    if seed % 3 == 0:
+        t = t * 7  # more records: sources of several chunks
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=2000 + seed, drop=drop)
+    m = t
+    slot_rows = t * min(k, e // r)
+    buf = rows_by_source(x_all, topk_all, rank, e, m, fmt, slot_rows)
+    routed = torch.stack([O.route(topk_all[s], e, m)[0] for s in range(r)]).to(torch.int32)
+    capacity = int(routed[:, rank * (e // r):(rank + 1) * (e // r)].sum()) + seed % 4
+    st, tokens_per_expert, meta = recv_by_source_on_gpu(rt, buf, routed, rank, e, m, h, fmt, slot_rows, capacity)
+    want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, m, fmt)
+    check_dispatch(st, want, fmt)
+    assert torch.equal(tokens_per_expert.cpu(), want["packed_recv_count"])
+
+
 @pytest.mark.parametrize("t", [24, 1500], ids=["one_workgroup_per_source", "chunked"])
 def test_dispatch_recv_by_source_drops_what_does_not_fit(rt, t):
     """A slot of M rows per source, as the reference sizes it (csrc/transport/ll_pipeline.cpp:1527): rows a
