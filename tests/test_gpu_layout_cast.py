@@ -353,6 +353,63 @@ def test_combine_reduce(capi, t, k, e, r, h, with_bias):
     assert torch.allclose(out_w.cpu().double(), ref_w, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("seed", range(int(os.environ.get("DEEPEP_TEST_RANDOM_SHAPES", "16"))))
+def test_pack_remap_reduce_seeded_random_shapes(capi, seed):
+    """Pack, top-k remap and the combine reduce on shapes nobody picked by hand: odd rank counts, ragged
+    hidden sizes, tokens that go nowhere."""
+    lib = capi.load()
+    g = np.random.default_rng(900 + seed)
+    r = int(g.choice([1, 2, 3, 5, 8, 9, 16, 24, 64, 65, 100]))
+    epr = int(g.choice([1, 2, 3, 8]))
+    e = r * epr
+    k = int(g.integers(1, min(e, 10) + 1))
+    t = int(g.choice([5, 6, 63, 64, 65, 255, 257, 1000, 1500]))
+    h = int(g.choice([8, 64, 128, 136, 512, 520, 1024, 2056]))  # row bytes = 2h: a multiple of 16
+    with_bias = bool(g.integers(0, 2))
+    topk, w, is_in, ids, counts, cumsum, total = _normal_world(t, k, e, r, seed=3000 + seed)
+    topk[:: max(2, t // 3)] = -1  # tokens no rank holds
+    _, _, _, is_in = O.get_dispatch_layout(topk, e, r)
+    ids, counts, cumsum, total = O.moe_routing_sort(is_in)
+    tg = torch.Generator().manual_seed(seed)
+    x = torch.randn((t, h), generator=tg).to(torch.bfloat16)
+    # pack: rows gathered into per-rank contiguous order
+    cap = total + 5
+    ids_full = torch.full((cap,), -1, dtype=torch.int64)
+    ids_full[:total] = ids
+    dev = dict(x=x.cuda(), ids=ids_full.cuda(), n=torch.tensor([total], dtype=torch.int64, device="cuda"))
+    packed = torch.full((cap, h), float("nan"), dtype=torch.bfloat16, device="cuda")
+    capi.check(lib.deepep_pack_rows(capi.ptr(dev["x"]), None, capi.ptr(dev["ids"]), capi.ptr(dev["n"]), cap, t, h * 2, 0,
+                                    capi.ptr(packed), None, stream()))
+    torch.cuda.synchronize()
+    assert torch.equal(packed[:total].cpu().view(torch.int16), x[ids].view(torch.int16))
+    assert packed[total:].isnan().all()
+    # remap
+    want_e, want_w = O.topk_remap(topk, w, ids, cumsum, epr)
+    out_e = torch.full((cap, k), -99, dtype=torch.int64, device="cuda")
+    out_w = torch.full((cap, k), -99.0, dtype=torch.float32, device="cuda")
+    topk_dev, w_dev, cumsum_dev = topk.cuda(), w.cuda(), cumsum.cuda()
+    capi.check(lib.deepep_topk_remap(capi.ptr(topk_dev), capi.ptr(w_dev), capi.ptr(dev["ids"]), capi.ptr(cumsum_dev), t, k,
+                                     r, epr, cap, capi.ptr(out_e), capi.ptr(out_w), stream()))
+    torch.cuda.synchronize()
+    assert torch.equal(out_e[:total].cpu(), want_e) and torch.equal(out_w[:total].cpu(), want_w)
+    assert (out_e[total:] == -99).all()
+    # reduce of rows that come back changed
+    rows = torch.randn((total, h), generator=tg).to(torch.bfloat16)
+    b0 = torch.randn((t, h), generator=tg).to(torch.bfloat16) if with_bias else None
+    b1 = torch.randn((t, h), generator=tg).to(torch.bfloat16) if with_bias else None
+    out_x = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    out_x.view(torch.int16).fill_(0x7FC0)
+    out_cw = torch.full((t, k), float("nan"), dtype=torch.float32, device="cuda")
+    ws = torch.full((max(256, lib.deepep_combine_reduce_workspace_bytes(t, r)),), 0x7F, dtype=torch.uint8, device="cuda")
+    held = [None if v is None else v.cuda() for v in (rows, want_w, ids, cumsum, is_in, b0, b1)]
+    capi.check(lib.deepep_combine_reduce(*[capi.ptr(v) for v in held], t, h, k, r, total, capi.ptr(out_x),
+                                         capi.ptr(out_cw), capi.ptr(ws), ws.numel(), stream()))
+    torch.cuda.synchronize()
+    chain_x, chain_w = O.combine_reduce_f32_chain(rows, want_w, ids, cumsum, t, b0, b1)
+    assert torch.equal(out_x.cpu().view(torch.int16), chain_x.view(torch.int16))
+    assert torch.equal(out_cw.cpu(), chain_w)
+
+
 def test_normal_mode_steps_through_the_host_module():
     """topk_remap / build_recv_src_meta / combine_reduce with the reference's Python-visible signatures."""
     from deepep_efa_amd import normal
