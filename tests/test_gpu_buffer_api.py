@@ -369,11 +369,14 @@ def test_normal_mode_layout_and_pack(deep_ep):
     buffer.destroy()
 
 
-def test_dispatch_and_combine_replay_in_a_hip_graph(deep_ep):
+@pytest.mark.parametrize("num_ranks,rank,t,h,k,e", [
+    (16, 4, 64, 2048, 6, 64),   # one launch per direction
+    (8, 3, 2200, 512, 8, 64),   # the large-batch kernels: histograms + send + index + copy, index + copy + reduce
+], ids=["decode_size", "large_batch"])
+def test_dispatch_and_combine_replay_in_a_hip_graph(deep_ep, num_ranks, rank, t, h, k, e):
     """Decode loops capture the dispatch + combine pair once and replay it.  The captured calls must
     allocate nothing and record no memset; every replay, with eager work and synchronisations in
     between, must give the eager result."""
-    num_ranks, rank, t, h, k, e = 16, 4, 64, 2048, 6, 64
     buffer = deep_ep.Buffer(None, low_latency_mode=True, explicitly_destroy=True, sim_num_ranks=num_ranks,
                             sim_rank=rank, sim_seed=21)
     x, topk_idx = buffer.loopback_synthesise(t, h, k, e)
