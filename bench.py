@@ -48,6 +48,8 @@ def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0, packed=None):
         "dispatch": (t * 2 * h + t * k * 8 + (p - own) * stride + own * packed + t * k * 4 + e * 4
                      + (rv - own) * (stride + packed) + small),
         "combine": (rv - own) * 2 * h * 2 + (e // r) * r * 8 + p * 2 * h + t * k * 16 + t * 2 * h,
+        # zero copy: no row is returned, the transport sends the ranges of layout_range from the expert outputs
+        "combine_zero_copy": (e // r) * r * 8 + p * 2 * h + t * k * 16 + t * 2 * h,
         "exchange_metadata": r * e * 4 + rv * 16 + r * 24,
         # the staged receive's bytes plus, per row, the record, the tail read and the descriptor
         "dispatch_recv_by_source": rv * stride + rv * packed + small + rv * 12,
@@ -381,10 +383,13 @@ def bench_api_step(torch, args):
     torch.cuda.synchronize()
     buffer.loopback_clear_world()  # the exchange is done: later calls run this rank's own kernels only
 
-    def step():
+    def step(zero_copy=False):
         _, _, hd, _, _ = buffer.low_latency_dispatch(x, topk_idx, t, e)
-        buffer.low_latency_combine(y, topk_idx, weights, hd)
+        buffer.low_latency_combine(y, topk_idx, weights, hd, zero_copy=zero_copy)
 
+    # zero_copy: the expert outputs are written into the buffer of get_next_low_latency_combine_buffer
+    # and sent from there, so the combine returns no rows (deep_ep/buffer.py:2831-2852)
+    buffer.get_next_low_latency_combine_buffer(handle)
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     for _ in range(args.warmup):
         step()
@@ -418,6 +423,20 @@ def bench_api_step(torch, args):
             ev1.record()
             torch.cuda.synchronize()
             res["graph_us"] = round(ev0.elapsed_time(ev1) * 1e3 / args.steps, 2)
+            del g
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for _ in range(per_graph):
+                    step(zero_copy=True)
+            for _ in range(max(1, args.warmup // per_graph)):
+                g.replay()
+            torch.cuda.synchronize()
+            ev0.record()
+            for _ in range(args.steps // per_graph):
+                g.replay()
+            ev1.record()
+            torch.cuda.synchronize()
+            res["graph_zero_copy_us"] = round(ev0.elapsed_time(ev1) * 1e3 / args.steps, 2)
             del g
         except Exception as exc:
             res["graph_us"] = None
@@ -530,6 +549,7 @@ def main():
             *meta_args, torch.cuda.current_stream().cuda_stream)),
         "dispatch": lambda: st.dispatch(x, topk),  # send + receive phase, one launch at this size
         "combine": lambda: st.combine(y, topk, weights, out),  # row return + reduce, one launch at this size
+        "combine_zero_copy": lambda: st.combine(y, topk, weights, out, zero_copy=True),  # the reduce alone
         "dispatch_send": lambda: st.dispatch_send(x, topk),
         "dispatch_recv": lambda: st.dispatch_recv(),
         "combine_send": lambda: st.combine_send(y),

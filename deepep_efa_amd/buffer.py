@@ -272,7 +272,9 @@ class Buffer:
         self.runtime.low_latency_clean_mask_buffer()
 
     def get_next_low_latency_combine_buffer(self, handle: tuple) -> torch.Tensor:
-        """The [E_l, N, H] bf16 buffer the next `low_latency_combine(..., zero_copy=True)` reads."""
+        """The [E_l, N, H] bf16 buffer the next `low_latency_combine(..., zero_copy=True)` reads and the transport
+        sends from (the rows of a source rank are one contiguous range of it, `layout_range`): that combine skips
+        the row return, as deep_ep/buffer.py:2831-2852 promises."""
         _, _, num_max_dispatch_tokens_per_rank, hidden, num_experts = handle
         return self.runtime.get_next_low_latency_combine_buffer(num_max_dispatch_tokens_per_rank, hidden, num_experts)
 

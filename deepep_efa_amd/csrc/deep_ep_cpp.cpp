@@ -556,7 +556,10 @@ struct Buffer {
         auto stream = current_stream();
 
         torch::Tensor src = x;
-        if (zero_copy) {  // the caller wrote its expert outputs into the buffer handed out earlier
+        // zero_copy: the caller wrote its expert outputs into the buffer handed out earlier, and that buffer is
+        // what the transport sends from (the ranges of layout_range are contiguous in it), so the combine skips
+        // the row return -- "the next combine kernel can skip the copying", deep_ep/buffer.py:2831-2852
+        if (zero_copy) {
             EP_HOST_ASSERT(!combine_input_buffers.empty() and combine_input_buffers[combine_buffer_idx].defined());
             src = combine_input_buffers[combine_buffer_idx];
             EP_HOST_ASSERT(src.size(0) == x.size(0) and src.size(1) == x.size(1) and src.size(2) == x.size(2));
@@ -579,7 +582,8 @@ struct Buffer {
         abi_check(deepep_ll_combine(src.data_ptr(), layout_range.data_ptr<int64_t>(), topk_idx.data_ptr<int64_t>(),
                                     topk_weights.data_ptr<float>(), c.pair_slot.data_ptr<int>(), num_combined_tokens,
                                     hidden, num_topk, num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,
-                                    accumulate ? 1 : 0, c.combine_staging.data_ptr(), c.combine_send_slots.data_ptr(),
+                                    accumulate ? 1 : 0, c.combine_staging.data_ptr(),
+                                    zero_copy ? nullptr : c.combine_send_slots.data_ptr(),
                                     combined_x.data_ptr(), /*expected_rows=*/std::max<int64_t>(num_combined_tokens, 1) * num_topk,
                                     c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
                                     c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));

@@ -440,11 +440,18 @@ int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t*
     // the phases back to back), although each phase timed alone on cache-warm data suggests otherwise
     if (estimated_rows(expected_rows, num_experts, num_max_dispatch_tokens_per_rank) > kLargeBatchRows) {
         // the two phases back to back, with the single launch's shortcut: the rows owed to this rank
-        // itself are not moved, the reduce reads them from x
-        if (int rc = launch_combine_send(x, layout_range, hidden, num_experts, num_ranks, rank,
-                                         num_max_dispatch_tokens_per_rank, combine_staging, combine_send_slots,
-                                         expected_rows, workspace, workspace_bytes, true, stream))
+        // itself are not moved, the reduce reads them from x.  Without send slots (zero copy: the transport
+        // sends layout_range's ranges straight from x) there is nothing to return.
+        if (combine_send_slots == nullptr) {
+            if (int rc = check_combine_send_args(x, layout_range, hidden, num_experts, num_ranks, rank,
+                                                 num_max_dispatch_tokens_per_rank, combine_staging, nullptr))
+                return rc;
+        } else if (int rc = launch_combine_send(x, layout_range, hidden, num_experts, num_ranks, rank,
+                                                num_max_dispatch_tokens_per_rank, combine_staging,
+                                                combine_send_slots, expected_rows, workspace, workspace_bytes, true,
+                                                stream)) {
             return rc;
+        }
         return launch_combine_recv(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden, num_topk,
                                    num_experts, num_max_dispatch_tokens_per_rank, accumulate, out, x, layout_range,
                                    rank, num_ranks, stream);

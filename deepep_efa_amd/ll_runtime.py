@@ -148,8 +148,9 @@ class LowLatencyState:
             current_stream_ptr()))
 
     def combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor,
-                layout_range: torch.Tensor = None, accumulate: bool = False) -> None:
-        """Row return + weighted reduce in one call; the remote experts' answers must already be staged."""
+                layout_range: torch.Tensor = None, accumulate: bool = False, zero_copy: bool = False) -> None:
+        """Row return + weighted reduce in one call; the remote experts' answers must already be staged.
+        zero_copy: no row return, the transport sends the ranges of layout_range straight from x."""
         s = self.shape
         t = topk_idx.shape[0]
         lr = self.packed_recv_layout_range if layout_range is None else layout_range
@@ -157,8 +158,9 @@ class LowLatencyState:
         _capi.check(self.lib.deepep_ll_combine(
             _capi.ptr(x), _capi.ptr(lr), _capi.ptr(topk_idx), _capi.ptr(topk_weights), _capi.ptr(self.pair_slot),
             t, s.hidden, s.num_topk, s.num_experts, s.num_ranks, s.rank, s.max_tokens, int(accumulate),
-            _capi.ptr(self.combine_staging), _capi.ptr(self.combine_send_slots), _capi.ptr(out),
-            self.expected_rows, _capi.ptr(sw), 0 if sw is None else sw.numel(), current_stream_ptr()))
+            _capi.ptr(self.combine_staging), None if zero_copy else _capi.ptr(self.combine_send_slots),
+            _capi.ptr(out), self.expected_rows, _capi.ptr(sw), 0 if sw is None else sw.numel(),
+            current_stream_ptr()))
 
 
 def exchange_metadata(all_num_routed: torch.Tensor, rank: int, max_tokens: int, row_capacity: int) -> dict:

@@ -430,7 +430,11 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx,
  * answers of this rank's own experts are read from x directly — the own
  * experts' part of combine_staging is neither written nor read.  When at most
  * 8192 rows are expected both phases run as one kernel launch, larger batches
- * launch them back to back. */
+ * launch them back to back.  combine_send_slots may be NULL (the reference's
+ * zero_copy, deep_ep/buffer.py:2831-2852: "the next combine kernel can skip the
+ * copying"): no row is returned, the call is the reduce alone, and the caller's
+ * transport sends the rows of (e_l, s) from where they are,
+ * x[e_l, begin .. begin + count) of layout_range[e_l, s], which is contiguous. */
 int deepep_ll_combine(const void* x, const int64_t* layout_range,
                       const int64_t* topk_idx, const float* topk_weights,
                       const int32_t* pair_slot,

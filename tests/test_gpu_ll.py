@@ -706,12 +706,15 @@ def test_large_batch_without_the_segment_workspace(rt, oracle_c):
     assert O.calc_diff(x_all[rank].float() * wsum, out.cpu()) < 9e-4
 
 
+@pytest.mark.parametrize("zero_copy", [False, True], ids=["rows_returned", "zero_copy"])
 @pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
-def test_every_rank_on_one_gpu_with_a_real_exchange(rt, fmt):
+def test_every_rank_on_one_gpu_with_a_real_exchange(rt, fmt, zero_copy):
     """All R ranks run on the one GPU, each with its own buffers, and the exchange between them is a
     plain copy of what the send sides produced (send_slots -> the peer's recv_staging, then
     combine_send_slots -> the peer's combine_staging).  Nothing is synthesised "in a peer's name":
-    this is the data flow of a multi-GPU run with the transport replaced by device copies."""
+    this is the data flow of a multi-GPU run with the transport replaced by device copies.
+    zero_copy: the combine returns no rows; the exchange takes each (expert, source) range straight
+    from the expert outputs, where layout_range says it lies."""
     r, t, h, k, e = 4, 12, 512, 3, 16
     epr = e // r
     x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=123, drop=4)
@@ -750,7 +753,8 @@ def test_every_rank_on_one_gpu_with_a_real_exchange(rt, fmt):
             q = st.packed_recv_x.float().view(epr, r * t, h // 128, 128)
             y = (q * st.packed_recv_scales.unsqueeze(-1)).view(epr, r * t, h).to(torch.bfloat16)
         y = torch.nan_to_num(y, nan=0.0, posinf=0.0, neginf=0.0)  # rows past the counts hold poison
-        st.combine_send(y)
+        if not zero_copy:
+            st.combine_send(y)
         outs.append(y)
     torch.cuda.synchronize()
     # the combine exchange: what rank q returns for rank s's pairs goes to s's staging for q's experts
@@ -762,15 +766,24 @@ def test_every_rank_on_one_gpu_with_a_real_exchange(rt, fmt):
             for s in range(r):
                 if s == q:
                     continue
-                cnt = int(lr[le, s] & 0xFFFFFFFF)
-                states[s].combine_staging[q * epr + le, :cnt] = back[le, s, :cnt]
+                begin, cnt = int(lr[le, s] >> 32), int(lr[le, s] & 0xFFFFFFFF)
+                if zero_copy:
+                    states[s].combine_staging[q * epr + le, :cnt] = outs[q][le, begin:begin + cnt]
+                else:
+                    states[s].combine_staging[q * epr + le, :cnt] = back[le, s, :cnt]
     for rank in range(r):
         st = states[rank]
         out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
         out.view(torch.int16).fill_(0x7FC0)
         topk, w = topk_all[rank].cuda(), w_all[rank].cuda()
-        st.combine_recv(topk, w, out)
+        if zero_copy:
+            st.combine_send_slots.view(torch.int16).fill_(0x7FC0)
+            st.combine(outs[rank], topk, w, out, zero_copy=True)  # the own experts' rows are read from the outputs
+        else:
+            st.combine_recv(topk, w, out)
         torch.cuda.synchronize()
+        if zero_copy:
+            assert (st.combine_send_slots.view(torch.int16) == 0x7FC0).all()
         wsum = w_all[rank].masked_fill(topk_all[rank] == -1, 0).sum(1, keepdim=True)
         diff = O.calc_diff(x_all[rank].float() * wsum, out.cpu())
         assert not torch.isnan(out.float()).any()
@@ -970,3 +983,26 @@ def test_single_launch_dispatch_past_the_streaming_bound(rt, fmt):
     send_count, pair_slot = O.route(topk_all[rank], e, t)
     assert torch.equal(st.send_count.cpu(), send_count)
     assert torch.equal(st.pair_slot.cpu(), pair_slot)
+
+
+@pytest.mark.parametrize("r,rank,t,h,k,e", [(8, 3, 64, 1024, 6, 64), (8, 3, 1500, 512, 8, 64)],
+                         ids=["one_launch", "large_batch"])
+def test_combine_without_row_return_reduces_the_same(rt, r, rank, t, h, k, e):
+    """NULL send slots (zero copy): the call is the reduce alone; `out` is bit-identical to the full call's
+    and no returned row is written."""
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=91, drop=7)
+    st, world = dispatch_on_gpu(rt, x_all, topk_all, rank, e, t, O.ROW_BF16, one_call=True)
+    y = torch.randn((e // r, r * t, h), generator=torch.Generator().manual_seed(9)).to(torch.bfloat16).cuda()
+    world.combine_from_peers(st, mode=1, seed=5)
+    topk, w = topk_all[rank].cuda(), torch.softmax(w_all[rank], dim=-1).cuda()
+    outs = []
+    for zero_copy in (False, True):
+        st.combine_send_slots.view(torch.int16).fill_(0x7FC0)
+        out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+        out.view(torch.int16).fill_(0x7FC0)
+        st.combine(y, topk, w, out, zero_copy=zero_copy)
+        torch.cuda.synchronize()
+        outs.append(out)
+        touched = bool((st.combine_send_slots.view(torch.int16) != 0x7FC0).any())
+        assert touched != zero_copy
+    assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
