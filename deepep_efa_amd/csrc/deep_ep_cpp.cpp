@@ -7,6 +7,7 @@
 // There is no device code in this file and no CPU fallback: a missing or
 // failing HIP library is an exception.
 #include <torch/extension.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/hip/HIPFunctions.h>
 #include <pybind11/functional.h>
@@ -188,6 +189,7 @@ struct Buffer {
     HostStream comm_stream;
     torch::Tensor nvl_buffer, rdma_buffer, mask_status;
     std::unordered_map<int64_t, torch::Tensor> layout_workspaces;  // one per stream that has run the layout kernel
+    static constexpr size_t kMaxLayoutWorkspaces = 8;
     LowLatencyCache ll;
     std::vector<torch::Tensor> combine_input_buffers;
     int combine_buffer_idx = 0;
@@ -310,8 +312,14 @@ struct Buffer {
             std::max<int64_t>(256, int64_t(deepep_layout_workspace_bytes(num_tokens, num_ranks, num_experts)));
         // the kernel's scratch belongs to the stream the kernel runs on: a call on the buffer's own stream and
         // one on the caller's stream may be in flight together
+        if (layout_workspaces.size() >= kMaxLayoutWorkspaces and layout_workspaces.count(int64_t(work_stream.id())) == 0)
+            layout_workspaces.clear();  // a caller cycling through streams does not grow the table without bound
         torch::Tensor& layout_workspace = layout_workspaces[int64_t(work_stream.id())];
         if (!layout_workspace.defined() or layout_workspace.numel() < ws_bytes) {
+            // allocated with the kernel's stream current, so that the caching allocator ties the block to that
+            // stream: a block dropped here (replaced, or the table cleared) is handed out again only to
+            // allocations ordered behind the kernels that used it
+            c10::hip::HIPStreamGuardMasqueradingAsCUDA on_work_stream(work_stream.unwrap());
             layout_workspace = torch::empty({ws_bytes}, torch::dtype(torch::kUInt8).device(torch::kCUDA));
         }
 

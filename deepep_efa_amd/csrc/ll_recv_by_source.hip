@@ -194,6 +194,12 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
         num_chunks = 1 << 30;  // until the source's records end
     }
     lds_barrier();
+    // a pair holds at most max_tokens rows, like a segment of the staged form (whose counts the staged
+    // receive clamps the same way): rows past that are dropped below, so that an expert's ranges never
+    // exceed its num_ranks * max_tokens packed slots whatever the slots and tails hold
+    for (int q = tid; q < num_segments; q += kBySourceThreads)
+        if (pair_prefix[q] > max_tokens) pair_prefix[q] = max_tokens;
+    lds_barrier();
     block_exclusive_scan(pair_prefix, num_segments, scan_tmp);
     if (blockIdx.x == 0) {
         // csrc/kernels/efa_kernels.cu:991-1010: begin = rows of the lower source ranks, 0 where the count is 0
@@ -242,13 +248,12 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
             int pos = running[e] + before_in_wave;
             for (int w2 = 0; w2 < w; ++w2) pos += wave_cnt[w2 * num_local_experts + e];
             const int64_t pair_begin = pair_prefix[e * num_ranks + s] - pair_prefix[e * num_ranks];
-            RowDesc d;
-            d.src_row = -1, d.dst_row = 0;  // a row past its expert's slots is not copied
-            if (pair_begin + pos < slots_per_expert) {
+            if (pos < max_tokens) {  // a row past its pair's max_tokens rows has no place and no descriptor
+                RowDesc d;
                 d.src_row = int32_t(offset);
                 d.dst_row = int32_t(int64_t(e) * slots_per_expert + pair_begin + pos);
+                desc[pair_prefix[e * num_ranks + s] + pos] = d;
             }
-            desc[pair_prefix[e * num_ranks + s] + pos] = d;
         }
         if constexpr (kChunked) break;  // one chunk per workgroup
         lds_barrier();

@@ -38,6 +38,11 @@ generative on CUDA RNG streams that cannot be replayed here):
 * ``ll_exchange_metadata`` — the reference's host loops restated loop for loop; pinned by the
   hand-derived two-rank world (``tests/golden/ll_tiny_world.json``) and by the identities that tie it to
   the dispatch (recv_counts = row sums of the receiver's ``recv_count``; records = a running index).
+* ``ll_send_by_dest``, ``ll_record_packed_rows``, ``ll_combine_send_by_dest``, ``ll_combine_recv_flat_rows`` — the
+  hand-derived two-rank world (``tests/golden/ll_tiny_world.json``: message order, per-record packed rows,
+  the flat buffers of both directions) and, on hypothesis-drawn tiny worlds, the round trip through literal
+  message copies: with identity experts every pair must get back exactly the row its token sent, and the
+  per-record rows must point at what ``ll_dispatch`` put there.
 * ``get_low_latency_rdma_size_hint`` — hand-computed values.
 * ``round_scale`` scales — the reference computes ``exp2(ceil(log2(s)))`` in float32
   (``deep_ep/buffer.py:1601``, ``csrc/kernels/efa_kernels.cu:158``); this oracle (and the kernel)
@@ -438,6 +443,118 @@ def staged_rows(x: torch.Tensor, topk_idx: torch.Tensor, src_rank: int, num_expe
     experts = topk_idx[tok, kk]
     slots = pair_slot[tok, kk].to(torch.int64)
     return send_count, pair_slot, experts, slots, rows
+
+
+# ----------------------------------------------------------------------------
+# Low-latency path over an all-to-all shaped transport: one contiguous message per peer in both
+# directions (deep_ep/buffer.py:2266-2301 dispatch, :2601-2608 and :2735 combine)
+# ----------------------------------------------------------------------------
+def ll_send_by_dest(x: torch.Tensor, topk_idx: torch.Tensor, src_rank: int, num_experts: int, max_tokens: int,
+                    fmt: int, num_ranks: int):
+    """The rows one rank sends, as ONE buffer that is contiguous per destination rank.
+
+    csrc/kernels/efa_kernels.cu:2332-2400 (ll_dispatch_route_and_pack_v3): send_counts[r] = pairs whose
+    expert lives on rank r, send_cumsum = their exclusive prefix (int64, [R] = total), rows grouped by
+    destination rank in send_cumsum order, every row ending in its [token, local expert] (:797-800).
+    Inside one destination's message the reference's live kernel leaves the order to an atomic
+    (rank_write_pos, :2378-2380); this build's order is by expert, then by the pair's slot (ascending
+    (token, k) inside an expert), i.e. the per-expert send slots laid end to end.  A row's place is then
+    send_expert_prefix[expert] + pair_slot, with send_expert_prefix the exclusive prefix of send_count.
+    Returns dict(send_count i32 [E], send_expert_prefix i32 [E+1], send_counts i32 [R], send_cumsum i64 [R+1],
+    pair_slot i32 [T, K], pair_send_row i32 [T, K] (-1 = not sent), rows u8 [P, stride]).
+    """
+    epr = num_experts // num_ranks
+    send_count, pair_slot, experts, slots, rows = staged_rows(x, topk_idx, src_rank, num_experts, max_tokens, fmt,
+                                                              num_ranks)
+    prefix = torch.zeros(num_experts + 1, dtype=torch.int64)
+    prefix[1:] = torch.cumsum(send_count.to(torch.int64), 0)
+    place = prefix[experts] + slots
+    out = torch.zeros_like(rows)
+    out[place] = rows
+    pair_send_row = torch.full(topk_idx.shape, -1, dtype=torch.int32)
+    tok, kk = torch.nonzero(pair_slot >= 0, as_tuple=True)
+    pair_send_row[tok, kk] = place.to(torch.int32)
+    send_counts = send_count.view(num_ranks, epr).sum(1).to(torch.int32)
+    return dict(send_count=send_count, send_expert_prefix=prefix.to(torch.int32), send_counts=send_counts,
+                send_cumsum=prefix[::epr].clone(), pair_slot=pair_slot, pair_send_row=pair_send_row, rows=out)
+
+
+def ll_record_packed_rows(all_topk_idx, rank: int, num_experts: int, max_tokens: int):
+    """For every row rank `rank` receives, in arrival order (source ranks ascending, inside a source the
+    order of that source's message, ll_send_by_dest): the packed row the receive side gives it,
+    local_expert * N + begin(expert, source) + its place among that pair's rows, N = R * max_tokens.
+
+    This is the per-row bookkeeping the reference's receive kernel leaves for the combine:
+    recv_expert_ids / recv_expert_pos of ll_recv_unpack_v2 (csrc/kernels/efa_kernels.cu:2121-2231,
+    scatter :1227-1389), which deep_ep/buffer.py:2601 uses as x[recv_expert_ids, recv_expert_pos].
+    Literal loops; returns int64 [rows received].
+    """
+    r = len(all_topk_idx)
+    epr = num_experts // r
+    n = max_tokens * r
+    cnt = [[0] * r for _ in range(epr)]
+    per_source = []
+    for s in range(r):
+        send_count, pair_slot = route(all_topk_idx[s], num_experts, max_tokens)
+        msg = []  # (local expert, slot) in message order: expert by expert, slots ascending
+        for le in range(epr):
+            c = int(send_count[rank * epr + le])
+            cnt[le][s] = c
+            msg += [(le, j) for j in range(c)]
+        per_source.append(msg)
+    out = []
+    for s in range(r):
+        for le, j in per_source[s]:
+            begin = sum(cnt[le][:s])
+            out.append(le * n + begin + j)
+    return torch.tensor(out, dtype=torch.int64)
+
+
+def ll_combine_send_by_dest(y: torch.Tensor, record_packed_row: torch.Tensor, padded_index: torch.Tensor,
+                            combine_send_offset: torch.Tensor) -> torch.Tensor:
+    """The expert outputs owed to the other ranks as one flat [Rv, H] buffer in arrival order, which is
+    contiguous per destination rank: flat[combine_send_offset[i]] = y_rows[record_packed_row[padded_index[i]]].
+
+    deep_ep/buffer.py:2601-2608 (x[recv_expert_ids, recv_expert_pos] un-sorted to arrival order) and
+    csrc/kernels/coop_combine_send.cuh:37-170 (send_buffer[combine_send_offset[i]] = expert_x[padded_index[i]]).
+    y [E_l, N, H] bf16.  Records whose row is -1 leave their flat row zero.
+    """
+    h = y.shape[-1]
+    rows = y.reshape(-1, h)
+    n = combine_send_offset.numel()
+    flat = torch.zeros((n, h), dtype=y.dtype)
+    for i in range(n):
+        src = int(record_packed_row[int(padded_index[i])])
+        if src >= 0:
+            flat[int(combine_send_offset[i])] = rows[src]
+    return flat
+
+
+def ll_combine_recv_flat_rows(recv_flat: torch.Tensor, slot_rows: int, send_expert_prefix: torch.Tensor,
+                              topk_idx: torch.Tensor, pair_slot: torch.Tensor, experts_per_rank: int):
+    """pair_rows[t, k] = the row of the returned buffer that answers pair (t, k), and which pairs are live.
+
+    The buffer holds one row per row sent, in send order (ll_send_by_dest), either flat (slot_rows == 0) or
+    with the rows from rank r starting at row r * slot_rows: csrc/kernels/efa_kernels.cu:1449-1466 (src_rank
+    from send_cumsum, within_rank = send_idx - send_cumsum[src_rank], byte offset src_rank * slot_size +
+    within_rank * hidden * 2, or send_idx * hidden when flat).
+    """
+    t, k = topk_idx.shape
+    h = recv_flat.shape[-1]
+    live = pair_slot >= 0
+    pair_rows = torch.zeros((t, k, h), dtype=recv_flat.dtype)
+    for ti in range(t):
+        for ki in range(k):
+            if not live[ti, ki]:
+                continue
+            e = int(topk_idx[ti, ki])
+            send_idx = int(send_expert_prefix[e]) + int(pair_slot[ti, ki])
+            if slot_rows > 0:
+                src_rank = e // experts_per_rank
+                within = send_idx - int(send_expert_prefix[src_rank * experts_per_rank])
+                send_idx = src_rank * slot_rows + within
+            pair_rows[ti, ki] = recv_flat[send_idx]
+    return pair_rows, live
 
 
 # ----------------------------------------------------------------------------

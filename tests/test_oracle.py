@@ -567,3 +567,39 @@ def test_round_scale_has_one_answer_for_every_bf16_amax():
     want = np.exp2(np.ceil(exact)).astype(np.float32)
     assert np.array_equal(O.pow2_ceil(s).numpy(), want)
     assert torch.equal(torch.exp2(torch.ceil(torch.log2(s))), O.pow2_ceil(s))
+
+
+@pytest.mark.parametrize("rank", [0, 1])
+def test_oracle_all_to_all_surface_against_the_hand_derived_world(rank):
+    """Message order, per-record packed rows and the flat buffers of both directions, against values worked
+    out on paper (tests/golden/ll_tiny_world.json)."""
+    g, x_all, topk_all = load_tiny_world()
+    e, m, h, r = g["num_experts"], g["max_tokens"], g["hidden"], g["num_ranks"]
+    want = g["send_by_dest"][f"rank{rank}"]
+    got = O.ll_send_by_dest(x_all[rank], topk_all[rank], rank, e, m, O.ROW_BF16, r)
+    assert got["send_expert_prefix"].tolist() == want["send_expert_prefix"]
+    assert got["send_counts"].tolist() == want["send_counts"]
+    assert got["send_cumsum"].tolist() == want["send_cumsum"]
+    assert got["pair_send_row"].tolist() == want["pair_send_row"]
+    tail_at = O.row_payload(h, O.ROW_BF16) - 16
+    tails = got["rows"][:, tail_at:tail_at + 16].contiguous().view(torch.int32)
+    assert tails[:, 0].tolist() == want["row_token"] and tails[:, 1].tolist() == want["row_topk_slot"]
+    assert tails[:, 2].tolist() == [rank] * len(want["row_token"]) and tails[:, 3].tolist() == want["row_local_expert"]
+    values = got["rows"][:, :2 * h].contiguous().view(torch.bfloat16).float()
+    assert torch.equal(values, torch.tensor([g["x_value"][rank][t] for t in want["row_token"]],
+                                            dtype=torch.float32).view(-1, 1).expand(-1, h))
+    rec = O.ll_record_packed_rows(topk_all, rank, e, m)
+    assert rec.tolist() == g["record_packed_row"][f"rank{rank}"]
+    meta = g["exchange_metadata"][f"rank{rank}"]
+    packed = O.ll_dispatch(x_all, topk_all, rank, e, m, O.ROW_BF16)
+    y = packed["packed_recv_x"].view(e // r, r * m, 2 * h).contiguous().view(torch.bfloat16)
+    flat = O.ll_combine_send_by_dest(y, rec, torch.tensor(meta["padded_index"]), torch.tensor(meta["combine_send_offset"]))
+    assert flat.float()[:, 0].tolist() == g["combine_send_flat_identity_experts"][f"rank{rank}"]
+    assert (flat.float() == flat.float()[:, :1]).all()
+    if rank == 0:
+        back = torch.tensor(g["combine_recv_flat_rank0_identity_experts"], dtype=torch.float32).view(-1, 1).expand(-1, h)
+        pair_rows, live = O.ll_combine_recv_flat_rows(back.to(torch.bfloat16), 0, got["send_expert_prefix"], topk_all[0],
+                                                      got["pair_slot"], e // r)
+        w = torch.tensor(g["topk_weights_rank0"], dtype=torch.float32)
+        out = O.ll_combine_f32_chain(pair_rows, w, live)
+        assert out.float()[:, 0].tolist() == g["combine_rank0_identity_experts"]

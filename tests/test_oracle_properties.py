@@ -129,3 +129,61 @@ def test_exchange_metadata_matches_the_dispatch(w):
     epr = e // r
     assert meta["send_counts"].tolist() == [int(routed[rank, d * epr:(d + 1) * epr].sum()) for d in range(r)]
     assert meta["source_rank"].tolist() == [s for s in range(r) for _ in range(int(per_source[s]))]
+
+
+@settings(max_examples=60, deadline=None)
+@given(worlds())
+def test_all_to_all_round_trip_returns_every_pair_its_own_row(w):
+    """Both directions over one contiguous message per peer, the messages moved by literal slice copies:
+    the per-record packed rows must point at what the dispatch put there, and with identity experts every
+    live pair must get back exactly the row its token sent."""
+    r, e, k, t, m, _, x_all, topk_all = w
+    epr, h = e // r, 128
+    sent = [O.ll_send_by_dest(x_all[s], topk_all[s], s, e, m, O.ROW_BF16, r) for s in range(r)]
+    routed = torch.stack([sd["send_count"] for sd in sent]).to(torch.int32)
+    flats, metas = [], []
+    for d in range(r):
+        # the message of source s to rank d, and where its rows land in arrival order
+        arrived = torch.cat([sent[s]["rows"][int(sent[s]["send_cumsum"][d]):int(sent[s]["send_cumsum"][d + 1])]
+                             for s in range(r)]) if r else None
+        meta = O.ll_exchange_metadata(routed, d, m)
+        assert meta["total_recv"] == arrived.shape[0]
+        packed = O.ll_dispatch(x_all, topk_all, d, e, m, O.ROW_BF16)
+        rec = O.ll_record_packed_rows(topk_all, d, e, m)
+        assert rec.numel() == arrived.shape[0]
+        px = packed["packed_recv_x"].view(epr * r * m, -1)
+        tail_at = O.row_payload(h, O.ROW_BF16) - 16
+        for i in range(rec.numel()):
+            assert torch.equal(px[int(rec[i])], arrived[i, :2 * h])  # the record's row is where the dispatch put it
+            tail = arrived[i, tail_at:tail_at + 16].contiguous().view(torch.int32)
+            assert int(rec[i]) // (r * m) == int(tail[3])  # ... inside the expert its tail names
+            assert int(packed["packed_recv_src_info"].view(-1)[int(rec[i])]) == int(tail[0])
+        y = packed["packed_recv_x"].view(epr, r * m, 2 * h).contiguous().view(torch.bfloat16)  # identity experts
+        flats.append(O.ll_combine_send_by_dest(y, rec, meta["padded_index"], meta["combine_send_offset"]))
+        metas.append(meta)
+    for s in range(r):
+        # the answers for rank s: peer d's rows for source s, landing behind what s sent to the ranks below d
+        total = int(sent[s]["send_cumsum"][r])
+        back = torch.zeros((total, h), dtype=torch.bfloat16)
+        for d in range(r):
+            first = int(metas[d]["recv_counts"][:s].sum())
+            n = int(metas[d]["recv_counts"][s])
+            at = int(metas[d]["combine_remote_recv_offset"][s])
+            assert at == int(sent[s]["send_cumsum"][d]) and n == int(sent[s]["send_counts"][d])
+            back[at:at + n] = flats[d][first:first + n]
+        pair_rows, live = O.ll_combine_recv_flat_rows(back, 0, sent[s]["send_expert_prefix"], topk_all[s],
+                                                      sent[s]["pair_slot"], epr)
+        assert torch.equal(live, sent[s]["pair_slot"] >= 0)
+        for i in range(t):
+            for j in range(k):
+                if live[i, j]:
+                    assert torch.equal(pair_rows[i, j], x_all[s][i])
+        # the slotted form of the same buffer: rank d's answers start at row d * slot_rows
+        slot_rows = m * epr
+        slotted = torch.zeros((r * slot_rows, h), dtype=torch.bfloat16)
+        for d in range(r):
+            lo, hi = int(sent[s]["send_cumsum"][d]), int(sent[s]["send_cumsum"][d + 1])
+            slotted[d * slot_rows:d * slot_rows + hi - lo] = back[lo:hi]
+        again, _ = O.ll_combine_recv_flat_rows(slotted, slot_rows, sent[s]["send_expert_prefix"], topk_all[s],
+                                               sent[s]["pair_slot"], epr)
+        assert torch.equal(again, pair_rows)
