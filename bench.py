@@ -56,6 +56,27 @@ def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0, packed=None):
     }
 
 
+def load_bench_probe():
+    """The measuring-stick kernels (bench_probe.hip beside this file, a library of its own: nothing of it is in
+    libdeepep_hip.so).  Built by __graft_entry__.build(); built here only if that has not happened."""
+    import ctypes
+    path = os.path.join(ROOT, "bench_probe.so")
+    if not os.path.exists(path):
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("deepep_build", os.path.join(ROOT, "deepep_efa_amd", "build.py"))
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        mod.build_bench_probe()
+    lib = ctypes.CDLL(path)
+    c = ctypes
+    lib.bench_probe_row_scatter.restype = c.c_int
+    lib.bench_probe_row_scatter.argtypes = [c.c_void_p, c.c_int, c.c_int, c.c_void_p, c.c_int, c.c_void_p, c.c_int64,
+                                            c.c_void_p]
+    lib.bench_probe_stream_copy.restype = c.c_int
+    lib.bench_probe_stream_copy.argtypes = [c.c_void_p, c.c_void_p, c.c_int64, c.c_void_p]
+    return lib
+
+
 def time_calls(torch, fn, n):
     for _ in range(3):
         fn()
@@ -67,6 +88,40 @@ def time_calls(torch, fn, n):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / n
+
+
+def time_graph_samples(torch, fn, warmup, steps, samples=10):
+    """`fn` enqueued by HIP-graph replays so that the GPU never waits for the host: the time is the stream's,
+    kernels plus the gaps between them.  The graph holds a whole multiple of `steps` calls, at least 20 (a
+    graph of one 16 us step would mostly measure the events around it); a sample is as many back-to-back
+    replays as make about 100 calls, between its own pair of events; `samples` of them are taken whatever
+    `steps` is.  Returns the median per call with the fastest and slowest sample beside it, so the figure does
+    not depend on how many steps were asked for."""
+    per_graph = steps * max(1, -(-20 // steps))
+    replays = max(1, 100 // per_graph)
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(g):
+        for _ in range(per_graph):
+            fn()
+    for _ in range(max(1, -(-warmup // per_graph))):
+        g.replay()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(samples)]
+    for e0, e1 in events:
+        e0.record()
+        for _ in range(replays):
+            g.replay()
+        e1.record()
+    torch.cuda.synchronize()
+    per_call = sorted(e0.elapsed_time(e1) * 1e3 / (replays * per_graph) for e0, e1 in events)
+    del g
+    return {"us": per_call[len(per_call) // 2], "min_us": per_call[0], "max_us": per_call[-1],
+            "calls_per_graph": per_graph, "replays_per_sample": replays, "samples": samples}
 
 
 def rotating(fns):
@@ -161,7 +216,7 @@ def by_source_receive(torch, _capi, lib, ll_runtime, st, world):
             _capi.ptr(meta["num_recv_tokens"]), rows, sh.hidden, e, r, m, sh.fmt, _capi.ptr(st.packed_recv_x),
             _capi.ptr(st.packed_recv_scales), _capi.ptr(st.packed_recv_src_info),
             _capi.ptr(st.packed_recv_layout_range), _capi.ptr(st.packed_recv_count), None,
-            _capi.ptr(tokens_per_expert), _capi.ptr(ws), ws.numel(), torch.cuda.current_stream().cuda_stream))
+            _capi.ptr(tokens_per_expert), None, _capi.ptr(ws), ws.numel(), torch.cuda.current_stream().cuda_stream))
     return call, rows
 
 
@@ -180,6 +235,7 @@ def bench_pack(torch, _capi, lib, loopback, args):
     counts, cumsum = torch.empty(r, **i32), torch.empty(r + 1, dtype=torch.int64, device="cuda")
     ws2 = torch.empty(max(256, lib.deepep_routing_sort_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
     cpm = torch.empty((r, 10), **i32)
+    row_of_pair = torch.empty((t, r), **i32)  # the sort's inverse table: with it the combine reduce is one launch
 
     def layout():
         _capi.check(lib.deepep_get_dispatch_layout(_capi.ptr(topk), t, k, r, e, _capi.ptr(per_rank), None,
@@ -188,7 +244,8 @@ def bench_pack(torch, _capi, lib, loopback, args):
 
     def sort():
         _capi.check(lib.deepep_moe_routing_sort(_capi.ptr(is_in), t, r, _capi.ptr(ids), _capi.ptr(counts),
-                                                _capi.ptr(cumsum), _capi.ptr(ws2), ws2.numel(), stream))
+                                                _capi.ptr(cumsum), _capi.ptr(row_of_pair), _capi.ptr(ws2), ws2.numel(),
+                                                stream))
 
     def prefix():
         _capi.check(lib.deepep_channel_prefix_matrix(_capi.ptr(is_in), t, r, 10, _capi.ptr(cpm), stream))
@@ -253,9 +310,15 @@ def bench_pack(torch, _capi, lib, loopback, args):
     def reduce_on(i):
         return lambda: _capi.check(lib.deepep_combine_reduce(
             _capi.ptr(out16s[i]), _capi.ptr(remap_w), _capi.ptr(ids), _capi.ptr(cumsum), _capi.ptr(is_in), None, None,
-            t, h, k, r, s, _capi.ptr(comb_xs[i]), _capi.ptr(comb_w), _capi.ptr(ws3), ws3.numel(), stream))
+            t, h, k, r, s, _capi.ptr(row_of_pair), _capi.ptr(comb_xs[i]), _capi.ptr(comb_w), None, 0, stream))
+
+    def reduce_from_list_on(i):  # without the sort's table: the positions are rebuilt from the list first
+        return lambda: _capi.check(lib.deepep_combine_reduce(
+            _capi.ptr(out16s[i]), _capi.ptr(remap_w), _capi.ptr(ids), _capi.ptr(cumsum), _capi.ptr(is_in), None, None,
+            t, h, k, r, s, None, _capi.ptr(comb_xs[i]), _capi.ptr(comb_w), _capi.ptr(ws3), ws3.numel(), stream))
 
     reduce = rotating([reduce_on(i) for i in range(2)])
+    reduce_from_list = rotating([reduce_from_list_on(i) for i in range(2)])
 
     n = max(10, args.steps // 4)
     res = {"workload": "4096 tokens x 7168 bf16, top-8 of 256 experts, 8 ranks x 32 experts", "rows_packed": s,
@@ -269,7 +332,9 @@ def bench_pack(torch, _capi, lib, loopback, args):
                              ("pack_fp8", pack_fp8, s * (h + h // 32) * 2 + s * 8),
                              ("topk_remap", remap, s * 8 + s * k * 12 * 2),
                              ("recv_src_meta", src_meta, s * 8),
-                             ("combine_reduce", reduce, s * 2 * h + s * k * 4 + s * 12 + t * r + t * 2 * h + t * k * 4)):
+                             ("combine_reduce", reduce, s * 2 * h + s * k * 4 + t * r * 5 + t * 2 * h + t * k * 4),
+                             ("combine_reduce_from_the_list", reduce_from_list,
+                              s * 2 * h + s * k * 4 + s * 12 + t * r + t * 2 * h + t * k * 4)):
         us = time_calls(torch, fn, n)
         res[name] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
                      "frac_of_8TBps": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
@@ -348,8 +413,16 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
     slot = st.pair_slot[:t].long()
     dst_rows = torch.where(slot >= 0, topk.clamp(min=0) * st.shape.max_tokens + slot, torch.full_like(slot, -1))
     dst_rows = dst_rows.to(torch.int32).contiguous()
-    probe = on_every_state(lambda s_, x_: lambda: _capi.check(lib.deepep_probe_row_scatter(
-        _capi.ptr(x_), t, h, _capi.ptr(dst_rows), k, _capi.ptr(s_.send_slots), s_.stride, stream)))
+    probe_lib = load_bench_probe()
+
+    def probe_on(s_, x_):
+        def call():
+            rc = probe_lib.bench_probe_row_scatter(_capi.ptr(x_), t, h, _capi.ptr(dst_rows), k, _capi.ptr(s_.send_slots),
+                                                   s_.stride, stream)
+            assert rc == 0, rc
+        return call
+
+    probe = on_every_state(probe_on)
     if skewed:
         samples = sorted(time_calls(torch, probe, 1) for _ in range(6))
         us = samples[len(samples) // 2]
@@ -404,40 +477,9 @@ def bench_api_step(torch, args):
            "eager_host_wall_us": round((time.perf_counter() - wall0) * 1e6 / args.steps, 2), "graph_us": None}
     if not args.no_graph:
         try:
-            per_graph = max(d for d in range(1, 26) if args.steps % d == 0)
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                step()
-            torch.cuda.current_stream().wait_stream(side)
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                for _ in range(per_graph):
-                    step()
-            for _ in range(max(1, args.warmup // per_graph)):
-                g.replay()
-            torch.cuda.synchronize()
-            ev0.record()
-            for _ in range(args.steps // per_graph):
-                g.replay()
-            ev1.record()
-            torch.cuda.synchronize()
-            res["graph_us"] = round(ev0.elapsed_time(ev1) * 1e3 / args.steps, 2)
-            del g
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                for _ in range(per_graph):
-                    step(zero_copy=True)
-            for _ in range(max(1, args.warmup // per_graph)):
-                g.replay()
-            torch.cuda.synchronize()
-            ev0.record()
-            for _ in range(args.steps // per_graph):
-                g.replay()
-            ev1.record()
-            torch.cuda.synchronize()
-            res["graph_zero_copy_us"] = round(ev0.elapsed_time(ev1) * 1e3 / args.steps, 2)
-            del g
+            res["graph_us"] = round(time_graph_samples(torch, step, args.warmup, args.steps)["us"], 2)
+            res["graph_zero_copy_us"] = round(
+                time_graph_samples(torch, lambda: step(zero_copy=True), args.warmup, args.steps)["us"], 2)
         except Exception as exc:
             res["graph_us"] = None
             res["graph_error"] = type(exc).__name__
@@ -584,29 +626,6 @@ def main():
         torch.cuda.synchronize()
         return ev0.elapsed_time(ev1) * 1e3 / reps, (time.perf_counter() - wall0) * 1e6 / reps
 
-    def time_graph(fn, warmup, reps):
-        """The same `reps` calls, enqueued by HIP-graph replays of `per_graph` calls each, so that the
-        GPU never waits for the host: the time is the stream's, kernels plus the gaps between them."""
-        per_graph = max(d for d in range(1, 26) if reps % d == 0)
-        g = torch.cuda.CUDAGraph()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            fn()
-        torch.cuda.current_stream().wait_stream(side)
-        with torch.cuda.graph(g):
-            for _ in range(per_graph):
-                fn()
-        for _ in range(max(1, warmup // per_graph)):
-            g.replay()
-        torch.cuda.synchronize()
-        ev0.record()
-        for _ in range(reps // per_graph):
-            g.replay()
-        ev1.record()
-        torch.cuda.synchronize()
-        return ev0.elapsed_time(ev1) * 1e3 / reps, per_graph
-
     flush = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
 
     def time_cold(fn, reps=40, by_reads=False):
@@ -669,16 +688,21 @@ def main():
 
     eager_us, host_wall_us = time_eager(step, args.warmup, args.steps)
     eager_phase_us, _ = time_eager(step_by_phase, 10, args.steps)
-    graph_us = graph_phase_us = per_graph = None
-    per_call = {}
+    graph_us = graph_phase_us = step_samples = None
+    per_call, per_call_spread = {}, {}
     timing = "eager launches"
     if not args.no_graph:
         try:
-            graph_us, per_graph = time_graph(step, args.warmup, args.steps)
-            graph_phase_us, _ = time_graph(step_by_phase, 10, args.steps)
+            step_samples = time_graph_samples(torch, step, args.warmup, args.steps)
+            graph_us = step_samples["us"]
+            graph_phase_us = time_graph_samples(torch, step_by_phase, 10, args.steps)["us"]
             for name, fn in calls.items():
-                per_call[name], _ = time_graph(fn, 10, args.steps)
-            timing = f"HIP graphs of {per_graph} steps each, replayed back to back"
+                got = time_graph_samples(torch, fn, 10, args.steps)
+                per_call[name] = got["us"]
+                per_call_spread[name] = [round(got["min_us"], 2), round(got["max_us"], 2)]
+            timing = (f"HIP graphs of {step_samples['calls_per_graph']} steps each; median of "
+                      f"{step_samples['samples']} samples of {step_samples['replays_per_sample']} back-to-back "
+                      "replays, whatever --steps is")
         except Exception as exc:  # fall back to eager timing, and say so
             graph_us = None
             timing = f"eager launches (graph capture unavailable: {type(exc).__name__})"
@@ -700,6 +724,8 @@ def main():
     nbytes = algorithmic_bytes(t, h, k, p, rv, st.payload_bytes, e, r, own, packed=st.data_bytes + st.scale_bytes + 4)
     kernels = {n: {"us": round(per_call[n], 2), "bytes": nbytes[n],
                    "GBps": round(nbytes[n] / per_call[n] / 1e3, 1)} for n in calls}
+    for n, spread in per_call_spread.items():
+        kernels[n]["us_min_max"] = spread
     dom = max(step_calls, key=per_call.get)
     stamp = build_stamp(lib)
     warm = nbytes[dom] / per_call[dom] / 1e3
@@ -725,6 +751,8 @@ def main():
     result = {
         "metric": "us per LL dispatch+combine (128 tok,7168,top-8); pack/combine HBM GB/s",
         "value": round(us_per_step, 2),
+        "value_min_max": ([round(step_samples["min_us"], 2), round(step_samples["max_us"], 2)]
+                          if step_samples is not None else None),
         "unit": "us",
         "n_gpus": 1,
         "steps": args.steps,

@@ -24,7 +24,7 @@ PROTOTYPES = {
     "deepep_layout_workspace_bytes": (_SZ, [_I, _I, _I]),
     "deepep_get_dispatch_layout": (_I, [_VP, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "deepep_routing_sort_workspace_bytes": (_SZ, [_I, _I]),
-    "deepep_moe_routing_sort": (_I, [_VP, _I, _I, _VP, _VP, _VP, _VP, _SZ, _VP]),
+    "deepep_moe_routing_sort": (_I, [_VP, _I, _I, _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "deepep_channel_prefix_matrix": (_I, [_VP, _I, _I, _I, _VP, _VP]),
     "deepep_pack_rows": (_I, [_VP, _VP, _VP, _VP, _I64, _I, _I, _I, _VP, _VP, _VP]),
     "deepep_per_token_cast_to_fp8": (_I, [_VP, _I, _I, _I, _VP, _VP, _VP]),
@@ -45,12 +45,17 @@ PROTOTYPES = {
     "deepep_ll_exchange_metadata": (_I, [_VP, _I, _I, _I, _I, _I64] + [_VP] * 11),
     "deepep_ll_by_source_workspace_bytes": (_SZ, [_I, _I64]),
     "deepep_ll_dispatch_recv_by_source": (_I, [_VP, _I64, _VP, _VP, _VP, _I64, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP,
-                                               _VP, _VP, _VP, _VP, _SZ, _VP]),
+                                               _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
+    "deepep_ll_dispatch_send_by_dest": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _I64, _VP, _VP, _VP, _VP,
+                                             _VP, _VP, _SZ, _VP]),
+    "deepep_ll_combine_send_by_dest": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _I64, _I, _I, _I, _I, _VP, _VP, _VP, _VP,
+                                            _VP, _VP]),
+    "deepep_ll_combine_recv_flat": (_I, [_VP, _I64, _I64, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _VP]),
     "deepep_combine_reduce_workspace_bytes": (_SZ, [_I, _I]),
-    "deepep_combine_reduce": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP, _SZ, _VP]),
+    "deepep_combine_reduce": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP, _VP, _SZ,
+                                   _VP]),
     "deepep_synth_topk_idx": (_I, [_VP, _VP, _I, _I, _I, _I, _U32, _VP, _VP]),
     "deepep_synth_bf16_rows": (_I, [_VP, _I64, _I, _I64, _VP, _U32, _U32, _I, _VP]),
-    "deepep_probe_row_scatter": (_I, [_VP, _I, _I, _VP, _I, _VP, _I64, _VP]),
     "deepep_loopback_dispatch_from_peers": (_I, [_VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _SZ,
                                                _VP]),
     "deepep_loopback_combine_from_peers": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _U32, _VP, _VP]),

@@ -29,6 +29,23 @@ def build_hip_library(verbose: bool = True) -> str:
     return LIB
 
 
+BENCH_PROBE_SRC = os.path.join(os.path.dirname(HERE), "bench_probe.hip")
+BENCH_PROBE = os.path.join(os.path.dirname(HERE), "bench_probe.so")
+
+
+def build_bench_probe(verbose: bool = True) -> str:
+    """Builds the measuring-stick kernels bench.py times beside the library's own (bench_probe.hip beside
+    bench.py -> bench_probe.so).  They are not part of libdeepep_hip.so."""
+    cmd = ["hipcc"] + FLAGS + [f"-I{os.path.dirname(HERE)}", BENCH_PROBE_SRC, "-o", BENCH_PROBE]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if verbose and out.strip():
+        print(out, file=sys.stderr)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    return BENCH_PROBE
+
+
 HOST_MODULE = os.path.join(HERE, "deep_ep_cpp.so")
 
 
@@ -57,3 +74,4 @@ def build_host_module(verbose: bool = True) -> str:
 if __name__ == "__main__":
     print(build_hip_library())
     print(build_host_module())
+    print(build_bench_probe())

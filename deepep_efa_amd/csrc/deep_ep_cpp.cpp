@@ -670,7 +670,8 @@ static std::tuple<torch::Tensor, torch::Tensor> per_token_cast_to_fp8(const torc
 }
 
 // reference: csrc/kernels/efa_kernels.cu:1591-1651 (the .item() host sync is the reference's)
-static std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, int64_t> moe_routing_sort(const torch::Tensor& is_token_in_rank) {
+static std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, int64_t, torch::Tensor> routing_sort_impl(
+    const torch::Tensor& is_token_in_rank, bool with_positions) {
     EP_HOST_ASSERT(is_token_in_rank.dim() == 2);
     EP_HOST_ASSERT(is_token_in_rank.scalar_type() == torch::kBool);
     EP_HOST_ASSERT(is_token_in_rank.is_contiguous());
@@ -682,11 +683,27 @@ static std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, int64_t> moe_rout
     auto ids = torch::empty({std::max<int64_t>(1, int64_t(num_tokens) * num_ranks)}, torch::dtype(torch::kInt64).device(dev));
     auto ws = torch::empty({std::max<int64_t>(256, int64_t(deepep_routing_sort_workspace_bytes(num_tokens, num_ranks)))},
                            torch::dtype(torch::kUInt8).device(dev));
+    torch::Tensor row_of_pair;
+    if (with_positions) row_of_pair = torch::empty({num_tokens, num_ranks}, torch::dtype(torch::kInt32).device(dev));
     abi_check(deepep_moe_routing_sort(reinterpret_cast<const uint8_t*>(is_token_in_rank.data_ptr<bool>()), num_tokens,
                                       num_ranks, ids.data_ptr<int64_t>(), send_counts.data_ptr<int>(),
-                                      send_cumsum.data_ptr<int64_t>(), ws.data_ptr(), size_t(ws.numel()), current_stream()));
+                                      send_cumsum.data_ptr<int64_t>(),
+                                      with_positions and num_tokens > 0 ? row_of_pair.data_ptr<int>() : nullptr,
+                                      ws.data_ptr(), size_t(ws.numel()), current_stream()));
     const int64_t total = send_cumsum.select(0, num_ranks).item<int64_t>();
-    return {ids.slice(0, 0, total), send_counts, send_cumsum, total};
+    return {ids.slice(0, 0, total), send_counts, send_cumsum, total, row_of_pair};
+}
+
+static std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, int64_t> moe_routing_sort(const torch::Tensor& is_token_in_rank) {
+    auto [ids, counts, cumsum, total, unused] = routing_sort_impl(is_token_in_rank, false);
+    (void)unused;
+    return {ids, counts, cumsum, total};
+}
+
+// The same plus row_of_pair [T, R] int32, the inverse of the list, which combine_reduce takes to run as one launch.
+static std::tuple<torch::Tensor, torch::Tensor, torch::Tensor, int64_t, torch::Tensor> moe_routing_sort_with_positions(
+    const torch::Tensor& is_token_in_rank) {
+    return routing_sort_impl(is_token_in_rank, true);
 }
 
 // reference: csrc/kernels/intranode.cu:90-112 (the channel part of notify_dispatch)
@@ -770,7 +787,8 @@ ll_exchange_metadata(const torch::Tensor& all_num_routed, int rank, int num_max_
 static std::tuple<torch::Tensor, std::optional<torch::Tensor>> combine_reduce(
     const torch::Tensor& recv_x, const std::optional<torch::Tensor>& recv_topk_weights,
     const torch::Tensor& sorted_token_ids, const torch::Tensor& send_cumsum, const torch::Tensor& is_token_in_rank,
-    const std::optional<torch::Tensor>& bias_0, const std::optional<torch::Tensor>& bias_1) {
+    const std::optional<torch::Tensor>& bias_0, const std::optional<torch::Tensor>& bias_1,
+    const std::optional<torch::Tensor>& row_of_pair) {
     EP_HOST_ASSERT(recv_x.dim() == 2 and recv_x.is_contiguous() and recv_x.is_cuda());
     EP_HOST_ASSERT(recv_x.scalar_type() == torch::kBFloat16);
     EP_HOST_ASSERT(is_token_in_rank.dim() == 2 and is_token_in_rank.is_contiguous());
@@ -792,6 +810,10 @@ static std::tuple<torch::Tensor, std::optional<torch::Tensor>> combine_reduce(
             EP_HOST_ASSERT((*b)->dim() == 2 and (*b)->is_contiguous() and (*b)->scalar_type() == torch::kBFloat16);
             EP_HOST_ASSERT((*b)->size(0) == num_tokens and (*b)->size(1) == hidden);
         }
+    if (row_of_pair.has_value()) {
+        EP_HOST_ASSERT(row_of_pair->scalar_type() == torch::kInt32 and row_of_pair->is_contiguous() and row_of_pair->is_cuda());
+        EP_HOST_ASSERT(row_of_pair->dim() == 2 and row_of_pair->size(0) == num_tokens and row_of_pair->size(1) == num_ranks);
+    }
     auto combined_x = torch::empty({num_tokens, hidden}, recv_x.options());
     std::optional<torch::Tensor> combined_w;
     if (recv_topk_weights.has_value()) combined_w = torch::empty({num_tokens, num_topk}, recv_topk_weights->options());
@@ -802,7 +824,8 @@ static std::tuple<torch::Tensor, std::optional<torch::Tensor>> combine_reduce(
         sorted_token_ids.data_ptr<int64_t>(), send_cumsum.data_ptr<int64_t>(),
         reinterpret_cast<const uint8_t*>(is_token_in_rank.data_ptr<bool>()),
         bias_0.has_value() ? bias_0->data_ptr() : nullptr, bias_1.has_value() ? bias_1->data_ptr() : nullptr, num_tokens,
-        hidden, num_topk, num_ranks, max_rows, combined_x.data_ptr(),
+        hidden, num_topk, num_ranks, max_rows, row_of_pair.has_value() ? row_of_pair->data_ptr<int>() : nullptr,
+        combined_x.data_ptr(),
         combined_w.has_value() ? combined_w->data_ptr<float>() : nullptr, ws.data_ptr(), size_t(ws.numel()),
         current_stream()));
     return {combined_x, combined_w};
@@ -902,11 +925,16 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("per_token_cast_to_fp8", &deep_ep::per_token_cast_to_fp8,
           "Per-token FP8 e4m3 quantisation with 128-channel groups");
     m.def("moe_routing_sort", &deep_ep::moe_routing_sort, "Token ids grouped by destination rank");
+    m.def("moe_routing_sort_with_positions", &deep_ep::moe_routing_sort_with_positions,
+          "moe_routing_sort plus row_of_pair [T, R], the inverse of the list");
     m.def("channel_prefix_matrix", &deep_ep::channel_prefix_matrix, "Per-rank prefix of token counts over channels");
     m.def("pack_rows", &deep_ep::pack_rows, "Gather rows into per-rank contiguous send buffers");
     m.def("topk_remap", &deep_ep::topk_remap, "Top-k of the send rows in the destination rank's expert numbering");
     m.def("build_recv_src_meta", &deep_ep::build_recv_src_meta, "Source-rank metadata of the received rows");
     m.def("ll_exchange_metadata", &deep_ep::ll_exchange_metadata,
           "Send/receive counts, combine offsets and per-row records from the gathered route counts");
-    m.def("combine_reduce", &deep_ep::combine_reduce, "Per-token sum of the rows that came back (normal-mode combine)");
+    m.def("combine_reduce", &deep_ep::combine_reduce, "Per-token sum of the rows that came back (normal-mode combine)",
+          py::arg("recv_x"), py::arg("recv_topk_weights"), py::arg("sorted_token_ids"), py::arg("send_cumsum"),
+          py::arg("is_token_in_rank"), py::arg("bias_0") = py::none(), py::arg("bias_1") = py::none(),
+          py::arg("row_of_pair") = py::none());
 }

@@ -132,7 +132,7 @@ constexpr int kSortChunk = 1024;
 template <bool kScatter>
 __global__ __launch_bounds__(kSortChunk) void routing_sort_pass_kernel(
     const uint8_t* __restrict__ is_token_in_rank, int num_tokens, int num_ranks, int32_t* __restrict__ chunk_table,
-    int64_t* __restrict__ sorted_token_ids) {
+    int64_t* __restrict__ sorted_token_ids, int32_t* __restrict__ row_of_pair) {
     extern __shared__ int32_t wave_cnt[];  // [16][R]
     const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
     const int c = blockIdx.x;
@@ -165,7 +165,9 @@ __global__ __launch_bounds__(kSortChunk) void routing_sort_pass_kernel(
         for (int r = 0; r < num_ranks; ++r) {
             const bool in = t < num_tokens && row[r] != 0;
             const uint64_t votes = __ballot(in);
-            if (in) sorted_token_ids[wave_cnt[w * num_ranks + r] + __popcll(votes & lanes_below(lane))] = t;
+            const int pos = wave_cnt[w * num_ranks + r] + __popcll(votes & lanes_below(lane));
+            if (in) sorted_token_ids[pos] = t;
+            if (row_of_pair != nullptr && t < num_tokens) row_of_pair[int64_t(t) * num_ranks + r] = in ? pos : -1;
         }
     }
 }
@@ -225,7 +227,8 @@ __device__ __forceinline__ uint64_t membership_mask(const uint8_t* row, int num_
 
 __global__ __launch_bounds__(kSortChunk) void routing_sort_single_kernel(
     const uint8_t* __restrict__ is_token_in_rank, int num_tokens, int num_ranks, int tokens_per_thread,
-    int32_t* __restrict__ send_counts, int64_t* __restrict__ send_cumsum, int64_t* __restrict__ sorted_token_ids) {
+    int32_t* __restrict__ send_counts, int64_t* __restrict__ send_cumsum, int64_t* __restrict__ sorted_token_ids,
+    int32_t* __restrict__ row_of_pair) {
     constexpr int kWaves = kSortChunk / kWave;
     __shared__ int32_t wave_own[kWaves];    // tokens of this rank in each wave
     __shared__ int32_t wave_lower[kWaves];  // memberships of lower ranks in each wave
@@ -259,8 +262,13 @@ __global__ __launch_bounds__(kSortChunk) void routing_sort_single_kernel(
     }
     int64_t pos = int64_t(base) + before + incl - own;
 #pragma unroll
-    for (int i = 0; i < kSingleSortTokensPerThread; ++i)
-        if ((own_bits >> i) & 1) sorted_token_ids[pos++] = first + i;
+    for (int i = 0; i < kSingleSortTokensPerThread; ++i) {
+        const bool mine = (own_bits >> i) & 1;
+        // the inverse of the list, for the reduce that adds up the rows coming back: where is (token, rank)?
+        if (row_of_pair != nullptr && i < tokens_per_thread && first + i < num_tokens)
+            row_of_pair[int64_t(first + i) * num_ranks + r] = mine ? int32_t(pos) : -1;
+        if (mine) sorted_token_ids[pos++] = first + i;
+    }
     if (tid == 0) {
         send_counts[r] = total;
         send_cumsum[r] = base;
@@ -396,8 +404,8 @@ size_t deepep_routing_sort_workspace_bytes(int num_tokens, int num_ranks) {
 }
 
 int deepep_moe_routing_sort(const uint8_t* is_token_in_rank, int num_tokens, int num_ranks,
-                            int64_t* sorted_token_ids, int32_t* send_counts, int64_t* send_cumsum, void* workspace,
-                            size_t workspace_bytes, void* stream) {
+                            int64_t* sorted_token_ids, int32_t* send_counts, int64_t* send_cumsum,
+                            int32_t* row_of_pair, void* workspace, size_t workspace_bytes, void* stream) {
     clear_error();
     EP_HOST_ASSERT(num_tokens >= 0 && num_ranks > 0 && num_ranks <= 1024);
     EP_HOST_ASSERT(send_counts != nullptr && send_cumsum != nullptr);
@@ -408,21 +416,22 @@ int deepep_moe_routing_sort(const uint8_t* is_token_in_rank, int num_tokens, int
     if (num_tokens <= kSortChunk * kSingleSortTokensPerThread && num_ranks <= 64) {
         const int per_thread = num_tokens == 0 ? 1 : (num_tokens + kSortChunk - 1) / kSortChunk;
         routing_sort_single_kernel<<<num_ranks, kSortChunk, 0, s>>>(is_token_in_rank, num_tokens, num_ranks, per_thread,
-                                                                   send_counts, send_cumsum, sorted_token_ids);
+                                                                   send_counts, send_cumsum, sorted_token_ids,
+                                                                   row_of_pair);
         EP_LAUNCH_CHECK();
         return 0;
     }
     int32_t* table = reinterpret_cast<int32_t*>(workspace);
     const size_t lds = size_t(kSortChunk / kWave) * num_ranks * 4;
     routing_sort_pass_kernel<false><<<chunks, kSortChunk, lds, s>>>(is_token_in_rank, num_tokens, num_ranks, table,
-                                                                    sorted_token_ids);
+                                                                    sorted_token_ids, nullptr);
     EP_LAUNCH_CHECK();
     routing_sort_scan_kernel<<<1, 256, size_t(num_ranks + 1) * 8, s>>>(table, chunks, num_ranks, send_counts,
                                                                        send_cumsum);
     EP_LAUNCH_CHECK();
     if (num_tokens > 0) {
         routing_sort_pass_kernel<true><<<chunks, kSortChunk, lds, s>>>(is_token_in_rank, num_tokens, num_ranks,
-                                                                       table, sorted_token_ids);
+                                                                       table, sorted_token_ids, row_of_pair);
         EP_LAUNCH_CHECK();
     }
     return 0;

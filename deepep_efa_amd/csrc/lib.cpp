@@ -23,7 +23,7 @@ extern "C" {
 
 const char* deepep_last_error(void) { return deepep::g_last_error.c_str(); }
 
-int deepep_abi_version(void) { return 9; }
+int deepep_abi_version(void) { return DEEPEP_HIP_ABI_VERSION; }
 
 // Same arithmetic as LowLatencyLayout (reference: csrc/config.hpp:127-193):
 // two send buffers, two receive buffers and two 128-byte-aligned signalling

@@ -112,6 +112,13 @@ struct CombineRecvArgs {
     int num_tokens, hidden, num_topk, num_experts, max_tokens, pieces_per_row;
     int accumulate;  // non-zero: the sum starts from what `out` already holds
     uint8_t* out;
+    // Flat form (rows returned through an all-to-all): combine_staging is one buffer with a row per row
+    // sent, in send order; pair (t, k) is answered by row flat_prefix[expert] + slot, or, when the rows of
+    // every answering rank start at a slot of flat_slot_rows rows, by row rank * flat_slot_rows + (that
+    // minus the first row sent to the rank).  Null flat_prefix: the per-expert staging area.
+    const int32_t* flat_prefix;  // [E + 1]
+    int64_t flat_rows, flat_slot_rows;
+    int experts_per_rank;
 };
 
 // What lane k of a wave knows about selection k of its token once the index loads are back.
@@ -159,7 +166,22 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
     if (lane < num_topk) {
         const int slot = sel.slot;
         const int64_t e = sel.expert;
-        if (slot >= 0 && slot < a.max_tokens && e >= 0 && e < a.num_experts) {
+        if (a.flat_prefix != nullptr) {
+            // csrc/kernels/efa_kernels.cu:1449-1466: the row's index in send order, flat or inside its rank's slot
+            if (slot >= 0 && e >= 0 && e < a.num_experts) {
+                const int first = a.flat_prefix[e], next = a.flat_prefix[e + 1];
+                int64_t idx = int64_t(first) + slot;
+                my_live = first >= 0 && slot < next - first;
+                if (a.flat_slot_rows > 0) {
+                    const int64_t r = e / a.experts_per_rank;
+                    const int64_t within = idx - a.flat_prefix[r * a.experts_per_rank];
+                    my_live = my_live && within >= 0 && within < a.flat_slot_rows;
+                    idx = r * a.flat_slot_rows + within;
+                }
+                my_live = my_live && idx < a.flat_rows;
+                my_row = reinterpret_cast<uint64_t>(a.combine_staging + idx * row_bytes);
+            }
+        } else if (slot >= 0 && slot < a.max_tokens && e >= 0 && e < a.num_experts) {
             const uint8_t* row = a.combine_staging + (e * a.max_tokens + slot) * row_bytes;
             my_live = true;
             const int64_t le = e - own_first_expert;
@@ -271,6 +293,70 @@ __global__ __launch_bounds__(256) void ll_combine_fused_kernel(CombineSendArgs s
     }
 }
 
+// ---------------------------------------------------------------------
+// Send side for an all-to-all shaped transport: the live expert-output rows in
+// arrival order, which is contiguous per destination rank.  Record i of the
+// exchange metadata names the row (padded_index[i] picks the record whose packed
+// row is read, record_packed_row says where the receive side put it) and its place
+// in the flat buffer (combine_send_offset[i]); reference:
+// send_buffer[combine_send_offset[i]] = expert_x[padded_index[i]]
+// (csrc/kernels/coop_combine_send.cuh:37-170; torch form deep_ep/buffer.py:2601-2608).
+// With a table of peer buffers the row skips the send buffer and goes straight to
+// its place in the destination's receive buffer, behind what that rank sent to the
+// ranks below this one (combine_remote_recv_offset,
+// csrc/transport/ll_pipeline.cpp:1283-1295; the reference's peer stores:
+// coop_combine_send.cuh:205-246).  One workgroup per record, one 16-byte vector per thread.
+// ---------------------------------------------------------------------
+struct CombineByDestArgs {
+    const uint8_t* x;
+    const int32_t* record_packed_row;
+    const uint32_t* source_rank;
+    const uint32_t* padded_index;
+    const uint32_t* combine_send_offset;
+    const uint32_t* num_recv_tokens;
+    int64_t row_capacity, x_rows;
+    int num_ranks, num_vec;
+    uint8_t* send_flat;
+    // direct delivery
+    uint8_t* const* peer_recv;  // [R] device pointers, or null
+    const int64_t* peer_rows;   // [R] rows each peer buffer holds
+    const int32_t* recv_counts;
+    const int64_t* remote_offset;
+};
+
+template <bool kStream>
+__global__ __launch_bounds__(1024) void ll_combine_send_by_dest_kernel(CombineByDestArgs a) {
+    int64_t records = a.num_recv_tokens[1];
+    if (records > a.row_capacity) records = a.row_capacity;
+    const int lane = lane_id();
+    const int64_t row_bytes = int64_t(a.num_vec) * 16;
+    for (int64_t i = blockIdx.x; i < records; i += gridDim.x) {
+        const uint32_t p = a.padded_index[i];
+        if (int64_t(p) >= a.row_capacity) continue;
+        const int64_t src_row = a.record_packed_row[p];
+        if (src_row < 0 || src_row >= a.x_rows) continue;  // the record has no row
+        const int64_t offset = a.combine_send_offset[i];
+        uint8_t* dst;
+        if (a.peer_recv == nullptr) {
+            if (offset >= a.row_capacity) continue;
+            dst = a.send_flat + offset * row_bytes;
+        } else {
+            const uint32_t s = a.source_rank[i];
+            if (s >= uint32_t(a.num_ranks)) continue;
+            // the record's place among the rows of its source: offset minus the rows of the lower sources
+            int part = 0;
+            for (int r = lane; r < int(s); r += kWave) part += a.recv_counts[r] < 0 ? 0 : a.recv_counts[r];
+            const int64_t j = offset - __builtin_amdgcn_readlane(wave_inclusive_sum(part), kWave - 1);
+            const int64_t at = a.remote_offset[s] + j;
+            if (j < 0 || j >= a.recv_counts[s] || at < 0 || at >= a.peer_rows[s]) continue;
+            dst = a.peer_recv[s] + at * row_bytes;
+        }
+        const uint8_t* src = a.x + src_row * row_bytes;
+        for (int v = threadIdx.x; v < a.num_vec; v += blockDim.x)
+            store_u32x4<kStream>(dst + int64_t(v) * 16, load_u32x4<kStream>(src + int64_t(v) * 16));
+    }
+}
+
 static CombineSendArgs make_combine_send_args(const void* x, const int64_t* layout_range, int hidden, int num_experts,
                                               int num_ranks, int rank, int max_tokens, void* combine_staging,
                                               void* combine_send_slots, int64_t expected_rows) {
@@ -296,6 +382,7 @@ static CombineRecvArgs make_combine_recv_args(const void* combine_staging, const
     ra.max_tokens = max_tokens, ra.pieces_per_row = (hidden * 2 + 1023) / 1024;
     ra.accumulate = accumulate;
     ra.out = reinterpret_cast<uint8_t*>(out);
+    ra.flat_prefix = nullptr, ra.flat_rows = 0, ra.flat_slot_rows = 0, ra.experts_per_rank = 1;
     return ra;
 }
 
@@ -427,6 +514,80 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
     return launch_combine_recv(combine_staging, topk_idx, topk_weights, pair_slot, num_tokens, hidden, num_topk,
                                num_experts, num_max_dispatch_tokens_per_rank, accumulate, out, nullptr, nullptr, 0, 1,
                                stream);
+}
+
+int deepep_ll_combine_send_by_dest(const void* x, const int32_t* record_packed_row, const uint32_t* source_rank,
+                                   const uint32_t* padded_index, const uint32_t* combine_send_offset,
+                                   const uint32_t* num_recv_tokens, int64_t row_capacity, int hidden, int num_experts,
+                                   int num_ranks, int num_max_dispatch_tokens_per_rank, void* send_flat,
+                                   const int32_t* recv_counts, const int64_t* combine_remote_recv_offset,
+                                   void* const* peer_recv_flat, const int64_t* peer_recv_rows, void* stream) {
+    clear_error();
+    EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
+    EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
+    EP_HOST_ASSERT(num_max_dispatch_tokens_per_rank > 0);
+    EP_HOST_ASSERT(row_capacity >= 0 && row_capacity < (int64_t(1) << 31));
+    if (row_capacity == 0) return 0;
+    EP_HOST_ASSERT(x != nullptr && record_packed_row != nullptr && padded_index != nullptr &&
+                   combine_send_offset != nullptr && num_recv_tokens != nullptr);
+    const bool direct = peer_recv_flat != nullptr;
+    EP_HOST_ASSERT(direct || send_flat != nullptr);
+    EP_HOST_ASSERT(!direct || (source_rank != nullptr && recv_counts != nullptr &&
+                               combine_remote_recv_offset != nullptr && peer_recv_rows != nullptr));
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(send_flat) & 15) == 0);
+    CombineByDestArgs a;
+    a.x = reinterpret_cast<const uint8_t*>(x);
+    a.record_packed_row = record_packed_row, a.source_rank = source_rank, a.padded_index = padded_index;
+    a.combine_send_offset = combine_send_offset, a.num_recv_tokens = num_recv_tokens;
+    a.row_capacity = row_capacity;
+    a.x_rows = int64_t(num_experts) * num_max_dispatch_tokens_per_rank;  // E_l * R * M rows of expert outputs
+    a.num_ranks = num_ranks, a.num_vec = hidden * 2 / 16;
+    a.send_flat = reinterpret_cast<uint8_t*>(send_flat);
+    a.peer_recv = reinterpret_cast<uint8_t* const*>(peer_recv_flat), a.peer_rows = peer_recv_rows;
+    a.recv_counts = recv_counts, a.remote_offset = combine_remote_recv_offset;
+    int threads = ((a.num_vec + 63) / 64) * 64;
+    if (threads > 1024) threads = 1024;
+    int64_t blocks = row_capacity;
+    if (blocks > 16384) blocks = blocks / 2 > 16384 ? blocks / 2 : 16384;
+    if (blocks > (int64_t(1) << 22)) blocks = int64_t(1) << 22;
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    if (2 * row_capacity * hidden * 2 > stream_bytes())
+        ll_combine_send_by_dest_kernel<true><<<unsigned(blocks), threads, 0, hs>>>(a);
+    else
+        ll_combine_send_by_dest_kernel<false><<<unsigned(blocks), threads, 0, hs>>>(a);
+    EP_LAUNCH_CHECK();
+    return 0;
+}
+
+int deepep_ll_combine_recv_flat(const void* recv_flat, int64_t recv_flat_rows, int64_t slot_rows,
+                                const int32_t* send_expert_prefix, const int64_t* topk_idx,
+                                const float* topk_weights, const int32_t* pair_slot, int num_tokens, int hidden,
+                                int num_topk, int num_experts, int num_ranks, int num_max_dispatch_tokens_per_rank,
+                                int accumulate, void* out, void* stream) {
+    clear_error();
+    EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
+    EP_HOST_ASSERT(recv_flat_rows >= 0 && slot_rows >= 0);
+    EP_HOST_ASSERT(slot_rows == 0 || slot_rows * num_ranks <= recv_flat_rows);
+    if (int rc = check_combine_recv_args(recv_flat, topk_idx, topk_weights, pair_slot, num_tokens, hidden, num_topk,
+                                         num_experts, num_max_dispatch_tokens_per_rank, out))
+        return rc;
+    if (num_tokens == 0) return 0;
+    EP_HOST_ASSERT(send_expert_prefix != nullptr);
+    CombineRecvArgs ra = make_combine_recv_args(recv_flat, topk_idx, topk_weights, pair_slot, num_tokens, hidden,
+                                                num_topk, num_experts, num_max_dispatch_tokens_per_rank, accumulate,
+                                                out);
+    ra.flat_prefix = send_expert_prefix, ra.flat_rows = recv_flat_rows, ra.flat_slot_rows = slot_rows;
+    ra.experts_per_rank = num_experts / num_ranks;
+    const int waves = 4;
+    const int64_t blocks = (int64_t(num_tokens) * ra.pieces_per_row + waves - 1) / waves;
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    if (int64_t(num_tokens) * num_topk * hidden * 2 > stream_bytes())
+        ll_combine_recv_kernel<true><<<dim3(unsigned(blocks)), waves * kWave, 0, hs>>>(ra, nullptr, nullptr, 0, 0, 1);
+    else
+        ll_combine_recv_kernel<false><<<dim3(unsigned(blocks)), waves * kWave, 0, hs>>>(ra, nullptr, nullptr, 0, 0, 1);
+    EP_LAUNCH_CHECK();
+    return 0;
 }
 
 int deepep_ll_combine(const void* x, const int64_t* layout_range, const int64_t* topk_idx, const float* topk_weights,

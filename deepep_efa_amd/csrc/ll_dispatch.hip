@@ -16,6 +16,7 @@
 #include "common.hpp"
 #include "quant.hpp"
 #include "segments.hpp"
+#include <algorithm>
 #include <cstdlib>
 #include <mutex>
 
@@ -131,6 +132,9 @@ struct SendArgs {
     int32_t* pair_slot;
     int32_t* recv_count;
     int32_t* send_count;
+    // By-destination form: send_slots is one buffer of rows, contiguous per destination rank, and every
+    // row (the rank's own included) goes to row expert_prefix[expert] + slot of it.  Null: per-expert slots.
+    const int32_t* expert_prefix;
 };
 
 // Final destination of the rows a rank sends to its own experts, used by the
@@ -238,6 +242,8 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
             local = my_expert - dst_rank * (num_experts / a.num_ranks);
         }
     }
+    int dest_first = 0;  // by-destination form: where the expert's run of rows begins in the send buffer
+    if (a.expert_prefix != nullptr && my_expert >= 0) dest_first = a.expert_prefix[my_expert];
     if (direct.packed_x != nullptr && tid < kWave) {
         // Rows for this rank's own experts go straight to the packed tensors, at the place the
         // reference's range builder gives them: behind the rows of the lower source ranks
@@ -347,7 +353,10 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
         uint8_t* scale_row = nullptr;
         bool staged = false;
         if (my_slot >= 0) {
-            if (dst_rank == a.rank && direct.packed_x != nullptr) {
+            if (a.expert_prefix != nullptr) {
+                row = a.send_slots + (int64_t(dest_first) + my_slot) * stride;
+                staged = true;
+            } else if (dst_rank == a.rank && direct.packed_x != nullptr) {
                 const int64_t out_row = int64_t(local) * a.num_ranks * a.max_tokens + direct_begin + my_slot;
                 row = direct.packed_x + out_row * data_bytes;
                 scale_row = direct.packed_scales + out_row * scale_bytes;
@@ -409,7 +418,8 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs 
     extern __shared__ int32_t lds_hist[];  // [E], counting workgroups only
     __shared__ SendLds lds;
     if (int(blockIdx.y) == a.num_tokens) {  // the counting row of the grid
-        if (blockIdx.x == 0) send_count_block(a, blockIdx.z, lds_hist);
+        // (the by-destination form has its counts already: ll_by_dest_prefix_kernel ran first)
+        if (blockIdx.x == 0 && a.expert_prefix == nullptr) send_count_block(a, blockIdx.z, lds_hist);
         return;
     }
     send_token_block<kFmt, kStream>(a, direct, blockIdx.z, blockIdx.y, blockIdx.x, lds);
@@ -695,6 +705,73 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_dispatch_fused_kernel
 }
 
 // ---------------------------------------------------------------------
+// By-destination send (what an all-to-all ships: one contiguous message per
+// peer).  Before the send kernel runs, one workgroup turns the route counts into
+// the tables the rows are placed by: send_count[e] (clamped to the M slots of a
+// pair), its exclusive prefix over the experts -- the first row of every expert's
+// run, experts ascending, hence destination ranks ascending -- and the per-rank
+// counts and prefix the transport cuts the buffer by.
+// Reference: the count + prefix phases of ll_dispatch_route_and_pack_v3
+// (csrc/kernels/efa_kernels.cu:2358-2371: ll_dispatch_count_kernel, prefix_sum_kernel).
+// ---------------------------------------------------------------------
+struct ByDestTables {
+    int32_t* expert_prefix;  // [E + 1]
+    int32_t* rank_counts;    // [R]
+    int64_t* rank_cumsum;    // [R + 1]
+};
+
+__global__ __launch_bounds__(1024) void ll_by_dest_prefix_kernel(const int64_t* __restrict__ topk_idx, int n,
+                                                                 int num_experts, int num_ranks, int max_tokens,
+                                                                 const int32_t* __restrict__ chunk_hist, int num_chunks,
+                                                                 int32_t* __restrict__ send_count, ByDestTables out) {
+    extern __shared__ int32_t hist[];  // [E + 1]
+    __shared__ int32_t wave_totals[kMaxBlockWaves];
+    const int tid = threadIdx.x, threads = blockDim.x;
+    if (chunk_hist != nullptr) {  // the column sums of the chunk histograms
+        for (int e = tid; e < num_experts; e += threads) {
+            int total = 0;
+            for (int c0 = 0; c0 < num_chunks; c0 += 8) {  // eight loads in flight
+                int v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = c0 + u < num_chunks ? chunk_hist[int64_t(c0 + u) * num_experts + e] : 0;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) total += v[u];
+            }
+            hist[e] = total;
+        }
+    } else {
+        for (int e = tid; e < num_experts; e += threads) hist[e] = 0;
+        lds_barrier();
+        for (int base = 0; base < n; base += 4 * threads) {  // four loads in flight per thread
+            int64_t v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = base + u * threads + tid;
+                v[u] = i < n ? topk_idx[i] : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (v[u] >= 0 && v[u] < num_experts) atomicAdd(&hist[int(v[u])], 1);
+        }
+    }
+    lds_barrier();
+    for (int e = tid; e < num_experts; e += threads) {
+        const int c = hist[e] < max_tokens ? hist[e] : max_tokens;
+        hist[e] = c;
+        send_count[e] = c;
+    }
+    lds_barrier();
+    block_exclusive_scan(hist, num_experts, wave_totals);
+    for (int e = tid; e <= num_experts; e += threads) out.expert_prefix[e] = hist[e];
+    const int experts_per_rank = num_experts / num_ranks;
+    for (int r = tid; r < num_ranks; r += threads) {
+        out.rank_counts[r] = hist[(r + 1) * experts_per_rank] - hist[r * experts_per_rank];
+        out.rank_cumsum[r] = hist[r * experts_per_rank];
+    }
+    if (tid == 0) out.rank_cumsum[num_ranks] = hist[num_experts];
+}
+
+// ---------------------------------------------------------------------
 // Host side
 // ---------------------------------------------------------------------
 static int check_ll_shape(int num_tokens, int hidden, int num_topk, int num_experts, int num_ranks, int rank,
@@ -716,7 +793,8 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
                             int max_tokens, int row_format, void* recv_staging, int32_t* recv_count,
                             void* send_slots, int32_t* send_count, int32_t* pair_slot, void* workspace,
                             size_t workspace_bytes, hipStream_t stream, const RecvArgs* fused_recv = nullptr,
-                            int64_t fused_recv_wave_items = 0, const DirectOut* own_rows_direct = nullptr) {
+                            int64_t fused_recv_wave_items = 0, const DirectOut* own_rows_direct = nullptr,
+                            const ByDestTables* by_dest = nullptr) {
     const int64_t scratch_bytes = route_scratch_bytes(num_tokens, num_topk, num_experts);
     EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(scratch_bytes) * size_t(num_src));
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
@@ -729,6 +807,14 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
         const int chunks = (num_tokens + tpc - 1) / tpc;
         ll_chunk_hist_kernel<<<dim3(chunks, num_src), 1024, size_t(num_experts) * sizeof(int32_t), stream>>>(
             topk_idx, n, tpc * num_topk, num_experts, scratch_bytes, ws);
+        EP_LAUNCH_CHECK();
+    }
+    if (by_dest != nullptr) {  // the tables the by-destination rows are placed by
+        EP_HOST_ASSERT(num_src == 1 && src_ranks == nullptr && fused_recv == nullptr && own_rows_direct == nullptr);
+        const int chunks = tpc > 0 ? (num_tokens + tpc - 1) / tpc : 0;
+        ll_by_dest_prefix_kernel<<<1, 1024, size_t(num_experts + 1) * sizeof(int32_t), stream>>>(
+            topk_idx, n, num_experts, num_ranks, max_tokens, tpc > 0 ? reinterpret_cast<const int32_t*>(ws) : nullptr,
+            chunks, send_count, *by_dest);
         EP_LAUNCH_CHECK();
     }
 
@@ -763,6 +849,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     sa.recv_staging = reinterpret_cast<uint8_t*>(recv_staging);
     sa.send_slots = reinterpret_cast<uint8_t*>(send_slots);
     sa.pair_slot = pair_slot, sa.recv_count = recv_count, sa.send_count = send_count;
+    sa.expert_prefix = by_dest != nullptr ? by_dest->expert_prefix : nullptr;
 
     if (fused_recv != nullptr) {  // single launch: send workgroups, the counting workgroup, receive workgroups
         EP_HOST_ASSERT(tpc == 0 && num_src == 1 && src_ranks == nullptr);
@@ -919,6 +1006,32 @@ int deepep_ll_dispatch_send_static(const void* x, const int64_t* topk_idx, int n
                             num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count, send_slots,
                             send_count, pair_slot, route_scratch, kStaticScratchBytes,
                             reinterpret_cast<hipStream_t>(stream));
+}
+
+int deepep_ll_dispatch_send_by_dest(const void* x, const int64_t* topk_idx, int num_tokens, int hidden, int num_topk,
+                                    int num_experts, int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                                    int row_format, void* send_rows, int64_t send_row_capacity, int32_t* send_count,
+                                    int32_t* send_expert_prefix, int32_t* send_counts, int64_t* send_cumsum,
+                                    int32_t* pair_slot, void* workspace, size_t workspace_bytes, void* stream) {
+    clear_error();
+    if (int rc = check_ll_shape(num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                                num_max_dispatch_tokens_per_rank, row_format))
+        return rc;
+    EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
+    EP_HOST_ASSERT(send_count != nullptr && send_expert_prefix != nullptr && send_counts != nullptr &&
+                   send_cumsum != nullptr && pair_slot != nullptr);
+    // every live pair sends one row, and an expert takes at most M of them
+    const int64_t most_rows = std::min<int64_t>(int64_t(num_tokens) * num_topk,
+                                                int64_t(num_experts) * num_max_dispatch_tokens_per_rank);
+    EP_HOST_ASSERT(send_row_capacity >= most_rows);
+    EP_HOST_ASSERT(most_rows == 0 || send_rows != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(send_rows) & 15) == 0);
+    const ByDestTables tables = {send_expert_prefix, send_counts, send_cumsum};
+    return launch_send_side(x, topk_idx, nullptr, 1, num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
+                            num_max_dispatch_tokens_per_rank, row_format, nullptr, nullptr, send_rows, send_count,
+                            pair_slot, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream), nullptr, 0,
+                            nullptr, &tables);
 }
 
 int deepep_loopback_dispatch_from_peers(const void* x, const int64_t* topk_idx, const int32_t* src_ranks,

@@ -146,7 +146,7 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
     const uint32_t* __restrict__ num_recv_tokens, int64_t row_capacity, int num_local_experts, int num_ranks,
     int max_tokens, const int32_t* __restrict__ hist, int64_t* __restrict__ layout_range,
     int32_t* __restrict__ packed_count, int32_t* __restrict__ stats, uint32_t* __restrict__ tokens_per_expert,
-    int32_t* __restrict__ flat_total, RowDesc* __restrict__ desc) {
+    int32_t* __restrict__ record_packed_row, int32_t* __restrict__ flat_total, RowDesc* __restrict__ desc) {
     // prefix [R + 1] | chunk_prefix [R + 1] | pair_prefix [E_l * R + 1] | running [E_l] | wave_cnt [waves][E_l]
     extern __shared__ int32_t lds[];
     __shared__ int32_t scan_tmp[kMaxBlockWaves];
@@ -242,6 +242,7 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
         const int before_in_wave = __popcll(same & lanes_below(lane));
         if (e >= 0 && (same >> lane) >> 1 == 0) wave_cnt[w * num_local_experts + e] = __popcll(same);  // the group's last lane
         lds_barrier();
+        int32_t packed_row = -1;  // where this record's row lands; -1: nowhere
         if (e >= 0) {
             // The descriptors are laid out in the order of the packed rows (expert, source, arrival), not of
             // the records: the copy then writes consecutive rows from consecutive workgroups.
@@ -253,8 +254,12 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
                 d.src_row = int32_t(offset);
                 d.dst_row = int32_t(int64_t(e) * slots_per_expert + pair_begin + pos);
                 desc[pair_prefix[e * num_ranks + s] + pos] = d;
+                packed_row = d.dst_row;
             }
         }
+        // what the combine needs to return the rows in arrival order: the reference's recv_expert_ids /
+        // recv_expert_pos (csrc/kernels/efa_kernels.cu:2121-2231), as one row index per record
+        if (record_packed_row != nullptr && i < end) record_packed_row[i] = packed_row;
         if constexpr (kChunked) break;  // one chunk per workgroup
         lds_barrier();
         for (int e2 = tid; e2 < num_local_experts; e2 += kBySourceThreads) {
@@ -292,7 +297,8 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
                                       void* packed_recv_scales, int32_t* packed_recv_src_info,
                                       int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
                                       int32_t* cumulative_local_expert_recv_stats, uint32_t* tokens_per_expert,
-                                      void* workspace, size_t workspace_bytes, void* stream) {
+                                      int32_t* record_packed_row, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
     clear_error();
     EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
     EP_HOST_ASSERT(num_ranks > 0 && num_ranks <= kBySourceMaxRanks);
@@ -337,7 +343,7 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
             rows_in, stride, tail_off, buffer_rows, int(slot_rows), recv_counts, source_offset, num_recv_tokens,
             row_capacity, num_local_experts, num_ranks, num_max_dispatch_tokens_per_rank, nullptr,
             packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, tokens_per_expert,
-            flat_total, desc);
+            record_packed_row, flat_total, desc);
         EP_LAUNCH_CHECK();
     } else {
         // every source's records round up to whole chunks: at most ceil(capacity / 512) + R of them
@@ -351,7 +357,7 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
             rows_in, stride, tail_off, buffer_rows, int(slot_rows), recv_counts, source_offset, num_recv_tokens,
             row_capacity, num_local_experts, num_ranks, num_max_dispatch_tokens_per_rank, hist,
             packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, tokens_per_expert,
-            flat_total, desc);
+            record_packed_row, flat_total, desc);
         EP_LAUNCH_CHECK();
     }
     if (row_capacity == 0) return 0;

@@ -145,26 +145,6 @@ __global__ __launch_bounds__(256) void combine_from_peers_kernel(
     }
 }
 
-// A measuring stick for the send side's access pattern and nothing else: one workgroup per token
-// reads the token's row (two 16-byte vectors per thread) and stores one vector per thread to each of
-// the token's K destination rows.  No routing, no quantisation, no scales.
-__global__ __launch_bounds__(1024) void row_scatter_probe_kernel(const uint8_t* __restrict__ x, int64_t x_row_bytes,
-                                                                 const int32_t* __restrict__ dst_rows, int num_topk,
-                                                                 uint8_t* __restrict__ dst, int64_t dst_stride,
-                                                                 int vecs) {
-    const int t = blockIdx.x, tid = threadIdx.x;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (tid < vecs) {
-        const uint8_t* src = x + int64_t(t) * x_row_bytes + int64_t(tid) * 32;
-        const u32x4 a = *reinterpret_cast<const u32x4*>(src), b = *reinterpret_cast<const u32x4*>(src + 16);
-        v = a ^ b;
-    }
-    for (int k = 0; k < num_topk; ++k) {
-        const int row = dst_rows[int64_t(t) * num_topk + k];
-        if (row >= 0 && tid < vecs) store_u32x4<true>(dst + int64_t(row) * dst_stride + int64_t(tid) * 16, v);  // streaming
-    }
-}
-
 }  // namespace deepep
 
 using namespace deepep;
@@ -201,23 +181,6 @@ int deepep_synth_bf16_rows(void* dst, int64_t num_rows, int hidden, int64_t row_
     synth_bf16_rows_kernel<<<dim3(unsigned(blocks)), 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(
         reinterpret_cast<uint8_t*>(dst), num_rows, hidden, row_stride_bytes, row_keys, first_key, seed,
         outlier_period);
-    EP_LAUNCH_CHECK();
-    return 0;
-}
-
-int deepep_probe_row_scatter(const void* x, int num_tokens, int hidden, const int32_t* dst_rows, int num_topk,
-                             void* dst, int64_t dst_stride_bytes, void* stream) {
-    clear_error();
-    EP_HOST_ASSERT(num_tokens >= 0 && hidden > 0 && hidden % 16 == 0 && hidden / 16 <= 1024 && num_topk > 0);
-    EP_HOST_ASSERT(dst_stride_bytes >= hidden && dst_stride_bytes % 16 == 0);
-    if (num_tokens == 0) return 0;
-    EP_HOST_ASSERT(x != nullptr && dst_rows != nullptr && dst != nullptr);
-    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0);
-    const int vecs = hidden / 16;
-    row_scatter_probe_kernel<<<dim3(unsigned(num_tokens)), ((vecs + 63) / 64) * 64, 0,
-                               reinterpret_cast<hipStream_t>(stream)>>>(
-        reinterpret_cast<const uint8_t*>(x), int64_t(hidden) * 2, dst_rows, num_topk, reinterpret_cast<uint8_t*>(dst),
-        dst_stride_bytes, vecs);
     EP_LAUNCH_CHECK();
     return 0;
 }

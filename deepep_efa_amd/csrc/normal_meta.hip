@@ -244,8 +244,8 @@ size_t deepep_combine_reduce_workspace_bytes(int num_tokens, int num_ranks) {
 int deepep_combine_reduce(const void* recv_x, const float* recv_topk_weights, const int64_t* sorted_token_ids,
                           const int64_t* send_cumsum, const uint8_t* is_token_in_rank, const void* bias_0,
                           const void* bias_1, int num_tokens, int hidden, int num_topk, int num_ranks,
-                          int64_t max_rows, void* combined_x, float* combined_topk_weights, void* workspace,
-                          size_t workspace_bytes, void* stream) {
+                          int64_t max_rows, const int32_t* row_of_pair_in, void* combined_x,
+                          float* combined_topk_weights, void* workspace, size_t workspace_bytes, void* stream) {
     clear_error();
     EP_HOST_ASSERT(num_tokens >= 0 && hidden > 0 && hidden % 8 == 0 && num_ranks > 0 && num_ranks <= 4096);
     EP_HOST_ASSERT(max_rows >= 0 && max_rows < (int64_t(1) << 31));
@@ -254,17 +254,21 @@ int deepep_combine_reduce(const void* recv_x, const float* recv_topk_weights, co
     EP_HOST_ASSERT(sorted_token_ids != nullptr && send_cumsum != nullptr && is_token_in_rank != nullptr &&
                    combined_x != nullptr);
     EP_HOST_ASSERT(max_rows == 0 || recv_x != nullptr);
-    EP_HOST_ASSERT(workspace != nullptr &&
-                   workspace_bytes >= deepep_combine_reduce_workspace_bytes(num_tokens, num_ranks));
+    EP_HOST_ASSERT(row_of_pair_in != nullptr ||
+                   (workspace != nullptr &&
+                    workspace_bytes >= deepep_combine_reduce_workspace_bytes(num_tokens, num_ranks)));
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_x) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(combined_x) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(bias_0) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias_1) & 15) == 0);
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 3) == 0);
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
-    int32_t* row_of_pair = reinterpret_cast<int32_t*>(workspace);
-    if (max_rows > 0) {
+    // with the table the routing sort left (where it wrote every list entry it also wrote the entry's
+    // place) the reduce is the only launch; otherwise the table is rebuilt from the list first
+    const int32_t* row_of_pair = row_of_pair_in;
+    if (row_of_pair_in == nullptr) row_of_pair = reinterpret_cast<int32_t*>(workspace);
+    if (max_rows > 0 && row_of_pair_in == nullptr) {
         combine_positions_kernel<<<meta_grid(max_rows), kMetaThreads, size_t(num_ranks + 1) * sizeof(int64_t), hs>>>(
-            sorted_token_ids, send_cumsum, num_tokens, num_ranks, max_rows, row_of_pair);
+            sorted_token_ids, send_cumsum, num_tokens, num_ranks, max_rows, reinterpret_cast<int32_t*>(workspace));
         EP_LAUNCH_CHECK();
     }
     const int pieces = (hidden * 2 + 1023) / 1024;

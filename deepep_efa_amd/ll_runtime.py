@@ -182,3 +182,99 @@ def exchange_metadata(all_num_routed: torch.Tensor, rank: int, max_tokens: int, 
         _capi.ptr(out["combine_send_offset"]), _capi.ptr(out["num_recv_tokens"]), _capi.ptr(out["tokens_per_expert"]),
         current_stream_ptr()))
     return out
+
+
+class AllToAllState:
+    """Device buffers and C-ABI calls of one rank's low-latency step over a transport that ships one
+    contiguous message per peer in each direction (the reference's dist.all_to_all_single branch,
+    deep_ep/buffer.py:2266-2301 and :2735).  The transport itself is the caller's: it moves
+    ``send_rows[send_cumsum[d]:send_cumsum[d + 1]]`` to row ``rank * slot_rows`` of rank d's
+    ``recv_by_source``, and on the way back ``send_flat[first(s):first(s) + recv_counts[s]]`` (first = the
+    prefix of ``recv_counts``) to row ``send_cumsum_of_s[rank]`` of rank s's ``recv_flat``.
+    """
+
+    def __init__(self, shape: LLShape, slot_rows: int = None, device="cuda"):
+        lib = _capi.load()
+        self.lib = lib
+        self.shape = s = shape
+        el, r, m, e, h, k = s.num_local_experts, s.num_ranks, s.max_tokens, s.num_experts, s.hidden, s.num_topk
+        self.stride = lib.deepep_ll_row_stride(h, s.fmt)
+        u8 = dict(dtype=torch.uint8, device=device)
+        i32 = dict(dtype=torch.int32, device=device)
+        # dispatch, send side
+        self.send_capacity = max(1, min(m * k, e * m))
+        self.send_rows = torch.empty((self.send_capacity, self.stride), **u8)
+        self.send_count = torch.zeros(e, **i32)
+        self.send_expert_prefix = torch.zeros(e + 1, **i32)
+        self.send_counts = torch.zeros(r, **i32)
+        self.send_cumsum = torch.zeros(r + 1, dtype=torch.int64, device=device)
+        self.pair_slot = torch.full((m, k), -1, **i32)
+        self.workspace = torch.empty(max(256, lib.deepep_ll_dispatch_workspace_bytes(m, k, e)), **u8)
+        # dispatch, receive side: one slot of slot_rows rows per source rank
+        self.slot_rows = m * min(k, el) if slot_rows is None else slot_rows
+        self.row_capacity = r * self.slot_rows
+        self.recv_by_source = torch.empty((self.row_capacity, self.stride), **u8)
+        self.by_source_workspace = torch.empty(lib.deepep_ll_by_source_workspace_bytes(e, self.row_capacity), **u8)
+        self.record_packed_row = torch.full((self.row_capacity,), -1, **i32)
+        self.tokens_per_expert = torch.zeros(el, **i32)
+        if s.fmt == ROW_BF16:
+            self.packed_recv_x = torch.empty((el, r * m, h), dtype=torch.bfloat16, device=device)
+            self.packed_recv_scales = None
+        else:
+            self.packed_recv_x = torch.empty((el, r * m, h), dtype=torch.float8_e4m3fn, device=device)
+            if s.fmt == ROW_FP8_UE8M0:
+                self.packed_recv_scales = torch.empty((el, r * m, h // 512), **i32)
+            else:
+                self.packed_recv_scales = torch.empty((el, r * m, h // 128), dtype=torch.float32, device=device)
+        self.packed_recv_count = torch.zeros(el, **i32)
+        self.packed_recv_src_info = torch.empty((el, r * m), **i32)
+        self.packed_recv_layout_range = torch.zeros((el, r), dtype=torch.int64, device=device)
+        # combine: the rows owed to the other ranks in arrival order; the answers in send order
+        self.send_flat = torch.empty((self.row_capacity, h), dtype=torch.bfloat16, device=device)
+        self.recv_flat = torch.empty((self.send_capacity, h), dtype=torch.bfloat16, device=device)
+        self.meta = None
+
+    def dispatch_send(self, x: torch.Tensor, topk_idx: torch.Tensor) -> None:
+        s = self.shape
+        _capi.check(self.lib.deepep_ll_dispatch_send_by_dest(
+            _capi.ptr(x), _capi.ptr(topk_idx), x.shape[0], s.hidden, s.num_topk, s.num_experts, s.num_ranks, s.rank,
+            s.max_tokens, s.fmt, _capi.ptr(self.send_rows), self.send_capacity, _capi.ptr(self.send_count),
+            _capi.ptr(self.send_expert_prefix), _capi.ptr(self.send_counts), _capi.ptr(self.send_cumsum),
+            _capi.ptr(self.pair_slot), _capi.ptr(self.workspace), self.workspace.numel(), current_stream_ptr()))
+
+    def exchange_metadata(self, all_num_routed: torch.Tensor) -> dict:
+        """all_num_routed [R, E] int32: the ranks' send_count, as an all-gather leaves them everywhere."""
+        self.meta = exchange_metadata(all_num_routed, self.shape.rank, self.slot_rows, self.row_capacity)
+        return self.meta
+
+    def dispatch_recv(self, stats: torch.Tensor = None) -> None:
+        s, m = self.shape, self.meta
+        _capi.check(self.lib.deepep_ll_dispatch_recv_by_source(
+            _capi.ptr(self.recv_by_source), self.slot_rows, _capi.ptr(m["recv_counts"]), _capi.ptr(m["source_offset"]),
+            _capi.ptr(m["num_recv_tokens"]), self.row_capacity, s.hidden, s.num_experts, s.num_ranks, s.max_tokens,
+            s.fmt, _capi.ptr(self.packed_recv_x), _capi.ptr(self.packed_recv_scales),
+            _capi.ptr(self.packed_recv_src_info), _capi.ptr(self.packed_recv_layout_range),
+            _capi.ptr(self.packed_recv_count), _capi.ptr(stats), _capi.ptr(self.tokens_per_expert),
+            _capi.ptr(self.record_packed_row), _capi.ptr(self.by_source_workspace), self.by_source_workspace.numel(),
+            current_stream_ptr()))
+
+    def combine_send(self, y: torch.Tensor, peer_recv_flat: torch.Tensor = None,
+                     peer_recv_rows: torch.Tensor = None) -> None:
+        """Rows owed to the other ranks into send_flat, or, with a table of the ranks' recv_flat addresses
+        (int64 [R]) and their row counts, straight to their place in those buffers."""
+        s, m = self.shape, self.meta
+        _capi.check(self.lib.deepep_ll_combine_send_by_dest(
+            _capi.ptr(y), _capi.ptr(self.record_packed_row), _capi.ptr(m["source_rank"]), _capi.ptr(m["padded_index"]),
+            _capi.ptr(m["combine_send_offset"]), _capi.ptr(m["num_recv_tokens"]), self.row_capacity, s.hidden,
+            s.num_experts, s.num_ranks, s.max_tokens, _capi.ptr(self.send_flat), _capi.ptr(m["recv_counts"]),
+            _capi.ptr(m["combine_remote_recv_offset"]), _capi.ptr(peer_recv_flat), _capi.ptr(peer_recv_rows),
+            current_stream_ptr()))
+
+    def combine_recv(self, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor,
+                     recv: torch.Tensor = None, slot_rows: int = 0, accumulate: bool = False) -> None:
+        s = self.shape
+        buf = self.recv_flat if recv is None else recv
+        _capi.check(self.lib.deepep_ll_combine_recv_flat(
+            _capi.ptr(buf), buf.shape[0], slot_rows, _capi.ptr(self.send_expert_prefix), _capi.ptr(topk_idx),
+            _capi.ptr(topk_weights), _capi.ptr(self.pair_slot), topk_idx.shape[0], s.hidden, s.num_topk,
+            s.num_experts, s.num_ranks, s.max_tokens, int(accumulate), _capi.ptr(out), current_stream_ptr()))

@@ -19,6 +19,12 @@ def moe_routing_sort(is_token_in_rank: torch.Tensor):
     return deep_ep_cpp.moe_routing_sort(is_token_in_rank)
 
 
+def moe_routing_sort_with_positions(is_token_in_rank: torch.Tensor):
+    """moe_routing_sort plus the inverse of the list, row_of_pair [T, R] int32 (-1 = token not sent to the rank):
+    handed to combine_reduce it saves that call a launch."""
+    return deep_ep_cpp.moe_routing_sort_with_positions(is_token_in_rank)
+
+
 def channel_prefix_matrix(is_token_in_rank: torch.Tensor, num_channels: int) -> torch.Tensor:
     """[T, R] bool -> [R, C] int32 inclusive prefix over channels of tokens bound for each rank."""
     return deep_ep_cpp.channel_prefix_matrix(is_token_in_rank, num_channels)
@@ -45,7 +51,8 @@ def build_recv_src_meta(recv_counts: torch.Tensor, recv_cumsum: torch.Tensor, nu
 
 def combine_reduce(recv_x: torch.Tensor, recv_topk_weights: Optional[torch.Tensor], sorted_token_ids: torch.Tensor,
                    send_cumsum: torch.Tensor, is_token_in_rank: torch.Tensor, bias_0: Optional[torch.Tensor] = None,
-                   bias_1: Optional[torch.Tensor] = None):
-    """combined_x[t] = sum over the ranks holding t of the row that came back (+ biases), float32 accumulate."""
+                   bias_1: Optional[torch.Tensor] = None, row_of_pair: Optional[torch.Tensor] = None):
+    """combined_x[t] = sum over the ranks holding t of the row that came back (+ biases), float32 accumulate.
+    row_of_pair: the table of moe_routing_sort_with_positions (one launch instead of two)."""
     return deep_ep_cpp.combine_reduce(recv_x, recv_topk_weights, sorted_token_ids, send_cumsum, is_token_in_rank,
-                                      bias_0, bias_1)
+                                      bias_0, bias_1, row_of_pair)

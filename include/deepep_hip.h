@@ -40,7 +40,9 @@ extern "C" {
 /* Message of the last failure on the calling thread ("" if none). */
 const char* deepep_last_error(void);
 
-/* ABI revision of this header; bumped on any signature change. */
+/* ABI revision of this header; bumped on any signature change.  deepep_abi_version() returns the
+ * revision the library was built from: a binding compares the two before its first call. */
+#define DEEPEP_HIP_ABI_VERSION 10
 int deepep_abi_version(void);
 
 /* ------------------------------------------------------------------ */
@@ -105,11 +107,14 @@ size_t deepep_routing_sort_workspace_bytes(int num_tokens, int num_ranks);
  *   sorted_token_ids  [T * R] int64 (out; first send_cumsum[R] entries valid)
  *   send_counts       [R] int32 (out)
  *   send_cumsum       [R + 1] int64 (out, exclusive prefix; [R] = total)
+ *   row_of_pair       [T, R] int32 (out) or NULL: the inverse of the list, row_of_pair[t, r] = the index
+ *                     i with sorted_token_ids[i] == t inside rank r's segment, -1 where token t does
+ *                     not go to rank r.  deepep_combine_reduce takes it and then needs one launch.
  * Replaces moe_routing_sort (csrc/kernels/efa_kernels.cu:220-318,1591-1651);
  * the total stays on the device — the caller reads send_cumsum[R]. */
 int deepep_moe_routing_sort(const uint8_t* is_token_in_rank, int num_tokens, int num_ranks,
                             int64_t* sorted_token_ids, int32_t* send_counts, int64_t* send_cumsum,
-                            void* workspace, size_t workspace_bytes, void* stream);
+                            int32_t* row_of_pair, void* workspace, size_t workspace_bytes, void* stream);
 
 /* channel_prefix_matrix[d, c] = number of tokens bound for rank d in
  * channels 0..c, channel c owning tokens [min(c*ceil(T/C),T), min(+ceil(T/C),T)).
@@ -172,13 +177,16 @@ size_t deepep_combine_reduce_workspace_bytes(int num_tokens, int num_ranks);
  *   bias_0, bias_1 [T, H] bf16 or NULL
  *   combined_x [T, H] bf16 (out)   combined_topk_weights [T, K] float32 (out) or NULL
  *   max_rows bounds the rows of recv_x that may be read.
+ *   row_of_pair  [T, R] int32 from deepep_moe_routing_sort, or NULL: without it the call first
+ *                rebuilds that table from the list (a second launch, into `workspace`); with it
+ *                `workspace` may be NULL.
  * Replaces the zero_() + index_add_ + bias adds of deep_ep/buffer.py:1542-1557
  * (which accumulate in bf16 through atomics, in arrival order). */
 int deepep_combine_reduce(const void* recv_x, const float* recv_topk_weights,
                           const int64_t* sorted_token_ids, const int64_t* send_cumsum,
                           const uint8_t* is_token_in_rank, const void* bias_0, const void* bias_1,
                           int num_tokens, int hidden, int num_topk, int num_ranks, int64_t max_rows,
-                          void* combined_x, float* combined_topk_weights,
+                          const int32_t* row_of_pair, void* combined_x, float* combined_topk_weights,
                           void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ */
@@ -257,6 +265,34 @@ int deepep_ll_dispatch_send_static(const void* x, const int64_t* topk_idx,
                                    void* send_slots, int32_t* send_count, int32_t* pair_slot,
                                    void* stream);
 
+/* Send side for a transport that ships one contiguous message per peer (an all-to-all): the same
+ * route + quantise + pack, but every row -- this rank's own included -- goes into ONE buffer that is
+ * contiguous per destination rank, destination ranks ascending.  Inside a destination's message the
+ * rows come expert by expert and, inside an expert, in pair_slot order (ascending (token, k)): the
+ * per-expert send slots laid end to end without their gaps.  The row of pair (t, k) is
+ * send_expert_prefix[topk_idx[t,k]] + pair_slot[t,k].
+ *   send_rows           [send_row_capacity] rows of deepep_ll_row_stride bytes (out); the first
+ *                       send_cumsum[R] are written; capacity >= min(T * K, E * M)
+ *   send_count          [E] int32 (out)      pairs per expert, clamped to M
+ *   send_expert_prefix  [E + 1] int32 (out)  exclusive prefix of send_count; [E] = rows sent
+ *   send_counts         [R] int32 (out)      rows for each destination rank
+ *   send_cumsum         [R + 1] int64 (out)  their exclusive prefix: the message for rank d is rows
+ *                       [send_cumsum[d], send_cumsum[d + 1])
+ *   pair_slot           [T, K] int32 (out)   as deepep_ll_dispatch_send
+ *   workspace           deepep_ll_dispatch_workspace_bytes(T, K, E) bytes
+ * Stacked over the ranks, send_count is the all_num_routed of deepep_ll_exchange_metadata.
+ * Replaces ll_dispatch_route_and_pack_v3 (csrc/kernels/efa_kernels.cu:2332-2400: send_counts,
+ * send_cumsum, rows grouped by destination rank; row tail :797-800), whose output
+ * dist.all_to_all_single ships (deep_ep/buffer.py:2297-2301).  The reference leaves the order inside
+ * a destination's message to an atomic (:2378-2380); here it is fixed as above. */
+int deepep_ll_dispatch_send_by_dest(const void* x, const int64_t* topk_idx,
+                                    int num_tokens, int hidden, int num_topk, int num_experts,
+                                    int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                                    int row_format, void* send_rows, int64_t send_row_capacity,
+                                    int32_t* send_count, int32_t* send_expert_prefix,
+                                    int32_t* send_counts, int64_t* send_cumsum, int32_t* pair_slot,
+                                    void* workspace, size_t workspace_bytes, void* stream);
+
 /* Receive side: compacts the staged rows of every (local expert, source
  * rank) segment into the packed layout.
  *   begin(e,s) = sum_{s' < s} recv_count[e,s'];  rows [begin, begin+cnt)
@@ -330,7 +366,13 @@ size_t deepep_ll_by_source_workspace_bytes(int num_experts, int64_t row_capacity
  *   source_offset   [row_capacity] uint32 row index of each record  } deepep_ll_exchange_metadata
  *   num_recv_tokens [2] uint32: [1] = records present               }
  *   tokens_per_expert [E_l] uint32 (out) = packed_recv_count, or NULL
+ *   record_packed_row [row_capacity] int32 (out) or NULL: for record i, the packed row its row was copied
+ *                   to, local_expert * N + position, or -1 if it got none (past its source's slot, no valid
+ *                   expert in its tail, past its pair's M rows) -- the reference's recv_expert_ids /
+ *                   recv_expert_pos (csrc/kernels/efa_kernels.cu:2121-2231), which the combine needs to
+ *                   return the rows in arrival order (deepep_ll_combine_send_by_dest)
  *   workspace       deepep_ll_by_source_workspace_bytes(E, row_capacity) bytes
+ * An (expert, source) pair takes at most M rows, as a segment of the staged form does.
  * Replaces ll_recv_unpack_v2 on its flat / slotted input (csrc/kernels/efa_kernels.cu:2121-2231,
  * kernels :877-1052 and :1227-1389, slot addressing :906-913) and consumes the records
  * a2a_dispatch_recv reads (csrc/kernels/coop_dispatch_recv.cuh:42, source_offset). */
@@ -343,7 +385,7 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
                                       int32_t* packed_recv_src_info, int64_t* packed_recv_layout_range,
                                       int32_t* packed_recv_count,
                                       int32_t* cumulative_local_expert_recv_stats,
-                                      uint32_t* tokens_per_expert,
+                                      uint32_t* tokens_per_expert, int32_t* record_packed_row,
                                       void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ */
@@ -383,6 +425,58 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
                            const float* topk_weights, const int32_t* pair_slot,
                            int num_tokens, int hidden, int num_topk, int num_experts,
                            int num_max_dispatch_tokens_per_rank, int accumulate, void* out, void* stream);
+
+/* Send side for an all-to-all shaped transport: every live expert-output row, in arrival order --
+ * which is contiguous per destination rank -- in one flat buffer.  For record i of
+ * deepep_ll_exchange_metadata (i < num_recv_tokens[1]):
+ *   send_flat[combine_send_offset[i], :] = x_rows[record_packed_row[padded_index[i]], :]
+ * with x_rows the [E_l * N, H] view of the expert outputs.  The message for rank s is then rows
+ * [prefix(recv_counts)[s], prefix(recv_counts)[s + 1]) of send_flat.  A record whose packed row is -1
+ * leaves its row untouched.
+ *   x                  [E_l, N, H] bf16 expert outputs
+ *   record_packed_row  [row_capacity] int32 from deepep_ll_dispatch_recv_by_source
+ *   source_rank, padded_index, combine_send_offset [row_capacity] uint32, num_recv_tokens [2] uint32:
+ *                      the records of deepep_ll_exchange_metadata
+ *   send_flat          [row_capacity, H] bf16 (out); may be NULL with peer_recv_flat
+ * Direct delivery (peer_recv_flat != NULL): when the destination ranks' receive buffers are mapped
+ * into this GPU's address space (peers on the same node), the row skips send_flat and is stored
+ * where the all-to-all would have put it: row combine_remote_recv_offset[s] + j of rank s's buffer, j
+ * being the record's place among the rows of source s = source_rank[i].
+ *   recv_counts                 [R] int32     } outputs of deepep_ll_exchange_metadata
+ *   combine_remote_recv_offset  [R] int64     }
+ *   peer_recv_flat  [R] device array of pointers to the ranks' receive buffers (the buffer
+ *                   deepep_ll_combine_recv_flat reads, flat form), peer_recv_rows [R] int64 their rows
+ * Replaces the gather + un-sort of deep_ep/buffer.py:2601-2608 and a2a_combine_send
+ * (csrc/kernels/coop_combine_send.cuh:37-275: send_buffer[combine_send_offset[i]] =
+ * expert_x[padded_index[i]], peer stores :205-246); landing offset
+ * csrc/transport/ll_pipeline.cpp:1283-1295. */
+int deepep_ll_combine_send_by_dest(const void* x, const int32_t* record_packed_row,
+                                   const uint32_t* source_rank, const uint32_t* padded_index,
+                                   const uint32_t* combine_send_offset, const uint32_t* num_recv_tokens,
+                                   int64_t row_capacity, int hidden, int num_experts, int num_ranks,
+                                   int num_max_dispatch_tokens_per_rank, void* send_flat,
+                                   const int32_t* recv_counts, const int64_t* combine_remote_recv_offset,
+                                   void* const* peer_recv_flat, const int64_t* peer_recv_rows,
+                                   void* stream);
+
+/* deepep_ll_combine_recv reading the answers from the buffer an all-to-all leaves them in: one row
+ * per row this rank sent, in send order (deepep_ll_dispatch_send_by_dest), so that pair (t, k) is
+ * answered by row send_expert_prefix[topk_idx[t,k]] + pair_slot[t,k].
+ *   recv_flat           [recv_flat_rows, H] bf16
+ *   slot_rows           0: the rows lie back to back (flat).  > 0: the answers of rank r start at row
+ *                       r * slot_rows (one fixed slot per answering rank; the reference's slot_size,
+ *                       in rows) and a pair's row is r * slot_rows + (its send index - the first
+ *                       send index of rank r)
+ *   send_expert_prefix  [E + 1] int32 from deepep_ll_dispatch_send_by_dest
+ *   other arguments and the arithmetic as deepep_ll_combine_recv.
+ * Replaces ll_combine_weighted_reduce_v2 on its flat / slotted input
+ * (csrc/kernels/efa_kernels.cu:1982-2031, kernel :1413-1474, addressing :1449-1466). */
+int deepep_ll_combine_recv_flat(const void* recv_flat, int64_t recv_flat_rows, int64_t slot_rows,
+                                const int32_t* send_expert_prefix, const int64_t* topk_idx,
+                                const float* topk_weights, const int32_t* pair_slot,
+                                int num_tokens, int hidden, int num_topk, int num_experts,
+                                int num_ranks, int num_max_dispatch_tokens_per_rank, int accumulate,
+                                void* out, void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Whole dispatch / whole combine in one call                          */
@@ -481,16 +575,6 @@ int deepep_loopback_dispatch_from_peers(const void* x, const int64_t* topk_idx,
                                         int num_max_dispatch_tokens_per_rank, int row_format,
                                         void* recv_staging, int32_t* recv_count,
                                         void* workspace, size_t workspace_bytes, void* stream);
-
-/* A measuring stick, not part of the path (no counterpart in the reference): reads T rows of
- * 2 * hidden bytes and writes, for every token, `hidden` bytes (the two halves of each 32 bytes
- * folded together) to each of its K destination rows — the memory traffic of the dispatch send side
- * at one byte per element, with no routing, quantisation or scales.  bench.py times it beside the
- * send kernel on the same destinations: what it reaches is what this access pattern gets from HBM.
- *   x         [T, hidden] 2-byte elements       dst_rows  [T, K] int32 row index, -1 = none
- *   dst       rows of dst_stride_bytes, the first `hidden` bytes of each named row written */
-int deepep_probe_row_scatter(const void* x, int num_tokens, int hidden, const int32_t* dst_rows, int num_topk,
-                             void* dst, int64_t dst_stride_bytes, void* stream);
 
 /* Plays the remote experts for this rank's own pairs: for every remote
  * expert e and slot j < send_count[e] writes combine_staging[e, j, :].

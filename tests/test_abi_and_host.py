@@ -26,7 +26,21 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in include/deepep_hip.h but not exported"
         assert name in _capi.PROTOTYPES, f"{name} has no ctypes prototype"
     assert sorted(_capi.PROTOTYPES) == declared
-    assert lib.deepep_abi_version() == 9
+
+
+def test_abi_revision_is_the_same_everywhere():
+    """The header's revision, what the built library reports and what the integration notes tell a
+    maintainer to gate on are one number."""
+    from deepep_efa_amd import _capi
+    header = open(os.path.join(ROOT, "include", "deepep_hip.h")).read()
+    revision = int(re.search(r"#define\s+DEEPEP_HIP_ABI_VERSION\s+(\d+)", header).group(1))
+    assert _capi.load().deepep_abi_version() == revision
+    notes = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    assert re.search(r"`deepep_abi_version\(\)` is (\d+)", notes).group(1) == str(revision)
+    # every *_workspace_bytes function the header declares is named there too
+    for name in _declared_symbols():
+        if name.endswith("_workspace_bytes"):
+            assert name in notes, f"INTEGRATION.md does not mention {name}"
 
 
 @pytest.mark.parametrize("hidden", [128, 512, 2048, 7168])
@@ -57,7 +71,7 @@ def test_host_argument_checks_without_a_gpu():
         int(re.search(r"cast\.hip:(\d+)", lib.deepep_last_error().decode()).group(1))
     rc = lib.deepep_ll_combine_recv(None, None, None, None, 4, 7168, 0, 256, 128, 0, None, None)
     assert rc != 0 and "num_topk > 0" in lib.deepep_last_error().decode()
-    rc = lib.deepep_moe_routing_sort(None, -1, 8, None, None, None, None, 0, None)
+    rc = lib.deepep_moe_routing_sort(None, -1, 8, None, None, None, None, None, 0, None)
     assert rc != 0 and lib.deepep_last_error().decode().startswith("Failed: Assertion error layout.hip:")
     with pytest.raises(_capi.DeepEPError):
         _capi.check(rc)

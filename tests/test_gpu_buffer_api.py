@@ -43,22 +43,19 @@ def reference_world(num_ranks, num_tokens, hidden, num_experts, num_topk, seed):
     return torch.stack(xs), torch.stack(tks), torch.stack(ws)
 
 
-@pytest.mark.parametrize("num_ranks,rank,num_tokens,hidden,num_topk,num_experts",
-                         [(8, 2, 128, 2048, 8, 288), (16, 15, 64, 7168, 8, 256),
-                          (4, 1, 2100, 512, 8, 64)])  # a prefill-sized batch: histograms + send, index + flat copies
-def test_low_latency_as_the_reference_tests_it(deep_ep, num_ranks, rank, num_tokens, hidden, num_topk, num_experts):
-    assert num_experts % num_ranks == 0
+def reference_test_main(deep_ep, buffer, num_ranks, rank, num_tokens, hidden, num_topk, num_experts, seed, check=True,
+                        cache=None):
+    """The body of the reference's test_main (tests/test_low_latency.py:38-193) for one rank: every payload
+    format, both completion styles, two inputs; returns the XOR of the hashes of every output (:118-193).
+    check=False repeats the calls and the hashing only (the pressure loop, :316-329), taking the experts'
+    outputs from `cache`, which a checking run filled."""
     num_local_experts = num_experts // num_ranks
-    x_all, topk_all, w_all = reference_world(num_ranks, num_tokens, hidden, num_experts, num_topk, seed=1)
+    x_all, topk_all, w_all = reference_world(num_ranks, num_tokens, hidden, num_experts, num_topk, seed=seed)
     x_rand = (torch.randn((num_tokens, hidden), generator=torch.Generator().manual_seed(5)) * 0.1).to(torch.bfloat16)
-
-    num_rdma_bytes = deep_ep.Buffer.get_low_latency_rdma_size_hint(num_tokens, hidden, num_ranks, num_experts)
-    buffer = deep_ep.Buffer(None, num_rdma_bytes=num_rdma_bytes, low_latency_mode=True,
-                            num_qps_per_rank=num_local_experts, explicitly_destroy=True,
-                            sim_num_ranks=num_ranks, sim_rank=rank)
     topk_idx = topk_all[rank].cuda().to(deep_ep.topk_idx_t)
     topk_weights = w_all[rank].cuda()
     all_topk_idx = topk_all
+    cache = {} if cache is None else cache
 
     hash_value, num_times, hashes = 0, 0, {}
     for which, x_cpu in (("const", x_all[rank]), ("rand", x_rand)):
@@ -80,59 +77,65 @@ def test_low_latency_as_the_reference_tests_it(deep_ep, num_ranks, rank, num_tok
                                 return_recv_hook=return_recv_hook, topk_weights=topk_weights)
                             hook() if return_recv_hook else event.current_stream_wait()
                         torch.cuda.synchronize()
-                        if use_fp8:
-                            assert packed_recv_x[0].dtype == torch.float8_e4m3fn
-                            assert packed_recv_x[0].shape == (num_local_experts, num_ranks * num_tokens, hidden)
-                            want_scale = (hidden // 512, torch.int32) if use_ue8m0 else (hidden // 128, torch.float32)
-                            assert packed_recv_x[1].shape[-1] == want_scale[0] and packed_recv_x[1].dtype == want_scale[1]
-                            fp8_cpu, scales_cpu = packed_recv_x[0].cpu(), packed_recv_x[1].cpu()
-                        else:
-                            assert packed_recv_x.dtype == torch.bfloat16
-                            recv_cpu = packed_recv_x.cpu()
                         count_cpu = packed_recv_count.cpu()
-                        src_info_cpu, layout_cpu = handle[0].cpu(), handle[1].cpu()
-                        assert handle[2:] == (num_tokens, hidden, num_experts)
-                        assert src_info_cpu.dtype == torch.int32 and layout_cpu.shape == (num_local_experts, num_ranks)
-                        simulated = torch.zeros((num_local_experts, num_ranks * num_tokens, hidden), dtype=torch.bfloat16)
                         key = (which, use_fp8, round_scale, use_ue8m0)
                         h = 0
-                        for i in range(num_local_experts):
-                            expert_id = rank * num_local_experts + i
+                        for i in range(num_local_experts):  # the hash of what arrived, taken where it lies
                             n = int(count_cpu[i])
-                            lr = layout_cpu[i]
-                            int_mask = (2 ** 32) - 1
-                            assert int(stats[i]) == n
-                            assert n == int((lr & int_mask).sum())
-                            assert n == int((all_topk_idx == expert_id).sum())
                             if n == 0:
                                 continue
                             if use_fp8:
-                                recv_x = O.per_token_cast_back(fp8_cpu[i, :n], scales_cpu[i, :n])
+                                h ^= hash_tensor(packed_recv_x[0][i, :n]) ^ hash_tensor(packed_recv_x[1][i, :n])
                             else:
-                                recv_x = recv_cpu[i, :n]
-                            simulated[i, :n] = recv_x
-                            src = src_info_cpu[i, :n]
-                            if which == "const":
-                                rf = recv_x.float()
-                                amin = rf[:, :-128].amin(dim=-1)
-                                assert torch.equal(amin, rf[:, :-128].amax(dim=-1))
-                                if round_scale:
-                                    assert O.calc_diff(rf[:, -1], src.float()) < 0.007
-                                else:
-                                    # the recipe stores the token index as bf16 (exact up to 256 tokens)
-                                    stored = (src % num_tokens).to(torch.bfloat16).float().view(-1, 1)
-                                    assert (rf[:, -128:] - stored).sum().item() == 0
-                                for j in range(num_ranks):
-                                    begin, cnt = int(lr[j] >> 32), int(lr[j] & int_mask)
-                                    if not round_scale:
-                                        assert int((amin == j - 128).sum()) == int((all_topk_idx[j] == expert_id).sum())
-                                        assert (rf[begin:begin + cnt, :-128] - j + 128).sum().item() == 0
+                                h ^= hash_tensor(packed_recv_x[i, :n])
+                        if check:
                             if use_fp8:
-                                h ^= hash_tensor(fp8_cpu[i, :n]) ^ hash_tensor(scales_cpu[i, :n])
+                                assert packed_recv_x[0].dtype == torch.float8_e4m3fn
+                                assert packed_recv_x[0].shape == (num_local_experts, num_ranks * num_tokens, hidden)
+                                want_scale = (hidden // 512, torch.int32) if use_ue8m0 else (hidden // 128, torch.float32)
+                                assert packed_recv_x[1].shape[-1] == want_scale[0] and packed_recv_x[1].dtype == want_scale[1]
+                                fp8_cpu, scales_cpu = packed_recv_x[0].cpu(), packed_recv_x[1].cpu()
                             else:
-                                h ^= hash_tensor(recv_cpu[i, :n])
+                                assert packed_recv_x.dtype == torch.bfloat16
+                                recv_cpu = packed_recv_x.cpu()
+                            src_info_cpu, layout_cpu = handle[0].cpu(), handle[1].cpu()
+                            assert handle[2:] == (num_tokens, hidden, num_experts)
+                            assert src_info_cpu.dtype == torch.int32 and layout_cpu.shape == (num_local_experts, num_ranks)
+                            simulated = torch.zeros((num_local_experts, num_ranks * num_tokens, hidden), dtype=torch.bfloat16)
+                            for i in range(num_local_experts):
+                                expert_id = rank * num_local_experts + i
+                                n = int(count_cpu[i])
+                                lr = layout_cpu[i]
+                                int_mask = (2 ** 32) - 1
+                                assert int(stats[i]) == n
+                                assert n == int((lr & int_mask).sum())
+                                assert n == int((all_topk_idx == expert_id).sum())
+                                if n == 0:
+                                    continue
+                                if use_fp8:
+                                    recv_x = O.per_token_cast_back(fp8_cpu[i, :n], scales_cpu[i, :n])
+                                else:
+                                    recv_x = recv_cpu[i, :n]
+                                simulated[i, :n] = recv_x
+                                src = src_info_cpu[i, :n]
+                                if which == "const":
+                                    rf = recv_x.float()
+                                    amin = rf[:, :-128].amin(dim=-1)
+                                    assert torch.equal(amin, rf[:, :-128].amax(dim=-1))
+                                    if round_scale:
+                                        assert O.calc_diff(rf[:, -1], src.float()) < 0.007
+                                    else:
+                                        # the recipe stores the token index as bf16 (exact up to 256 tokens)
+                                        stored = (src % num_tokens).to(torch.bfloat16).float().view(-1, 1)
+                                        assert (rf[:, -128:] - stored).sum().item() == 0
+                                    for j in range(num_ranks):
+                                        begin, cnt = int(lr[j] >> 32), int(lr[j] & int_mask)
+                                        if not round_scale:
+                                            assert int((amin == j - 128).sum()) == int((all_topk_idx[j] == expert_id).sum())
+                                            assert (rf[begin:begin + cnt, :-128] - j + 128).sum().item() == 0
+                            cache[key] = simulated.cuda()
                         # combine, with and without the zero-copy buffer
-                        sim_dev = simulated.cuda()
+                        sim_dev = cache[key]
                         for zero_copy in (False, True):
                             if zero_copy:
                                 buffer.get_next_low_latency_combine_buffer(handle)[:, :, :] = sim_dev
@@ -142,18 +145,53 @@ def test_low_latency_as_the_reference_tests_it(deep_ep, num_ranks, rank, num_tok
                                 zero_copy=zero_copy, return_recv_hook=return_recv_hook, out=out)
                             hook() if return_recv_hook else event.current_stream_wait()
                             torch.cuda.synchronize()
-                            assert combined_x.data_ptr() == out.data_ptr()
-                            want = x_cpu.float() * topk_weights.cpu().masked_fill(topk_idx.cpu() == -1, 0).sum(dim=1).view(-1, 1)
-                            diff = O.calc_diff(want, combined_x.cpu())
-                            assert torch.isnan(combined_x.float()).sum().item() == 0
-                            if not round_scale:
-                                assert diff < (9e-4 if use_fp8 else 1e-5), f"{diff=} {use_fp8=} {zero_copy=}"
-                            h ^= hash_tensor(combined_x.cpu())
+                            if check:
+                                assert combined_x.data_ptr() == out.data_ptr()
+                                want = x_cpu.float() * topk_weights.cpu().masked_fill(topk_idx.cpu() == -1, 0).sum(dim=1).view(-1, 1)
+                                diff = O.calc_diff(want, combined_x.cpu())
+                                assert torch.isnan(combined_x.float()).sum().item() == 0
+                                if not round_scale:
+                                    assert diff < (9e-4 if use_fp8 else 1e-5), f"{diff=} {use_fp8=} {zero_copy=}"
+                            h ^= hash_tensor(combined_x)
                         # the same inputs give the same bytes on every call (tests/test_low_latency.py:319-329)
                         if key in hashes:
                             assert hashes[key] == h
                         hashes[key] = h
                         hash_value ^= h
+    return hash_value
+
+
+@pytest.mark.parametrize("num_ranks,rank,num_tokens,hidden,num_topk,num_experts",
+                         [(8, 2, 128, 2048, 8, 288), (16, 15, 64, 7168, 8, 256),
+                          (4, 1, 2100, 512, 8, 64)])  # a prefill-sized batch: histograms + send, index + flat copies
+def test_low_latency_as_the_reference_tests_it(deep_ep, num_ranks, rank, num_tokens, hidden, num_topk, num_experts):
+    assert num_experts % num_ranks == 0
+    num_rdma_bytes = deep_ep.Buffer.get_low_latency_rdma_size_hint(num_tokens, hidden, num_ranks, num_experts)
+    buffer = deep_ep.Buffer(None, num_rdma_bytes=num_rdma_bytes, low_latency_mode=True,
+                            num_qps_per_rank=num_experts // num_ranks, explicitly_destroy=True,
+                            sim_num_ranks=num_ranks, sim_rank=rank)
+    reference_test_main(deep_ep, buffer, num_ranks, rank, num_tokens, hidden, num_topk, num_experts, seed=1)
+    buffer.clean_low_latency_buffer(num_tokens, hidden, num_experts)
+    buffer.destroy()
+
+
+def test_pressure_every_rerun_hashes_the_same(deep_ep):
+    """The reference's pressure check (tests/test_low_latency.py:316-329) at the headline shape, one rank of
+    EP=32 with 128 tokens x 7168 and top-8 of 256 experts: test_main once for the reference hash, then twenty
+    more times, and every rerun must hash every output to the same value; the loop stops at the first that
+    does not.  No kernel on this path claims a slot or adds with an atomic in HBM, so nothing depends on
+    scheduling."""
+    num_ranks, rank, num_tokens, hidden, num_topk, num_experts = 32, 5, 128, 7168, 8, 256
+    buffer = deep_ep.Buffer(None, low_latency_mode=True, num_qps_per_rank=num_experts // num_ranks,
+                            explicitly_destroy=True, sim_num_ranks=num_ranks, sim_rank=rank)
+    for seed in (0,):
+        experts_outputs = {}
+        ref_hash = reference_test_main(deep_ep, buffer, num_ranks, rank, num_tokens, hidden, num_topk, num_experts,
+                                       seed=seed, check=True, cache=experts_outputs)
+        for rerun in range(20):
+            got = reference_test_main(deep_ep, buffer, num_ranks, rank, num_tokens, hidden, num_topk, num_experts,
+                                      seed=seed, check=False, cache=experts_outputs)
+            assert got == ref_hash, f"Error: seed={seed} rerun={rerun}"
     buffer.clean_low_latency_buffer(num_tokens, hidden, num_experts)
     buffer.destroy()
 

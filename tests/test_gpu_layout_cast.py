@@ -90,11 +90,13 @@ def test_hand_derived_world_layout_sort_and_prefix(capi):
     counts = torch.full((r,), -1, dtype=torch.int32, device="cuda")
     cumsum = torch.full((r + 1,), -1, dtype=torch.int64, device="cuda")
     ws = torch.empty(max(16, lib.deepep_routing_sort_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
+    inverse = torch.full((max(1, t * r),), -7, dtype=torch.int32, device="cuda")
     capi.check(lib.deepep_moe_routing_sort(capi.ptr(dev), t, r, capi.ptr(ids), capi.ptr(counts), capi.ptr(cumsum),
-                                           capi.ptr(ws), ws.numel(), stream()))
+                                           capi.ptr(inverse), capi.ptr(ws), ws.numel(), stream()))
     torch.cuda.synchronize()
     assert counts.cpu().tolist() == want["send_counts"] and cumsum.cpu().tolist() == want["send_cumsum"]
     assert ids[:4].cpu().tolist() == want["sorted_token_ids"]
+    assert inverse[:t * r].view(t, r).cpu().tolist() == want["row_of_pair"]
     for c in (2, 3):
         cpm = torch.full((r, c), -1, dtype=torch.int32, device="cuda")
         capi.check(lib.deepep_channel_prefix_matrix(capi.ptr(dev), t, r, c, capi.ptr(cpm), stream()))
@@ -124,12 +126,14 @@ def test_routing_sort_channel_prefix(capi, t, r, p):
     counts = torch.full((r,), -1, dtype=torch.int32, device="cuda")
     cumsum = torch.full((r + 1,), -1, dtype=torch.int64, device="cuda")
     ws = torch.empty(max(16, lib.deepep_routing_sort_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
+    inverse = torch.full((max(1, t * r),), -7, dtype=torch.int32, device="cuda")
     capi.check(lib.deepep_moe_routing_sort(capi.ptr(dev), t, r, capi.ptr(ids), capi.ptr(counts), capi.ptr(cumsum),
-                                           capi.ptr(ws), ws.numel(), stream()))
+                                           capi.ptr(inverse), capi.ptr(ws), ws.numel(), stream()))
     torch.cuda.synchronize()
     w_ids, w_counts, w_cumsum, total = O.moe_routing_sort(is_in)
     assert torch.equal(counts.cpu(), w_counts) and torch.equal(cumsum.cpu(), w_cumsum)
     assert torch.equal(ids[:total].cpu(), w_ids)
+    assert torch.equal(inverse[:t * r].view(t, r).cpu(), _want_row_of_pair(is_in, w_ids, w_cumsum))
     for c in (10, 12, 1, 7):
         cpm = torch.full((r, c), -1, dtype=torch.int32, device="cuda")
         capi.check(lib.deepep_channel_prefix_matrix(capi.ptr(dev), t, r, c, capi.ptr(cpm), stream()))
@@ -158,12 +162,14 @@ def test_layout_sort_prefix_seeded_random_shapes(capi, seed):
     counts = torch.full((r,), -1, dtype=torch.int32, device="cuda")
     cumsum = torch.full((r + 1,), -1, dtype=torch.int64, device="cuda")
     ws = torch.empty(max(16, lib.deepep_routing_sort_workspace_bytes(t, r)), dtype=torch.uint8, device="cuda")
+    inverse = torch.full((max(1, t * r),), -7, dtype=torch.int32, device="cuda")
     capi.check(lib.deepep_moe_routing_sort(capi.ptr(dev), t, r, capi.ptr(ids), capi.ptr(counts), capi.ptr(cumsum),
-                                           capi.ptr(ws), ws.numel(), stream()))
+                                           capi.ptr(inverse), capi.ptr(ws), ws.numel(), stream()))
     torch.cuda.synchronize()
     w_ids, w_counts, w_cumsum, total = O.moe_routing_sort(is_in)
     assert torch.equal(counts.cpu(), w_counts) and torch.equal(cumsum.cpu(), w_cumsum)
     assert torch.equal(ids[:total].cpu(), w_ids) and (ids[total:] == -1).all()
+    assert torch.equal(inverse[:t * r].view(t, r).cpu(), _want_row_of_pair(is_in, w_ids, w_cumsum))
     c = int(g.choice([1, 3, 10, 12, 17, 40]))
     cpm = torch.full((r, c), -1, dtype=torch.int32, device="cuda")
     capi.check(lib.deepep_channel_prefix_matrix(capi.ptr(dev), t, r, c, capi.ptr(cpm), stream()))
@@ -276,6 +282,16 @@ def test_cast_argument_errors(capi):
 
 
 # ---- the steps either side of the normal-mode pack ------------------------------------------------
+def _want_row_of_pair(is_in, ids, cumsum):
+    """The inverse of the per-rank token list: where (token, rank) stands in it, -1 for non-members."""
+    t, r = is_in.shape
+    inv = torch.full((t, r), -1, dtype=torch.int32)
+    for rank in range(r):
+        lo, hi = int(cumsum[rank]), int(cumsum[rank + 1])
+        inv[ids[lo:hi], rank] = torch.arange(lo, hi, dtype=torch.int32)
+    return inv
+
+
 def _normal_world(t, k, e, r, seed, drop=3):
     topk = _topk(t, k, e, seed, drop)
     if t > 2:
@@ -341,12 +357,21 @@ def test_combine_reduce(capi, t, k, e, r, h, with_bias):
     out_w = torch.full((t, k), float("nan"), dtype=torch.float32, device="cuda")
     ws = torch.full((max(256, lib.deepep_combine_reduce_workspace_bytes(t, r)),), 0x7F, dtype=torch.uint8, device="cuda")
     dev = [None if v is None else v.cuda() for v in (rows, rw, ids, cumsum, is_in, b0, b1)]  # outlive the launch
-    capi.check(lib.deepep_combine_reduce(*[capi.ptr(v) for v in dev], t, h, k, r, total, capi.ptr(out_x),
+    capi.check(lib.deepep_combine_reduce(*[capi.ptr(v) for v in dev], t, h, k, r, total, None, capi.ptr(out_x),
                                          capi.ptr(out_w), capi.ptr(ws), ws.numel(), stream()))
     torch.cuda.synchronize()
     chain_x, chain_w = O.combine_reduce_f32_chain(rows, rw, ids, cumsum, t, b0, b1)
     assert torch.equal(out_x.cpu().view(torch.int16), chain_x.view(torch.int16))
     assert torch.equal(out_w.cpu(), chain_w)
+    # with the table the routing sort leaves: one launch, no workspace, the same bits
+    table = _want_row_of_pair(is_in, ids, cumsum).cuda()
+    out_x2 = torch.empty_like(out_x)
+    out_x2.view(torch.int16).fill_(0x7FC0)
+    out_w2 = torch.full_like(out_w, float("nan"))
+    capi.check(lib.deepep_combine_reduce(*[capi.ptr(v) for v in dev], t, h, k, r, total, capi.ptr(table),
+                                         capi.ptr(out_x2), capi.ptr(out_w2), None, 0, stream()))
+    torch.cuda.synchronize()
+    assert torch.equal(out_x2.view(torch.int16), out_x.view(torch.int16)) and torch.equal(out_w2, out_w)
     ref_x, ref_w = O.combine_reduce(rows, rw, ids, t, b0, b1)
     err = (out_x.cpu().double() - ref_x).abs()
     assert (err <= 1e-2 * ref_x.abs() + 1e-2 * ref_x.abs().mean()).all()
@@ -402,8 +427,9 @@ def test_pack_remap_reduce_seeded_random_shapes(capi, seed):
     out_cw = torch.full((t, k), float("nan"), dtype=torch.float32, device="cuda")
     ws = torch.full((max(256, lib.deepep_combine_reduce_workspace_bytes(t, r)),), 0x7F, dtype=torch.uint8, device="cuda")
     held = [None if v is None else v.cuda() for v in (rows, want_w, ids, cumsum, is_in, b0, b1)]
-    capi.check(lib.deepep_combine_reduce(*[capi.ptr(v) for v in held], t, h, k, r, total, capi.ptr(out_x),
-                                         capi.ptr(out_cw), capi.ptr(ws), ws.numel(), stream()))
+    table = _want_row_of_pair(is_in, ids, cumsum).cuda() if seed % 2 else None  # with and without the sort's table
+    capi.check(lib.deepep_combine_reduce(*[capi.ptr(v) for v in held], t, h, k, r, total, capi.ptr(table),
+                                         capi.ptr(out_x), capi.ptr(out_cw), capi.ptr(ws), ws.numel(), stream()))
     torch.cuda.synchronize()
     chain_x, chain_w = O.combine_reduce_f32_chain(rows, want_w, ids, cumsum, t, b0, b1)
     assert torch.equal(out_x.cpu().view(torch.int16), chain_x.view(torch.int16))
@@ -426,6 +452,11 @@ def test_normal_mode_steps_through_the_host_module():
     x = torch.randn((t, h), generator=torch.Generator().manual_seed(2)).to(torch.bfloat16)
     send_x, _ = normal.pack_rows(x.cuda(), None, ids_d, cumsum_d)
     cx, cw = normal.combine_reduce(send_x, rw, ids_d, cumsum_d, is_in.cuda())
+    ids_p, counts_p, cumsum_p, total_p, row_of_pair = normal.moe_routing_sort_with_positions(is_in.cuda())
+    assert total_p == total and torch.equal(ids_p, ids_d) and torch.equal(cumsum_p, cumsum_d)
+    assert torch.equal(row_of_pair.cpu(), _want_row_of_pair(is_in, ids, cumsum))
+    cx2, cw2 = normal.combine_reduce(send_x, rw, ids_d, cumsum_d, is_in.cuda(), row_of_pair=row_of_pair)
+    assert torch.equal(cx2.view(torch.int16), cx.view(torch.int16)) and torch.equal(cw2, cw)
     # remapped weights are zero outside the destination's experts, so their sum is the original weight row
     want_cw = torch.where(topk >= 0, w, torch.zeros_like(w))
     assert torch.allclose(cw.cpu(), want_cw, rtol=1e-6, atol=1e-7)
@@ -438,7 +469,8 @@ def test_normal_mode_steps_through_the_host_module():
 def test_row_scatter_probe(capi):
     """The bare read-rows / store-K-copies kernel bench.py times beside the send side: every named row gets
     the fold of its token's row, every other byte is left alone."""
-    lib = capi.load()
+    import bench
+    probe = bench.load_bench_probe()
     t, h, k, rows, stride = 37, 512, 3, 200, 640
     g = torch.Generator().manual_seed(5)
     x = torch.randint(0, 2 ** 16, (t, h), generator=g, dtype=torch.int32).to(torch.uint16)
@@ -446,8 +478,8 @@ def test_row_scatter_probe(capi):
     dst_rows[::5, 1] = -1
     dst = torch.full((rows, stride), 0xEE, dtype=torch.uint8, device="cuda")
     x_dev, rows_dev = x.cuda(), dst_rows.cuda()
-    capi.check(lib.deepep_probe_row_scatter(capi.ptr(x_dev), t, h, capi.ptr(rows_dev), k, capi.ptr(dst), stride,
-                                            stream()))
+    assert probe.bench_probe_row_scatter(capi.ptr(x_dev), t, h, capi.ptr(rows_dev), k, capi.ptr(dst), stride,
+                                         stream()) == 0
     torch.cuda.synchronize()
     words = x.view(torch.uint8).view(t, h // 16, 2, 16)          # 32 bytes per thread: two 16-byte vectors
     fold = (words[:, :, 0] ^ words[:, :, 1]).reshape(t, h)       # one vector out

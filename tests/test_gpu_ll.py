@@ -280,7 +280,7 @@ def recv_by_source_on_gpu(rt, buf, routed, rank, e, m, h, fmt, slot_rows, capaci
         capi.ptr(dev), slot_rows, capi.ptr(meta["recv_counts"]), capi.ptr(meta["source_offset"]),
         capi.ptr(meta["num_recv_tokens"]), capacity, h, e, r, m, fmt, capi.ptr(st.packed_recv_x),
         capi.ptr(st.packed_recv_scales), capi.ptr(st.packed_recv_src_info), capi.ptr(st.packed_recv_layout_range),
-        capi.ptr(st.packed_recv_count), None, capi.ptr(tokens_per_expert), capi.ptr(ws), ws.numel(),
+        capi.ptr(st.packed_recv_count), None, capi.ptr(tokens_per_expert), None, capi.ptr(ws), ws.numel(),
         torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     return st, tokens_per_expert, meta
@@ -959,7 +959,8 @@ def test_every_rank_on_one_gpu_through_an_all_to_all(rt, fmt):
             capi.ptr(buf), slot_rows, capi.ptr(meta["recv_counts"]), capi.ptr(meta["source_offset"]),
             capi.ptr(meta["num_recv_tokens"]), capacity, h, e, r, t, fmt, capi.ptr(st.packed_recv_x),
             capi.ptr(st.packed_recv_scales), capi.ptr(st.packed_recv_src_info), capi.ptr(st.packed_recv_layout_range),
-            capi.ptr(st.packed_recv_count), None, None, capi.ptr(ws), ws.numel(), torch.cuda.current_stream().cuda_stream))
+            capi.ptr(st.packed_recv_count), None, None, None, capi.ptr(ws), ws.numel(),
+            torch.cuda.current_stream().cuda_stream))
         torch.cuda.synchronize()
         want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
         check_dispatch(st, want, fmt)
@@ -1006,3 +1007,298 @@ def test_combine_without_row_return_reduces_the_same(rt, r, rank, t, h, k, e):
         touched = bool((st.combine_send_slots.view(torch.int16) != 0x7FC0).any())
         assert touched != zero_copy
     assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+
+
+# ---------------------------------------------------------------------------------------------
+# The all-to-all shaped transport: one contiguous message per peer in both directions
+# ---------------------------------------------------------------------------------------------
+def send_by_dest_on_gpu(rt, x, topk, rank, r, e, m, fmt):
+    t, h = x.shape
+    k = topk.shape[1]
+    st = rt.ll.AllToAllState(rt.ll.LLShape(r, rank, e, m, h, k, fmt))
+    st.send_rows.fill_(0xEE)
+    st.pair_slot.fill_(-7)
+    for name in ("send_count", "send_expert_prefix", "send_counts", "send_cumsum"):
+        getattr(st, name).fill_(-7)
+    st.dispatch_send(x.cuda(), topk.cuda())
+    torch.cuda.synchronize()
+    return st
+
+
+def check_send_by_dest(st, want, t):
+    payload = st.lib.deepep_ll_row_payload_bytes(st.shape.hidden, st.shape.fmt)
+    assert torch.equal(st.send_count.cpu(), want["send_count"])
+    assert torch.equal(st.send_expert_prefix.cpu(), want["send_expert_prefix"])
+    assert torch.equal(st.send_counts.cpu(), want["send_counts"])
+    assert torch.equal(st.send_cumsum.cpu(), want["send_cumsum"])
+    assert torch.equal(st.pair_slot[:t].cpu(), want["pair_slot"])
+    n = want["rows"].shape[0]
+    got = st.send_rows.cpu()
+    h, fmt = st.shape.hidden, st.shape.fmt
+    db, sb = O.row_data_bytes(h, fmt), O.row_scale_bytes(h, fmt)
+    dp, sp = O.align_up(db, 16), O.align_up(sb, 16)
+    touched = torch.zeros(got.shape[1], dtype=torch.bool)
+    for lo, hi in ((0, db), (dp, dp + sb), (dp + sp, dp + sp + 16)):  # data, scales, tail: the padding is nobody's
+        assert torch.equal(got[:n, lo:hi], want["rows"][:, lo:hi]), (lo, hi)
+        touched[lo:hi] = True
+    assert payload == dp + sp + 16
+    assert (got[:n, ~touched] == 0xEE).all() and (got[n:] == 0xEE).all()  # nothing between the parts or behind the rows
+
+
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16, O.ROW_FP8_UE8M0])
+@pytest.mark.parametrize("r,rank,t,h,k,e", [
+    (4, 1, 8, 512, 3, 16), (8, 7, 33, 1024, 4, 64), (2, 0, 1, 512, 1, 2),
+    (32, 5, 128, 7168, 8, 256),  # the headline shape
+    (2, 0, 1100, 512, 8, 16),    # T * K > 8192: the tables come from the chunk histograms
+    (8, 5, 4200, 512, 4, 64),
+    (16, 9, 12, 512, 6, 1024),   # the most experts
+    (1, 0, 16, 512, 2, 4),       # a world of one rank
+    (4, 2, 24, 1536, 4, 16),     # hidden not a multiple of 1024
+    (512, 500, 3, 512, 2, 1024),
+])
+def test_send_by_dest(rt, fmt, r, rank, t, h, k, e):
+    """One buffer, contiguous per destination rank, rows by expert and slot; counts, prefixes and every
+    row byte against the oracle (csrc/kernels/efa_kernels.cu:2332-2400, row tail :797-800)."""
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=r * 17 + t, drop=min(5, t))
+    st = send_by_dest_on_gpu(rt, x_all[rank], topk_all[rank], rank, r, e, t, fmt)
+    check_send_by_dest(st, O.ll_send_by_dest(x_all[rank], topk_all[rank], rank, e, t, fmt, r), t)
+
+
+def test_send_by_dest_with_repeated_experts_and_full_pairs(rt):
+    """Tokens naming an expert more than once: pairs beyond a pair's M slots are dropped from the counts,
+    the prefixes and the buffer alike."""
+    r, rank, t, m, h, k, e = 2, 1, 6, 6, 256, 4, 4
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((t, h), generator=g).to(torch.bfloat16)
+    topk = torch.tensor([[2, 2, 0, -1], [2, 3, 3, 1], [3, 3, 3, 3], [2, 1, 2, 1], [-1, -1, 3, 3], [3, 3, 3, 3]])
+    st = send_by_dest_on_gpu(rt, x, topk, rank, r, e, m, O.ROW_FP8)
+    want = O.ll_send_by_dest(x, topk, rank, e, m, O.ROW_FP8, r)
+    assert int(want["send_count"][3]) == m and int((want["pair_slot"] == -1).sum()) > 3
+    check_send_by_dest(st, want, t)
+
+
+def all_to_all_dispatch(states, fmt):
+    """The dispatch all-to-all between ranks that share the GPU: the gathered counts, then one slice copy per
+    (source, destination) pair -- no regrouping of rows on the way."""
+    r = len(states)
+    routed = torch.stack([st.send_count for st in states])
+    cums = [st.send_cumsum.cpu().tolist() for st in states]
+    for d, dst in enumerate(states):
+        dst.recv_by_source.fill_(0xEE)
+        dst.exchange_metadata(routed)
+        for s, src in enumerate(states):
+            lo, hi = cums[s][d], cums[s][d + 1]
+            assert hi - lo <= dst.slot_rows
+            dst.recv_by_source[s * dst.slot_rows:s * dst.slot_rows + hi - lo] = src.send_rows[lo:hi]
+    return routed
+
+
+@pytest.mark.parametrize("delivery", ["flat", "slotted", "direct"])
+@pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
+@pytest.mark.parametrize("r,t,h,k,e", [(4, 40, 512, 3, 16), (8, 700, 512, 8, 64), (3, 5, 256, 2, 3)],
+                         ids=["small", "chunked_receive", "one_expert_per_rank"])
+def test_all_to_all_round_trip_on_one_gpu(rt, oracle_c, fmt, delivery, r, t, h, k, e):
+    """Every rank on the one GPU, the transport replaced by slice copies of contiguous ranges: send by
+    destination, exchange metadata from the gathered counts, receive by source, experts, return by
+    destination (into a flat buffer that is copied range by range, or -- `direct` -- straight into the
+    peers' receive buffers), reduce from the flat (or slotted) buffer.  Dispatch outputs bit-exact against
+    the oracle, per-record rows against its loops, the combine against the float32 chain.
+    (deep_ep/buffer.py:2266-2301,2601-2608,2735; csrc/transport/ll_pipeline.cpp:1204-1361)"""
+    epr = e // r
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=555 + r, drop=min(6, t))
+    states = []
+    for rank in range(r):
+        st = rt.ll.AllToAllState(rt.ll.LLShape(r, rank, e, t, h, k, fmt))
+        st.dispatch_send(x_all[rank].cuda(), topk_all[rank].cuda())
+        states.append(st)
+    torch.cuda.synchronize()
+    all_to_all_dispatch(states, fmt)
+    ys = []
+    for rank, st in enumerate(states):
+        poison_outputs_keep_pair_slot(st)
+        st.record_packed_row.fill_(-7)
+        st.dispatch_recv()
+        torch.cuda.synchronize()
+        want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
+        check_dispatch(st, want, fmt)
+        n = int(st.meta["num_recv_tokens"][1])
+        rec = O.ll_record_packed_rows(list(topk_all), rank, e, t)
+        assert n == rec.numel() and torch.equal(st.record_packed_row[:n].cpu().long(), rec)
+        assert (st.record_packed_row[n:] == -7).all()
+        # the experts: a seeded row per packed slot
+        y = torch.empty((epr, r * t, h), dtype=torch.bfloat16, device="cuda")
+        rt.capi.check(rt.capi.load().deepep_synth_bf16_rows(rt.capi.ptr(y), epr * r * t, h, h * 2, None, 0, 900 + rank,
+                                                            0, torch.cuda.current_stream().cuda_stream))
+        ys.append(y)
+    peer_table = torch.tensor([st.recv_flat.data_ptr() for st in states], dtype=torch.int64, device="cuda")
+    peer_rows = torch.tensor([st.recv_flat.shape[0] for st in states], dtype=torch.int64, device="cuda")
+    for st in states:
+        st.recv_flat.view(torch.int16).fill_(0x7FC0)
+        st.send_flat.view(torch.int16).fill_(0x7FC0)
+    for rank, st in enumerate(states):
+        if delivery == "direct":
+            st.combine_send(ys[rank], peer_table, peer_rows)
+        else:
+            st.combine_send(ys[rank])
+    torch.cuda.synchronize()
+    slot_rows = t * min(k, epr)
+    slotted = [torch.full((r * slot_rows, h), float("nan"), dtype=torch.bfloat16, device="cuda") for _ in states]
+    if delivery != "direct":  # the all-to-all back: one slice copy per (answering rank, asking rank) pair
+        cums = [st.send_cumsum.cpu().tolist() for st in states]
+        for d, ans in enumerate(states):
+            recv_counts = ans.meta["recv_counts"].cpu().tolist()
+            first = 0
+            for s, ask in enumerate(states):
+                n = recv_counts[s]
+                assert n == cums[s][d + 1] - cums[s][d]
+                assert int(ans.meta["combine_remote_recv_offset"][s]) == cums[s][d]
+                ask.recv_flat[cums[s][d]:cums[s][d] + n] = ans.send_flat[first:first + n]
+                slotted[s][d * slot_rows:d * slot_rows + n] = ans.send_flat[first:first + n]
+                first += n
+    else:
+        assert all((st.send_flat.view(torch.int16) == 0x7FC0).all() for st in states)  # nothing went the long way
+    for rank, st in enumerate(states):
+        topk, w = topk_all[rank], w_all[rank]
+        out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+        out.view(torch.int16).fill_(0x7FC0)
+        if delivery == "slotted":
+            st.combine_recv(topk.cuda(), w.cuda(), out, recv=slotted[rank], slot_rows=slot_rows)
+        else:
+            st.combine_recv(topk.cuda(), w.cuda(), out)
+        torch.cuda.synchronize()
+        # which seeded row answers each pair: the packed row the owner of the expert gave it
+        _, pair_slot = O.route(topk, e, t)
+        live = pair_slot >= 0
+        pair_rows = torch.zeros((t, k, h), dtype=torch.bfloat16)
+        for d in range(r):
+            lr = states[d].packed_recv_layout_range.cpu()
+            sel = live & (topk // epr == d)
+            ti, ki = torch.nonzero(sel, as_tuple=True)
+            if ti.numel() == 0:
+                continue
+            le = (topk[ti, ki] % epr)
+            begin = (lr[le, rank] >> 32)
+            keys = (le * (r * t) + begin + pair_slot[ti, ki].long()).numpy().astype(np.uint32)
+            pair_rows[ti, ki] = O.synth_bf16_rows(keys, h, 900 + d)
+        chain = torch.empty((t, h), dtype=torch.int16)
+        live8 = live.to(torch.uint8).contiguous()
+        oracle_c.oracle_combine_chain(ctypes.c_void_p(pair_rows.view(torch.int16).data_ptr()),
+                                      ctypes.c_void_p(w.contiguous().data_ptr()), ctypes.c_void_p(live8.data_ptr()),
+                                      t, k, h, ctypes.c_void_p(chain.data_ptr()))
+        assert torch.equal(out.cpu().view(torch.int16), chain), (rank, delivery)
+        ref = O.ll_combine(pair_rows, topk, w, live)
+        err = (out.cpu().double() - ref).abs()
+        assert (err <= 1e-2 * ref.abs() + 1e-2 * ref.abs().mean()).all()  # the 1e-2 bar against the float64 sum
+
+
+def test_all_to_all_hand_derived_world(rt):
+    """The same flow on the two-rank world worked out on paper (tests/golden/ll_tiny_world.json): message order,
+    tables, per-record packed rows, the flat buffers of both directions and the combined rows -- no oracle."""
+    g, x_all, topk_all = load_tiny_world()
+    e, m, h, t, k, r = g["num_experts"], g["max_tokens"], g["hidden"], g["num_tokens"], g["num_topk"], g["num_ranks"]
+    states = []
+    for rank in range(r):
+        st = rt.ll.AllToAllState(rt.ll.LLShape(r, rank, e, m, h, k, O.ROW_BF16))
+        st.dispatch_send(x_all[rank].cuda(), topk_all[rank].cuda())
+        states.append(st)
+    torch.cuda.synchronize()
+    tail_at = O.row_payload(h, O.ROW_BF16) - 16
+    for rank, st in enumerate(states):
+        want = g["send_by_dest"][f"rank{rank}"]
+        assert st.send_expert_prefix.cpu().tolist() == want["send_expert_prefix"]
+        assert st.send_counts.cpu().tolist() == want["send_counts"]
+        assert st.send_cumsum.cpu().tolist() == want["send_cumsum"]
+        n = want["send_cumsum"][-1]
+        tails = st.send_rows[:n, tail_at:tail_at + 16].cpu().contiguous().view(torch.int32)
+        assert tails[:, 0].tolist() == want["row_token"] and tails[:, 1].tolist() == want["row_topk_slot"]
+        assert tails[:, 3].tolist() == want["row_local_expert"]
+        slot = st.pair_slot[:t].cpu()
+        prefix = torch.tensor(want["send_expert_prefix"])
+        row = torch.where(slot >= 0, prefix[topk_all[rank].clamp(min=0)] + slot, torch.full_like(slot, -1))
+        assert row.tolist() == want["pair_send_row"]
+    all_to_all_dispatch(states, O.ROW_BF16)
+    for rank, st in enumerate(states):
+        st.dispatch_recv()
+        torch.cuda.synchronize()
+        rec = g["record_packed_row"][f"rank{rank}"]
+        assert st.record_packed_row[:len(rec)].cpu().tolist() == rec
+        want, layout = tiny_world_expected(g, f"rank{rank}_ascending")
+        assert st.packed_recv_count.cpu().tolist() == want["count"]
+        assert torch.equal(st.packed_recv_layout_range.cpu(), layout)
+        st.combine_send(st.packed_recv_x)  # identity experts
+        torch.cuda.synchronize()
+        flat = g["combine_send_flat_identity_experts"][f"rank{rank}"]
+        assert st.send_flat[:len(flat)].cpu().float()[:, 0].tolist() == flat
+    cums = [st.send_cumsum.cpu().tolist() for st in states]
+    for d, ans in enumerate(states):
+        recv_counts, first = ans.meta["recv_counts"].cpu().tolist(), 0
+        for s, ask in enumerate(states):
+            ask.recv_flat[cums[s][d]:cums[s][d] + recv_counts[s]] = ans.send_flat[first:first + recv_counts[s]]
+            first += recv_counts[s]
+    want_back = g["combine_recv_flat_rank0_identity_experts"]
+    assert states[0].recv_flat[:len(want_back)].cpu().float()[:, 0].tolist() == want_back
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    w = torch.tensor(g["topk_weights_rank0"], dtype=torch.float32, device="cuda")
+    states[0].combine_recv(topk_all[0].cuda(), w, out)
+    torch.cuda.synchronize()
+    expect = torch.tensor(g["combine_rank0_identity_experts"]).view(-1, 1).expand(-1, h)
+    assert torch.equal(out.cpu().float(), expect)
+
+
+@pytest.mark.parametrize("t", [24, 1500], ids=["one_workgroup_per_source", "chunked"])
+def test_dispatch_recv_by_source_clamps_a_pair_to_max_tokens(rt, t):
+    """Slots wider than M and senders that put more than M rows into one (expert, source) pair: the pair keeps
+    its first M rows in arrival order, the counts and ranges count only those, and an expert's ranges stay
+    inside its R * M packed slots -- what the staged receive does with an over-full count."""
+    r, rank, h, k, e, fmt = 2, 0, 512, 4, 8, O.ROW_FP8
+    m = t // 3  # what the receiver was built for; the senders route as if M were t
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=11, drop=0)
+    topk_all[1, :, :] = torch.tensor([0, 1, 2, 3])  # source 1: t rows for each of rank 0's experts
+    slot_rows = 4 * t
+    buf = rows_by_source(x_all, topk_all, rank, e, t, fmt, slot_rows)
+    routed = torch.stack([O.route(topk_all[s], e, t)[0] for s in range(r)]).to(torch.int32)
+    capacity = 8 * t
+    lib, capi = rt.capi.load(), rt.capi
+    meta = rt.ll.exchange_metadata(routed.clamp(max=slot_rows).cuda(), rank, slot_rows, capacity)
+    st = rt.ll.LowLatencyState(rt.ll.LLShape(r, rank, e, m, h, 1, fmt), keep_remote_rows=False)
+    poison_outputs(st)
+    ws = torch.empty(lib.deepep_ll_by_source_workspace_bytes(e, capacity), dtype=torch.uint8, device="cuda")
+    rec = torch.full((capacity,), -7, dtype=torch.int32, device="cuda")
+    capi.check(lib.deepep_ll_dispatch_recv_by_source(
+        capi.ptr(buf.cuda()), slot_rows, capi.ptr(meta["recv_counts"]), capi.ptr(meta["source_offset"]),
+        capi.ptr(meta["num_recv_tokens"]), capacity, h, e, r, m, fmt, capi.ptr(st.packed_recv_x),
+        capi.ptr(st.packed_recv_scales), capi.ptr(st.packed_recv_src_info), capi.ptr(st.packed_recv_layout_range),
+        capi.ptr(st.packed_recv_count), None, None, capi.ptr(rec), capi.ptr(ws), ws.numel(),
+        torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    epr, n_slots = e // r, r * m
+    tail_at = O.row_payload(h, fmt) - 16
+    tail = buf[:, tail_at:tail_at + 16].contiguous().view(torch.int32)
+    recv_counts = meta["recv_counts"].cpu().tolist()
+    kept = [[[] for _ in range(r)] for _ in range(epr)]
+    want_rec, i = [], 0
+    for s in range(r):
+        for j in range(recv_counts[s]):
+            row = s * slot_rows + j
+            le = int(tail[row, 3])
+            if len(kept[le][s]) < m:
+                kept[le][s].append((row, i))
+            i += 1
+    want_rec = [-1] * i
+    count = st.packed_recv_count.cpu().tolist()
+    layout = st.packed_recv_layout_range.cpu()
+    px = st.packed_recv_x.view(torch.uint8).cpu()
+    for le in range(epr):
+        begin = 0
+        for s in range(r):
+            rows = kept[le][s]
+            assert int(layout[le, s]) == (((begin << 32) | len(rows)) if rows else 0), (le, s)
+            if rows:
+                idx = torch.tensor([row for row, _ in rows])
+                assert torch.equal(px[le, begin:begin + len(rows)], buf[idx, :h])
+                for pos, (_, rec_i) in enumerate(rows):
+                    want_rec[rec_i] = le * n_slots + begin + pos
+            begin += len(rows)
+        assert count[le] == begin and begin <= n_slots
+    assert max(count) == n_slots or t < 30  # source 1 alone fills its half of every expert
+    assert rec[:i].cpu().tolist() == want_rec

@@ -19,16 +19,29 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("one_call", [False, True], ids=["two_calls", "one_call"])
 def test_skew_stress_full_size(one_call):
-    from deepep_efa_amd import _capi, ll_runtime, loopback
-    _capi.load()
-    assert torch.cuda.is_available(), "this test needs the MI355X"
     import gc
     gc.collect()
     torch.cuda.empty_cache()  # what earlier tests left in the caching allocator
     free, _ = torch.cuda.mem_get_info()
     if free < 170 * 2 ** 30:
-        pytest.skip("needs ~150 GB of free HBM")
-    r, rank, t, h, k, e, seed = 64, 0, 8192, 7168, 8, 256, 4242
+        pytest.skip(f"needs ~150 GB of free HBM, {free >> 30} GiB are free: "
+                    "test_skew_stress_reduced_size covers the same code paths")
+    run_skew_stress(64, 0, 8192, 7168, 8, 256, 4242, one_call)
+
+
+@pytest.mark.parametrize("one_call", [False, True], ids=["two_calls", "one_call"])
+def test_skew_stress_reduced_size(one_call):
+    """The same world at 1280 tokens x 2048 per rank (a few GB): still more than 8192 pairs sent and far more
+    than 8192 rows received, so the send runs on chunk histograms and the receive, the row return and the
+    reduce take the large-batch kernels, with the hottest expert past half of its slots.  It never skips."""
+    run_skew_stress(64, 0, 1280, 2048, 8, 256, 777, one_call)
+
+
+def run_skew_stress(r, rank, t, h, k, e, seed, one_call):
+    from deepep_efa_amd import _capi, ll_runtime, loopback
+    _capi.load()
+    assert torch.cuda.is_available(), "this test needs the MI355X"
+    assert t * k > 8192, "the point is the large-batch kernels"
     epr, n_slots = e // r, r * t
     shape = ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8)
     st = ll_runtime.LowLatencyState(shape)
