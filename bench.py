@@ -53,6 +53,11 @@ def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0, packed=None):
         "exchange_metadata": r * e * 4 + rv * 16 + r * 24,
         # the staged receive's bytes plus, per row, the record, the tail read and the descriptor
         "dispatch_recv_by_source": rv * stride + rv * packed + small + rv * 12,
+        "dispatch_recv_by_source_ordered": rv * stride + rv * packed + small + r * e * 4 + rv * 8,
+        # the all-to-all shaped transport: one buffer per direction, contiguous per peer
+        "dispatch_send_by_dest": t * 2 * h + t * k * 8 * 2 + p * stride + t * k * 4 + e * 8,
+        "combine_send_by_dest": rv * 2 * h * 2 + rv * 16,
+        "combine_recv_flat": p * 2 * h + t * k * 16 + e * 4 + t * 2 * h,
     }
 
 
@@ -187,37 +192,37 @@ def read_traffic_summary(kernel, stamp):
     return None
 
 
-def by_source_receive(torch, _capi, lib, ll_runtime, st, world):
-    """Sets up the receive path a source-grouped transport feeds: the staged rows regrouped by source rank
-    into one slotted buffer (slot = the most rows one source can send), the exchange-metadata records for the
-    world's route counts, and the call that consumes both.  Returns (callable, rows expected)."""
+def all_to_all_entries(torch, _capi, lib, ll_runtime, st, world, x, topk, weights, y, out):
+    """The same rank's step over a transport that ships one contiguous message per peer (an all-to-all):
+    send by destination; receive from the per-source buffer (placing the rows from their tails through the
+    exchange-metadata records, or, for messages in this build's own order, from the gathered counts alone);
+    return by destination; reduce from the flat buffer.  The peers' messages are the staged rows regrouped by
+    source rank (expert by expert, the order the send side emits), set up once.  Returns the callables."""
     sh = st.shape
     r, e, m, el = sh.num_ranks, sh.num_experts, sh.max_tokens, sh.num_local_experts
-    slot_rows = m * min(sh.num_topk, el)
+    a2a = ll_runtime.AllToAllState(sh)
+    a2a.dispatch_send(x, topk)
     staging = st.recv_staging.view(el, r, m, st.stride)
     count = st.recv_count.view(el, r).cpu()
-    buf = torch.empty((r * slot_rows, st.stride), dtype=torch.uint8, device="cuda")
     for src in range(r):
-        off = src * slot_rows
+        off = src * a2a.slot_rows
         for le in range(el):
             c = int(count[le, src])
-            buf[off:off + c] = staging[le, src, :c]
+            a2a.recv_by_source[off:off + c] = staging[le, src, :c]
             off += c
     tk = world.topk_idx_all.view(r, -1)
     routed = torch.stack([torch.bincount(tk[s][tk[s] >= 0], minlength=e) for s in range(r)]).to(torch.int32)
-    rows = int(count.sum())
-    meta = ll_runtime.exchange_metadata(routed, sh.rank, slot_rows, rows)
-    ws = torch.empty(lib.deepep_ll_by_source_workspace_bytes(e, rows), dtype=torch.uint8, device="cuda")
-    tokens_per_expert = torch.empty(el, dtype=torch.int32, device="cuda")
-
-    def call():
-        _capi.check(lib.deepep_ll_dispatch_recv_by_source(
-            _capi.ptr(buf), slot_rows, _capi.ptr(meta["recv_counts"]), _capi.ptr(meta["source_offset"]),
-            _capi.ptr(meta["num_recv_tokens"]), rows, sh.hidden, e, r, m, sh.fmt, _capi.ptr(st.packed_recv_x),
-            _capi.ptr(st.packed_recv_scales), _capi.ptr(st.packed_recv_src_info),
-            _capi.ptr(st.packed_recv_layout_range), _capi.ptr(st.packed_recv_count), None,
-            _capi.ptr(tokens_per_expert), None, _capi.ptr(ws), ws.numel(), torch.cuda.current_stream().cuda_stream))
-    return call, rows
+    a2a.exchange_metadata(routed)
+    a2a.dispatch_recv()
+    a2a.recv_flat.normal_()  # the peers' answers, one row per row sent
+    torch.cuda.synchronize()
+    return {
+        "dispatch_send_by_dest": lambda: a2a.dispatch_send(x, topk),
+        "dispatch_recv_by_source": lambda: a2a.dispatch_recv(),
+        "dispatch_recv_by_source_ordered": lambda: a2a.dispatch_recv_ordered(routed),
+        "combine_send_by_dest": lambda: a2a.combine_send(y),
+        "combine_recv_flat": lambda: a2a.combine_recv(topk, weights, out),
+    }
 
 
 def bench_pack(torch, _capi, lib, loopback, args):
@@ -374,6 +379,24 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
     rv = int(st.packed_recv_count.sum())
     own = int((st.packed_recv_layout_range[:, rank] & 0xFFFFFFFF).sum())
     nbytes = algorithmic_bytes(t, h, k, p, rv, st.payload_bytes, e, r, own)
+    balanced_hint = st.expected_rows
+    if skewed:
+        # The hint a caller has: the rows the step before received (packed_recv_count is an output of every
+        # dispatch; deep_ep.Buffer reads it back without blocking and sizes the next large call by it).  The
+        # row copies take their grid from it; with the balanced guess T * K, twenty times too low here, they
+        # walk the batch in a loop, which the *_with_balanced_hint lines show.
+        for s_ in states:
+            s_.expected_rows = rv
+
+    def with_hint(fn, s_, hint):
+        def call():
+            keep, s_.expected_rows = s_.expected_rows, hint
+            try:
+                fn()
+            finally:
+                s_.expected_rows = keep
+        return call
+
     def on_every_state(make):
         return rotating([make(s_, x_) for s_, x_ in zip(states, xs)])
 
@@ -386,12 +409,19 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
         "dispatch": on_every_state(lambda s_, x_: lambda: s_.dispatch(x_, topk)),
         "combine": on_every_state(lambda s_, x_: lambda: s_.combine(y, topk, weights, out)),
     }
-    if not skewed:  # the receive side fed by a source-grouped transport (same bytes as dispatch_recv)
-        calls["dispatch_recv_by_source"] = on_every_state(
-            lambda s_, x_: by_source_receive(torch, _capi, lib, ll_runtime, s_, world)[0])
+    if skewed:
+        calls["dispatch_recv_with_balanced_hint"] = with_hint(lambda: st.dispatch_recv(), st, balanced_hint)
+        calls["combine_send_with_balanced_hint"] = with_hint(lambda: st.combine_send(y), st, balanced_hint)
+        nbytes["dispatch_recv_with_balanced_hint"] = nbytes["dispatch_recv"]
+        nbytes["combine_send_with_balanced_hint"] = nbytes["combine_send"]
+    if not skewed:  # the same step over an all-to-all shaped transport (two sets of buffers like the others)
+        per_state = [all_to_all_entries(torch, _capi, lib, ll_runtime, s_, world, x_, topk, weights, y, out)
+                     for s_, x_ in zip(states, xs)]
+        for name in per_state[0]:
+            calls[name] = rotating([entries[name] for entries in per_state])
     res = {"workload": f"LL dispatch+combine at {t} tokens x {h}, top-{k} of {e} experts, {r} ranks x {epr} experts"
                        + (", Zipf(1.2) expert popularity, 1 % outlier rows" if skewed else ""),
-           "pairs_sent": p, "rows_received": rv, "rows_to_own_experts": own,
+           "pairs_sent": p, "rows_received": rv, "rows_to_own_experts": own, "expected_rows_hint": st.expected_rows,
            "buffers": "one set" if skewed else "two sets taken in turn, so no call finds its bytes in the memory-side cache"}
     for name, fn in calls.items():
         if skewed:  # millisecond kernels: every call between its own events, so the spread shows
@@ -435,6 +465,27 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
                                        "the send's traffic pattern without routing, quantisation or scales"}
     res["dispatch_send"]["us_per_byte_against_bare_row_scatter"] = round(
         (res["dispatch_send"]["us"] / nbytes["dispatch_send"]) / (us / probe_bytes), 3)
+    # For scale beside the row copies: one contiguous streaming copy of as many bytes as the receive copy reads
+    # (and writes), 16 bytes per thread, nothing to look up.
+    half = (nbytes["dispatch_recv"] // 2) // 4096 * 4096
+    pairs = [(torch.empty(half, dtype=torch.uint8, device="cuda"), torch.empty(half, dtype=torch.uint8, device="cuda"))
+             for _ in range(1 if skewed else 2)]
+
+    def copy_on(a, b):
+        def call():
+            assert probe_lib.bench_probe_stream_copy(_capi.ptr(a), _capi.ptr(b), half, stream) == 0
+        return call
+
+    plain = rotating([copy_on(a, b) for a, b in pairs])
+    if skewed:
+        samples = sorted(time_calls(torch, plain, 1) for _ in range(6))
+        us = samples[len(samples) // 2]
+    else:
+        us = time_calls(torch, plain, max(10, args.steps // 10))
+    res["plain_stream_copy"] = {"us": round(us, 2), "bytes": 2 * half, "GBps": round(2 * half / us / 1e3, 1),
+                                "frac_of_8TBps": round(2 * half / us / 1e3 / HBM_PEAK_GBS, 4),
+                                "what": "one contiguous copy of the bytes the receive copy moves"}
+    del pairs
     return res
 
 
@@ -597,8 +648,8 @@ def main():
         "combine_send": lambda: st.combine_send(y),
         "combine_recv": lambda: st.combine_recv(topk, weights, out),
     }
-    # the receive side fed by a source-grouped transport: consumes the exchange-metadata records
-    calls["dispatch_recv_by_source"], _ = by_source_receive(torch, _capi, lib, ll_runtime, st, world)
+    # the same step over an all-to-all shaped transport: one contiguous message per peer in each direction
+    calls.update(all_to_all_entries(torch, _capi, lib, ll_runtime, st, world, x, topk, weights, y, out))
     step_calls = ("dispatch", "combine")  # what deep_ep.Buffer.low_latency_dispatch / _combine launch
     phase_calls = ("dispatch_send", "dispatch_recv", "combine_send", "combine_recv")
 

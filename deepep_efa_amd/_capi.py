@@ -45,11 +45,13 @@ PROTOTYPES = {
     "deepep_ll_exchange_metadata": (_I, [_VP, _I, _I, _I, _I, _I64] + [_VP] * 11),
     "deepep_ll_by_source_workspace_bytes": (_SZ, [_I, _I64]),
     "deepep_ll_dispatch_recv_by_source": (_I, [_VP, _I64, _VP, _VP, _VP, _I64, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP,
-                                               _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
+                                               _VP, _VP, _VP, _VP, _I64, _VP, _SZ, _VP]),
+    "deepep_ll_dispatch_recv_by_source_ordered": (_I, [_VP, _I64, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP, _VP, _VP,
+                                                       _VP, _VP, _VP, _I64, _I64, _VP, _SZ, _VP]),
     "deepep_ll_dispatch_send_by_dest": (_I, [_VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP, _I64, _VP, _VP, _VP, _VP,
                                              _VP, _VP, _SZ, _VP]),
     "deepep_ll_combine_send_by_dest": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _I64, _I, _I, _I, _I, _VP, _VP, _VP, _VP,
-                                            _VP, _VP]),
+                                            _VP, _I64, _VP]),
     "deepep_ll_combine_recv_flat": (_I, [_VP, _I64, _I64, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP, _VP]),
     "deepep_combine_reduce_workspace_bytes": (_SZ, [_I, _I]),
     "deepep_combine_reduce": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I64, _VP, _VP, _VP, _VP, _SZ,

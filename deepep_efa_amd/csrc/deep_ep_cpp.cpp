@@ -10,6 +10,7 @@
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <c10/hip/HIPFunctions.h>
+#include <c10/hip/HIPGraphsC10Utils.h>
 #include <pybind11/functional.h>
 
 #include <algorithm>
@@ -193,6 +194,12 @@ struct Buffer {
     LowLatencyCache ll;
     std::vector<torch::Tensor> combine_input_buffers;
     int combine_buffer_idx = 0;
+    // Rows the last large dispatch received, read back without blocking: the next large call is sized by it.
+    // (Under skewed routing a rank can receive many times num_tokens * num_topk rows; the row-copy kernels
+    // take their grid from the rows expected, and one sized for a balanced world walks such a batch in a slow loop.)
+    torch::Tensor observed_count_host;
+    std::optional<torch::Event> observed_ready;
+    int64_t observed_rows = 0;
     // loopback world
     std::optional<torch::Tensor> world_x, world_topk_idx;
     torch::Tensor ranks_below, ranks_above, peer_workspace;
@@ -255,6 +262,8 @@ struct Buffer {
         rdma_buffer = torch::Tensor();
         layout_workspaces.clear();
         ll = LowLatencyCache();
+        observed_ready.reset();
+        observed_count_host = torch::Tensor();
         combine_input_buffers.clear();
         world_x.reset();
         world_topk_idx.reset();
@@ -498,6 +507,18 @@ struct Buffer {
         auto stream = current_stream();
 
         stage_peer_rows(c);  // what the exchange would have delivered
+        // Large batches: the hint is what the dispatch before this one received, if that has arrived on the host
+        const bool large = int64_t(num_tokens) * num_topk > 8192;
+        int64_t expected_rows = std::max<int64_t>(num_tokens, 1) * num_topk;
+        const bool capturing = c10::hip::currentStreamCaptureStatusMayInitCtx() != c10::hip::CaptureStatus::None;
+        if (large) {
+            // (an event may not be queried while a stream is being captured: a captured call keeps the last hint)
+            if (not capturing and observed_ready.has_value() and observed_ready->query()) {
+                observed_rows = observed_count_host.sum().item<int64_t>();
+                observed_ready.reset();
+            }
+            expected_rows = std::max(expected_rows, observed_rows);
+        }
         // send and receive phase in one call (one kernel launch for decode-sized batches)
         abi_check(deepep_ll_dispatch(
             x.data_ptr(), topk_idx.data_ptr<int64_t>(), num_tokens, hidden, num_topk, num_experts, num_ranks, rank,
@@ -507,10 +528,18 @@ struct Buffer {
             c.packed_recv_src_info.data_ptr<int>(), c.packed_recv_layout_range.data_ptr<int64_t>(),
             c.packed_recv_count.data_ptr<int>(),
             cumulative_local_expert_recv_stats.has_value() ? cumulative_local_expert_recv_stats->data_ptr<int>() : nullptr,
-            /*expected_rows=*/std::max<int64_t>(num_tokens, 1) * num_topk, c.workspace.data_ptr(),
+            expected_rows, c.workspace.data_ptr(),
             size_t(c.workspace.numel()), c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
             c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));
         c.dispatched = true;
+        if (large and not capturing and not observed_ready.has_value()) {
+            if (!observed_count_host.defined() or observed_count_host.numel() != c.packed_recv_count.numel())
+                observed_count_host = torch::empty({c.packed_recv_count.numel()},
+                                                   torch::dtype(torch::kInt32).pinned_memory(true));
+            observed_count_host.copy_(c.packed_recv_count, /*non_blocking=*/true);
+            observed_ready = torch::Event(torch::kCUDA);
+            observed_ready->record(c10::hip::getCurrentHIPStreamMasqueradingAsCUDA());
+        }
 
         std::optional<EventHandle> event;
         if (async) event = EventHandle();
@@ -592,7 +621,9 @@ struct Buffer {
                                     hidden, num_topk, num_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,
                                     accumulate ? 1 : 0, c.combine_staging.data_ptr(),
                                     zero_copy ? nullptr : c.combine_send_slots.data_ptr(),
-                                    combined_x.data_ptr(), /*expected_rows=*/std::max<int64_t>(num_combined_tokens, 1) * num_topk,
+                                    combined_x.data_ptr(),
+                                    /*expected_rows=*/std::max<int64_t>(std::max<int64_t>(num_combined_tokens, 1) * num_topk,
+                                                                         int64_t(num_combined_tokens) * num_topk > 8192 ? observed_rows : 0),
                                     c.segment_workspace.defined() ? c.segment_workspace.data_ptr() : nullptr,
                                     c.segment_workspace.defined() ? size_t(c.segment_workspace.numel()) : 0, stream));
 

@@ -521,7 +521,8 @@ int deepep_ll_combine_send_by_dest(const void* x, const int32_t* record_packed_r
                                    const uint32_t* num_recv_tokens, int64_t row_capacity, int hidden, int num_experts,
                                    int num_ranks, int num_max_dispatch_tokens_per_rank, void* send_flat,
                                    const int32_t* recv_counts, const int64_t* combine_remote_recv_offset,
-                                   void* const* peer_recv_flat, const int64_t* peer_recv_rows, void* stream) {
+                                   void* const* peer_recv_flat, const int64_t* peer_recv_rows,
+                                   int64_t expected_rows, void* stream) {
     clear_error();
     EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
     EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
@@ -548,14 +549,14 @@ int deepep_ll_combine_send_by_dest(const void* x, const int32_t* record_packed_r
     a.recv_counts = recv_counts, a.remote_offset = combine_remote_recv_offset;
     int threads = ((a.num_vec + 63) / 64) * 64;
     if (threads > 1024) threads = 1024;
-    int64_t blocks = row_capacity;
-    if (blocks > 16384) blocks = blocks / 2 > 16384 ? blocks / 2 : 16384;
-    if (blocks > (int64_t(1) << 22)) blocks = int64_t(1) << 22;
+    // grid from the rows expected, not from the capacity (an idle workgroup is not free)
+    const int64_t rows = expected_rows > 0 && expected_rows < row_capacity ? expected_rows : row_capacity;
+    const unsigned blocks = flat_grid_blocks(rows, row_capacity, num_max_dispatch_tokens_per_rank);
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
-    if (2 * row_capacity * hidden * 2 > stream_bytes())
-        ll_combine_send_by_dest_kernel<true><<<unsigned(blocks), threads, 0, hs>>>(a);
+    if (2 * rows * hidden * 2 > stream_bytes())
+        ll_combine_send_by_dest_kernel<true><<<blocks, threads, 0, hs>>>(a);
     else
-        ll_combine_send_by_dest_kernel<false><<<unsigned(blocks), threads, 0, hs>>>(a);
+        ll_combine_send_by_dest_kernel<false><<<blocks, threads, 0, hs>>>(a);
     EP_LAUNCH_CHECK();
     return 0;
 }

@@ -413,16 +413,29 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
     DEEPEP_PHASE(6);
 }
 
+// index_rows > 0: the grid has that many rows in front of the token rows whose workgroups build the
+// receive side's row index (one (local expert, source) segment each), so that a large one-call
+// dispatch needs no launch for it.
 template <int kFmt, bool kStream>
-__global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs a, DirectOut direct) {
-    extern __shared__ int32_t lds_hist[];  // [E], counting workgroups only
+__global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs a, DirectOut direct, FusedIndexArgs index,
+                                                                       int index_rows) {
+    extern __shared__ int32_t lds_hist[];  // counting workgroups: [E]; index workgroups: [2 * (E + 1)]
     __shared__ SendLds lds;
-    if (int(blockIdx.y) == a.num_tokens) {  // the counting row of the grid
+    __shared__ int32_t index_wave_totals[kMaxBlockWaves];
+    // Grid rows: first the index rows (started first, so that their few microseconds of scans run beside
+    // the token rows instead of behind them), then one row per token, then the counting row.
+    const int y = int(blockIdx.y) - index_rows;
+    if (y < 0) {
+        const int seg = int(blockIdx.y) * int(gridDim.x) + int(blockIdx.x);
+        if (seg < index.num_local_experts * index.num_ranks) recv_index_block(index, seg, lds_hist, index_wave_totals);
+        return;
+    }
+    if (y == a.num_tokens) {  // the counting row of the grid
         // (the by-destination form has its counts already: ll_by_dest_prefix_kernel ran first)
         if (blockIdx.x == 0 && a.expert_prefix == nullptr) send_count_block(a, blockIdx.z, lds_hist);
         return;
     }
-    send_token_block<kFmt, kStream>(a, direct, blockIdx.z, blockIdx.y, blockIdx.x, lds);
+    send_token_block<kFmt, kStream>(a, direct, blockIdx.z, y, blockIdx.x, lds);
 }
 
 // ---------------------------------------------------------------------
@@ -794,7 +807,8 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
                             void* send_slots, int32_t* send_count, int32_t* pair_slot, void* workspace,
                             size_t workspace_bytes, hipStream_t stream, const RecvArgs* fused_recv = nullptr,
                             int64_t fused_recv_wave_items = 0, const DirectOut* own_rows_direct = nullptr,
-                            const ByDestTables* by_dest = nullptr) {
+                            const ByDestTables* by_dest = nullptr, FusedIndexArgs* fused_index = nullptr,
+                            bool* index_was_fused = nullptr) {
     const int64_t scratch_bytes = route_scratch_bytes(num_tokens, num_topk, num_experts);
     EP_HOST_ASSERT(workspace != nullptr && workspace_bytes >= size_t(scratch_bytes) * size_t(num_src));
     EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
@@ -889,8 +903,19 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
         return 0;
     }
 
-    const dim3 grid(blocks_per_token, num_tokens + 1, num_src);  // + the counting workgroup
-    const size_t lds = size_t(num_experts) * sizeof(int32_t);
+    // The receive index rides along when the chunk histograms exist (its own counts come from them)
+    FusedIndexArgs index = {};
+    int index_rows = 0;
+    if (fused_index != nullptr && tpc > 0 && num_src == 1 && own_rows_direct != nullptr) {
+        index = *fused_index;
+        index.chunk_hist = reinterpret_cast<const int32_t*>(ws);
+        index.num_chunks = (num_tokens + tpc - 1) / tpc;
+        index_rows = (num_experts + blocks_per_token - 1) / blocks_per_token;
+        if (num_tokens + 1 + index_rows > 65535) index_rows = 0, index = FusedIndexArgs{};
+    }
+    if (index_was_fused != nullptr) *index_was_fused = index_rows > 0;
+    const dim3 grid(blocks_per_token, num_tokens + 1 + index_rows, num_src);  // + the counting row, + the index rows
+    const size_t lds = size_t(index_rows > 0 ? 2 * (num_experts + 1) : num_experts) * sizeof(int32_t);
     // own_rows_direct (the two-launch form of the one-call dispatch): as in the single launch, the rows
     // for this rank's own experts go straight to their packed position behind the lower ranks' rows
     EP_HOST_ASSERT(own_rows_direct == nullptr || (num_src == 1 && src_ranks == nullptr));
@@ -901,8 +926,8 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     const bool streams = traffic > send_stream_bytes();
 #define DEEPEP_LAUNCH_SEND(FMT)                                                           \
     do {                                                                                  \
-        if (streams) ll_send_kernel<FMT, true><<<grid, waves * kWave, lds, stream>>>(sa, direct);  \
-        else ll_send_kernel<FMT, false><<<grid, waves * kWave, lds, stream>>>(sa, direct);         \
+        if (streams) ll_send_kernel<FMT, true><<<grid, waves * kWave, lds, stream>>>(sa, direct, index, index_rows);  \
+        else ll_send_kernel<FMT, false><<<grid, waves * kWave, lds, stream>>>(sa, direct, index, index_rows);         \
     } while (0)
     switch (row_format) {
         case kRowBF16: DEEPEP_LAUNCH_SEND(kRowBF16); break;
@@ -1102,7 +1127,7 @@ static int launch_recv_side(const void* recv_staging, const int32_t* recv_count,
                             void* packed_recv_x, void* packed_recv_scales, int32_t* packed_recv_src_info,
                             int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
                             int32_t* cumulative_local_expert_recv_stats, int64_t expected_rows, void* workspace,
-                            size_t workspace_bytes, int own_rank, void* stream) {
+                            size_t workspace_bytes, int own_rank, void* stream, bool index_done = false) {
     if (int rc = check_recv_args(recv_staging, recv_count, hidden, num_experts, num_ranks,
                                  num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                                  packed_recv_src_info, packed_recv_layout_range, packed_recv_count))
@@ -1117,10 +1142,12 @@ static int launch_recv_side(const void* recv_staging, const int32_t* recv_count,
         int32_t* flat = reinterpret_cast<int32_t*>(workspace);
         RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) +
                                                    (((int64_t(num_experts) + 1) * 4 + 255) & ~int64_t(255)));
-        ll_segment_index_kernel<<<num_experts, kIndexThreads, 0, hs>>>(
-            0, recv_count, nullptr, num_local_experts, num_ranks, own_rank, num_max_dispatch_tokens_per_rank,
-            packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, flat, desc);
-        EP_LAUNCH_CHECK();
+        if (!index_done) {  // (a large one-call dispatch builds the index inside its send launch)
+            ll_segment_index_kernel<<<num_experts, kIndexThreads, 0, hs>>>(
+                0, recv_count, nullptr, num_local_experts, num_ranks, own_rank, num_max_dispatch_tokens_per_rank,
+                packed_recv_layout_range, packed_recv_count, cumulative_local_expert_recv_stats, flat, desc);
+            EP_LAUNCH_CHECK();
+        }
         const int64_t data_bytes = row_data_bytes(hidden, row_format);
         const int64_t scale_bytes = row_scale_bytes(hidden, row_format);
         const int num_vec = int(data_bytes / 16);
@@ -1202,16 +1229,37 @@ int deepep_ll_dispatch(const void* x, const int64_t* topk_idx, int num_tokens, i
             return rc;
         const DirectOut direct = {reinterpret_cast<uint8_t*>(packed_recv_x),
                                   reinterpret_cast<uint8_t*>(packed_recv_scales), packed_recv_src_info};
+        // When the receive side will run as index + flat copy, the index is built by extra workgroups of
+        // the send launch: three launches (histograms, send + index, copy) instead of four.
+        FusedIndexArgs index = {};
+        const bool flat_copy =
+            segment_workspace != nullptr && num_experts <= 1024 &&
+            estimated_rows(expected_rows, num_experts, num_max_dispatch_tokens_per_rank) > kLargeBatchRows;
+        if (flat_copy) {
+            EP_HOST_ASSERT(segment_workspace_bytes >=
+                           size_t(deepep::segment_workspace_bytes(num_experts, num_max_dispatch_tokens_per_rank)));
+            EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(segment_workspace) & 15) == 0);
+            index.recv_count = recv_count;
+            index.num_experts = num_experts, index.num_local_experts = num_experts / num_ranks;
+            index.num_ranks = num_ranks, index.rank = rank, index.max_tokens = num_max_dispatch_tokens_per_rank;
+            index.layout_out = packed_recv_layout_range, index.packed_count = packed_recv_count;
+            index.stats = cumulative_local_expert_recv_stats;
+            index.flat_out = reinterpret_cast<int32_t*>(segment_workspace);
+            index.desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(segment_workspace) +
+                                                    (((int64_t(num_experts) + 1) * 4 + 255) & ~int64_t(255)));
+        }
+        bool index_done = false;
         if (int rc = launch_send_side(x, topk_idx, nullptr, 1, num_tokens, hidden, num_topk, num_experts, num_ranks,
                                       rank, num_max_dispatch_tokens_per_rank, row_format, recv_staging, recv_count,
                                       send_slots, send_count, pair_slot, workspace, workspace_bytes,
-                                      reinterpret_cast<hipStream_t>(stream), nullptr, 0, &direct))
+                                      reinterpret_cast<hipStream_t>(stream), nullptr, 0, &direct, nullptr,
+                                      flat_copy ? &index : nullptr, &index_done))
             return rc;
         return launch_recv_side(recv_staging, recv_count, hidden, num_experts, num_ranks,
                                 num_max_dispatch_tokens_per_rank, row_format, packed_recv_x, packed_recv_scales,
                                 packed_recv_src_info, packed_recv_layout_range, packed_recv_count,
                                 cumulative_local_expert_recv_stats, expected_rows, segment_workspace,
-                                segment_workspace_bytes, rank, stream);
+                                segment_workspace_bytes, rank, stream, index_done);
     }
     EP_HOST_ASSERT(num_tokens == 0 || (x != nullptr && topk_idx != nullptr));
     EP_HOST_ASSERT(send_count != nullptr && pair_slot != nullptr);

@@ -18,6 +18,8 @@
 // its own 512 rows on top of the histograms of its source's earlier chunks); and the flat row copy
 // the other large-batch paths use.  Small batches, two launches: no histograms, one workgroup per
 // source counts every record's expert itself and walks its source's chunks in order.
+#include <algorithm>
+
 #include "common.hpp"
 #include "segments.hpp"
 #include "../../include/deepep_hip.h"
@@ -271,6 +273,92 @@ __global__ __launch_bounds__(kBySourceThreads) void ll_by_source_index_kernel(
     }
 }
 
+// ---------------------------------------------------------------------
+// The same receive when every source's message is known to come ordered by local expert, the rows of
+// an expert in the sender's slot order -- what deepep_ll_dispatch_send_by_dest emits -- and the
+// gathered route counts are at hand.  Then nothing has to be read from the rows to place them: row j
+// of source s belongs to the expert e whose run [first(e, s), first(e, s) + cnt(e, s)) holds j, with
+// first(e, s) the count of the lower experts in that source's column of the counts, and it lands at
+// begin(e, s) + (j - first(e, s)), begin being the prefix over the lower sources
+// (csrc/kernels/efa_kernels.cu:991-1010).  One launch of arithmetic (a workgroup per (expert, source)
+// pair, like ll_segment_index_kernel) in front of the flat row copy; both sides of every pair are
+// contiguous runs of rows.  Rows of a message past the source's slot are lost: a pair keeps
+// min(cnt, slot_rows - first) rows.
+// ---------------------------------------------------------------------
+__global__ __launch_bounds__(kIndexThreads) void ll_by_source_ordered_index_kernel(
+    const int32_t* __restrict__ all_num_routed, int num_experts, int num_local_experts, int num_ranks, int rank,
+    int max_tokens, int slot_rows, int64_t row_capacity, int64_t* __restrict__ layout_range,
+    int32_t* __restrict__ packed_count, int32_t* __restrict__ stats, uint32_t* __restrict__ tokens_per_expert,
+    int32_t* __restrict__ record_packed_row, int32_t* __restrict__ flat_total, RowDesc* __restrict__ desc) {
+    __shared__ int32_t sent[kIndexThreads];       // cnt(e, s) as the sender counted it (clamped to max_tokens)
+    __shared__ int32_t place[kIndexThreads + 1];  // prefix over the rows kept, pairs in (expert, source) order
+    __shared__ int32_t source_total[kIndexThreads];
+    __shared__ int32_t wave_totals[kIndexThreads / kWave];
+    const int tid = threadIdx.x;
+    const int num_segments = num_local_experts * num_ranks;
+    const int le_of = tid / num_ranks, s_of = tid - le_of * num_ranks;
+    int c = 0;
+    if (tid < num_segments) {
+        c = all_num_routed[int64_t(s_of) * num_experts + rank * num_local_experts + le_of];
+        c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+    }
+    sent[tid] = c;
+    __syncthreads();
+    // first(e, s): this source's rows for the lower experts; the source's whole message
+    int first = 0, kept = 0;
+    if (tid < num_segments) {
+        for (int e2 = 0; e2 < le_of; ++e2) first += sent[e2 * num_ranks + s_of];
+        const int room = slot_rows - first;
+        kept = room <= 0 ? 0 : (c < room ? c : room);
+    }
+    if (tid < num_ranks) {
+        int total = 0;
+        for (int e2 = 0; e2 < num_local_experts; ++e2) total += sent[e2 * num_ranks + tid];
+        source_total[tid] = total;
+    }
+    int total;
+    const int prefix = block_exclusive_scan_1024(kept, wave_totals, total);
+    if (tid < num_segments) place[tid] = prefix;
+    if (tid == 0) place[num_segments] = total;
+    __syncthreads();
+    const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
+    if (blockIdx.x == 0) {
+        if (tid < num_segments) {
+            const int64_t begin = place[tid] - place[le_of * num_ranks];
+            layout_range[tid] = kept > 0 ? ((begin << 32) | int64_t(kept)) : 0;
+        }
+        if (tid < num_local_experts) {
+            const int n = place[(tid + 1) * num_ranks] - place[tid * num_ranks];
+            packed_count[tid] = n;
+            if (stats != nullptr) stats[tid] += n;
+            if (tokens_per_expert != nullptr) tokens_per_expert[tid] = uint32_t(n);
+        }
+        if (tid == 0) flat_total[0] = total;
+    }
+    // this workgroup's pair: one descriptor per row kept, and every record of the pair
+    const int seg = blockIdx.x;
+    const int le = seg / num_ranks, s = seg - le * num_ranks;
+    // thread `seg` holds the pair's numbers; hand them to the workgroup
+    __shared__ int32_t pair_first, pair_kept, pair_sent;
+    if (tid == seg) pair_first = first, pair_kept = kept, pair_sent = c;
+    __syncthreads();
+    const int64_t begin = place[seg] - place[le * num_ranks];
+    int64_t record_base = 0;  // records of the lower sources: their whole messages, kept or not
+    for (int s2 = 0; s2 < s; ++s2) record_base += source_total[s2];
+    record_base += pair_first;
+    for (int j = tid; j < pair_sent; j += kIndexThreads) {
+        int32_t packed_row = -1;
+        if (j < pair_kept) {
+            RowDesc d;
+            d.src_row = int32_t(int64_t(s) * slot_rows + pair_first + j);
+            d.dst_row = int32_t(int64_t(le) * slots_per_expert + begin + j);
+            desc[place[seg] + j] = d;
+            packed_row = d.dst_row;
+        }
+        if (record_packed_row != nullptr && record_base + j < row_capacity) record_packed_row[record_base + j] = packed_row;
+    }
+}
+
 }  // namespace deepep
 
 using namespace deepep;
@@ -297,8 +385,8 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
                                       void* packed_recv_scales, int32_t* packed_recv_src_info,
                                       int64_t* packed_recv_layout_range, int32_t* packed_recv_count,
                                       int32_t* cumulative_local_expert_recv_stats, uint32_t* tokens_per_expert,
-                                      int32_t* record_packed_row, void* workspace, size_t workspace_bytes,
-                                      void* stream) {
+                                      int32_t* record_packed_row, int64_t expected_rows, void* workspace,
+                                      size_t workspace_bytes, void* stream) {
     clear_error();
     EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
     EP_HOST_ASSERT(num_ranks > 0 && num_ranks <= kBySourceMaxRanks);
@@ -338,7 +426,10 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
                                                by_source_hist_bytes(num_experts, capacity));
     const uint8_t* rows_in = reinterpret_cast<const uint8_t*>(recv_by_source);
 
-    if (row_capacity <= kBySourceSmallRecords) {
+    // Which form indexes the records depends on how many are expected, not on how many fit: both give the
+    // same result, and a buffer sized for its largest batch still takes the short form for a small one.
+    const int64_t expected_records = expected_rows > 0 && expected_rows < row_capacity ? expected_rows : row_capacity;
+    if (expected_records <= kBySourceSmallRecords) {
         ll_by_source_index_kernel<false><<<num_ranks, kBySourceThreads, index_lds, hs>>>(
             rows_in, stride, tail_off, buffer_rows, int(slot_rows), recv_counts, source_offset, num_recv_tokens,
             row_capacity, num_local_experts, num_ranks, num_max_dispatch_tokens_per_rank, nullptr,
@@ -365,14 +456,73 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
     int threads = ((num_vec + 63) / 64) * 64;
     int extra = 64;  // one more wave for scales + source index
     if (threads + extra > 1024) threads = 1024, extra = 0;
-    int64_t blocks = row_capacity;
-    if (blocks > 16384) blocks = blocks / 2 > 16384 ? blocks / 2 : 16384;
-    if (blocks > (int64_t(1) << 22)) blocks = int64_t(1) << 22;
-    ll_rows_flat_kernel<<<unsigned(blocks), threads + extra, 0, hs>>>(
+    // the copy's grid follows the rows expected, not the capacity: a workgroup that finds no row still costs
+    // a fraction of a nanosecond, and a capacity of R slots is many times what a balanced world fills
+    const unsigned blocks = flat_grid_blocks(expected_rows > 0 ? expected_rows : row_capacity, row_capacity,
+                                             num_max_dispatch_tokens_per_rank);
+    ll_rows_flat_kernel<<<blocks, threads + extra, 0, hs>>>(
         flat_total, 0, desc, rows_in, stride, num_vec,
         reinterpret_cast<uint8_t*>(packed_recv_x), nullptr, data_bytes, int(scale_bytes / 4), align16(data_bytes),
         scale_bytes > 0 ? reinterpret_cast<uint8_t*>(packed_recv_scales) : nullptr, tail_off, packed_recv_src_info,
         extra);
+    EP_LAUNCH_CHECK();
+    return 0;
+}
+
+int deepep_ll_dispatch_recv_by_source_ordered(const void* recv_by_source, int64_t slot_rows,
+                                              const int32_t* all_num_routed, int hidden, int num_experts,
+                                              int num_ranks, int rank, int num_max_dispatch_tokens_per_rank,
+                                              int row_format, void* packed_recv_x, void* packed_recv_scales,
+                                              int32_t* packed_recv_src_info, int64_t* packed_recv_layout_range,
+                                              int32_t* packed_recv_count,
+                                              int32_t* cumulative_local_expert_recv_stats,
+                                              uint32_t* tokens_per_expert, int32_t* record_packed_row,
+                                              int64_t row_capacity, int64_t expected_rows, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
+    clear_error();
+    EP_HOST_ASSERT(hidden > 0 && hidden % 128 == 0);
+    EP_HOST_ASSERT(num_ranks > 0 && num_experts > 0 && num_experts % num_ranks == 0);
+    EP_HOST_ASSERT(rank >= 0 && rank < num_ranks);
+    EP_HOST_ASSERT(num_experts <= kIndexThreads);  // one thread per (local expert, source) pair
+    EP_HOST_ASSERT(num_max_dispatch_tokens_per_rank > 0);
+    EP_HOST_ASSERT(row_format >= kRowBF16 && row_format <= kRowFP8UE8M0);
+    EP_HOST_ASSERT(row_format != kRowFP8UE8M0 || (hidden / 128) % 4 == 0);
+    EP_HOST_ASSERT(slot_rows > 0 && slot_rows * num_ranks < (int64_t(1) << 31));
+    EP_HOST_ASSERT(row_capacity >= 0 && row_capacity < (int64_t(1) << 31));
+    EP_HOST_ASSERT(int64_t(num_experts) * num_max_dispatch_tokens_per_rank < (int64_t(1) << 31));
+    EP_HOST_ASSERT(recv_by_source != nullptr && all_num_routed != nullptr);
+    EP_HOST_ASSERT(packed_recv_x != nullptr && (row_format == kRowBF16 || packed_recv_scales != nullptr));
+    EP_HOST_ASSERT(packed_recv_src_info != nullptr && packed_recv_layout_range != nullptr &&
+                   packed_recv_count != nullptr);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(recv_by_source) & 15) == 0);
+    EP_HOST_ASSERT((reinterpret_cast<uintptr_t>(packed_recv_x) & 15) == 0);
+    EP_HOST_ASSERT(workspace != nullptr && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0);
+    // one descriptor per row that can be kept: a source's slot, and an expert's packed slots, bound them
+    const int64_t most_rows = std::min<int64_t>(slot_rows * num_ranks,
+                                                int64_t(num_experts) * num_max_dispatch_tokens_per_rank);
+    EP_HOST_ASSERT(workspace_bytes >= size_t(by_source_head_bytes() + most_rows * int64_t(sizeof(RowDesc))));
+    const int num_local_experts = num_experts / num_ranks;
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    int32_t* flat_total = reinterpret_cast<int32_t*>(workspace);
+    RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) + by_source_head_bytes());
+    ll_by_source_ordered_index_kernel<<<num_experts, kIndexThreads, 0, hs>>>(
+        all_num_routed, num_experts, num_local_experts, num_ranks, rank, num_max_dispatch_tokens_per_rank,
+        int(slot_rows), row_capacity, packed_recv_layout_range, packed_recv_count,
+        cumulative_local_expert_recv_stats, tokens_per_expert, record_packed_row, flat_total, desc);
+    EP_LAUNCH_CHECK();
+    const int64_t data_bytes = row_data_bytes(hidden, row_format);
+    const int64_t scale_bytes = row_scale_bytes(hidden, row_format);
+    const int num_vec = int(data_bytes / 16);
+    int threads = ((num_vec + 63) / 64) * 64;
+    int extra = 64;  // one more wave for scales + source index
+    if (threads + extra > 1024) threads = 1024, extra = 0;
+    const unsigned blocks = flat_grid_blocks(expected_rows > 0 ? expected_rows : most_rows, most_rows,
+                                             num_max_dispatch_tokens_per_rank);
+    ll_rows_flat_kernel<<<blocks, threads + extra, 0, hs>>>(
+        flat_total, 0, desc, reinterpret_cast<const uint8_t*>(recv_by_source), row_stride_bytes(hidden, row_format),
+        num_vec, reinterpret_cast<uint8_t*>(packed_recv_x), nullptr, data_bytes, int(scale_bytes / 4),
+        align16(data_bytes), scale_bytes > 0 ? reinterpret_cast<uint8_t*>(packed_recv_scales) : nullptr,
+        align16(data_bytes) + align16(scale_bytes), packed_recv_src_info, extra);
     EP_LAUNCH_CHECK();
     return 0;
 }

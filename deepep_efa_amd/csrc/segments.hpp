@@ -285,6 +285,78 @@ static __global__ __launch_bounds__(kIndexThreads) void ll_segment_index_kernel(
     }
 }
 
+// The dispatch-receive index (mode 0 above with the rank's own rows already placed) as one workgroup's
+// share inside another launch: the send kernel of a large one-call dispatch carries these workgroups
+// beside its own, so the index costs no launch.  The launch that carries it is still writing the
+// rank's own counts into recv_count, so they are taken from what that launch reads them from: the
+// column sums of the per-chunk expert histograms.  Any workgroup size that is a multiple of 64;
+// lds holds 2 * (segments + 1) ints, wave_totals 16.
+struct FusedIndexArgs {
+    const int32_t* recv_count;  // [E_l][R]; the own column is not read
+    const int32_t* chunk_hist;  // [chunks][E] of this rank's own entries
+    int num_chunks, num_experts, num_local_experts, num_ranks, rank, max_tokens;
+    int64_t* layout_out;
+    int32_t* packed_count;
+    int32_t* stats;
+    int32_t* flat_out;
+    RowDesc* desc;
+};
+
+__device__ __forceinline__ void recv_index_block(const FusedIndexArgs& a, int seg, int32_t* lds, int32_t* wave_totals) {
+    const int tid = threadIdx.x, threads = blockDim.x;
+    const int num_ranks = a.num_ranks, max_tokens = a.max_tokens;
+    const int num_segments = a.num_local_experts * num_ranks;
+    int32_t* flat = lds;                      // prefix over the rows that get descriptors
+    int32_t* place = lds + num_segments + 1;  // prefix over all rows: where a segment lands
+    for (int s = tid; s < num_segments; s += threads) {
+        const int le = s / num_ranks, src = s - le * num_ranks;
+        int c = 0;
+        if (src == a.rank) {
+            const int e = a.rank * a.num_local_experts + le;
+            for (int c0 = 0; c0 < a.num_chunks; c0 += 8) {  // eight loads in flight
+                int v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    v[u] = c0 + u < a.num_chunks ? a.chunk_hist[int64_t(c0 + u) * a.num_experts + e] : 0;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) c += v[u];
+            }
+        } else {
+            c = a.recv_count[s];
+        }
+        c = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+        place[s] = c;
+        flat[s] = src == a.rank ? 0 : c;  // own rows are in place already: no descriptors
+    }
+    lds_barrier();
+    block_exclusive_scan(flat, num_segments, wave_totals);
+    block_exclusive_scan(place, num_segments, wave_totals);
+    const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
+    if (seg == 0) {
+        for (int s = tid; s <= num_segments; s += threads) a.flat_out[s] = flat[s];
+        for (int s = tid; s < num_segments; s += threads) {
+            const int le = s / num_ranks;
+            const int64_t cnt = place[s + 1] - place[s];
+            const int64_t begin = place[s] - place[le * num_ranks];
+            a.layout_out[s] = cnt > 0 ? ((begin << 32) | cnt) : 0;
+        }
+        for (int le = tid; le < a.num_local_experts; le += threads) {
+            const int n = place[(le + 1) * num_ranks] - place[le * num_ranks];
+            a.packed_count[le] = n;
+            if (a.stats != nullptr) a.stats[le] += n;
+        }
+    }
+    const int le = seg / num_ranks;
+    const int cnt = flat[seg + 1] - flat[seg];
+    const int64_t begin = place[seg] - place[le * num_ranks];
+    for (int j = tid; j < cnt; j += threads) {
+        RowDesc d;
+        d.src_row = seg * max_tokens + j;
+        d.dst_row = int32_t(le * slots_per_expert + begin + j);
+        a.desc[flat[seg] + j] = d;
+    }
+}
+
 // One workgroup per described row (looping only if there are more rows than workgroups).  Only
 // batches too large for the caches come here, so the payload streams.
 static __global__ __launch_bounds__(1024) void ll_rows_flat_kernel(

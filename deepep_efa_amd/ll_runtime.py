@@ -233,6 +233,7 @@ class AllToAllState:
         self.send_flat = torch.empty((self.row_capacity, h), dtype=torch.bfloat16, device=device)
         self.recv_flat = torch.empty((self.send_capacity, h), dtype=torch.bfloat16, device=device)
         self.meta = None
+        self.expected_rows = m * k  # what a balanced world delivers; sizes grids, never the result
 
     def dispatch_send(self, x: torch.Tensor, topk_idx: torch.Tensor) -> None:
         s = self.shape
@@ -247,6 +248,19 @@ class AllToAllState:
         self.meta = exchange_metadata(all_num_routed, self.shape.rank, self.slot_rows, self.row_capacity)
         return self.meta
 
+    def dispatch_recv_ordered(self, all_num_routed: torch.Tensor, stats: torch.Tensor = None) -> None:
+        """The receive for messages in this build's own order (what dispatch_send emits): places every row by
+        arithmetic on the gathered counts, without the record list and without reading the rows' tails."""
+        s = self.shape
+        _capi.check(self.lib.deepep_ll_dispatch_recv_by_source_ordered(
+            _capi.ptr(self.recv_by_source), self.slot_rows, _capi.ptr(all_num_routed), s.hidden, s.num_experts,
+            s.num_ranks, s.rank, s.max_tokens, s.fmt, _capi.ptr(self.packed_recv_x),
+            _capi.ptr(self.packed_recv_scales), _capi.ptr(self.packed_recv_src_info),
+            _capi.ptr(self.packed_recv_layout_range), _capi.ptr(self.packed_recv_count), _capi.ptr(stats),
+            _capi.ptr(self.tokens_per_expert), _capi.ptr(self.record_packed_row), self.row_capacity,
+            self.expected_rows, _capi.ptr(self.by_source_workspace), self.by_source_workspace.numel(),
+            current_stream_ptr()))
+
     def dispatch_recv(self, stats: torch.Tensor = None) -> None:
         s, m = self.shape, self.meta
         _capi.check(self.lib.deepep_ll_dispatch_recv_by_source(
@@ -255,8 +269,8 @@ class AllToAllState:
             s.fmt, _capi.ptr(self.packed_recv_x), _capi.ptr(self.packed_recv_scales),
             _capi.ptr(self.packed_recv_src_info), _capi.ptr(self.packed_recv_layout_range),
             _capi.ptr(self.packed_recv_count), _capi.ptr(stats), _capi.ptr(self.tokens_per_expert),
-            _capi.ptr(self.record_packed_row), _capi.ptr(self.by_source_workspace), self.by_source_workspace.numel(),
-            current_stream_ptr()))
+            _capi.ptr(self.record_packed_row), self.expected_rows, _capi.ptr(self.by_source_workspace),
+            self.by_source_workspace.numel(), current_stream_ptr()))
 
     def combine_send(self, y: torch.Tensor, peer_recv_flat: torch.Tensor = None,
                      peer_recv_rows: torch.Tensor = None) -> None:
@@ -268,7 +282,7 @@ class AllToAllState:
             _capi.ptr(m["combine_send_offset"]), _capi.ptr(m["num_recv_tokens"]), self.row_capacity, s.hidden,
             s.num_experts, s.num_ranks, s.max_tokens, _capi.ptr(self.send_flat), _capi.ptr(m["recv_counts"]),
             _capi.ptr(m["combine_remote_recv_offset"]), _capi.ptr(peer_recv_flat), _capi.ptr(peer_recv_rows),
-            current_stream_ptr()))
+            self.expected_rows, current_stream_ptr()))
 
     def combine_recv(self, topk_idx: torch.Tensor, topk_weights: torch.Tensor, out: torch.Tensor,
                      recv: torch.Tensor = None, slot_rows: int = 0, accumulate: bool = False) -> None:

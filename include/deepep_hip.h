@@ -371,6 +371,8 @@ size_t deepep_ll_by_source_workspace_bytes(int num_experts, int64_t row_capacity
  *                   expert in its tail, past its pair's M rows) -- the reference's recv_expert_ids /
  *                   recv_expert_pos (csrc/kernels/efa_kernels.cu:2121-2231), which the combine needs to
  *                   return the rows in arrival order (deepep_ll_combine_send_by_dest)
+ *   expected_rows   rows the caller expects to receive (0 = unknown: row_capacity is assumed); it only
+ *                   sizes the copy's grid, and any value gives the same result
  *   workspace       deepep_ll_by_source_workspace_bytes(E, row_capacity) bytes
  * An (expert, source) pair takes at most M rows, as a segment of the staged form does.
  * Replaces ll_recv_unpack_v2 on its flat / slotted input (csrc/kernels/efa_kernels.cu:2121-2231,
@@ -386,7 +388,38 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
                                       int32_t* packed_recv_count,
                                       int32_t* cumulative_local_expert_recv_stats,
                                       uint32_t* tokens_per_expert, int32_t* record_packed_row,
+                                      int64_t expected_rows,
                                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* deepep_ll_dispatch_recv_by_source for messages whose order is known: every source sent its rows
+ * for this rank expert by expert (local experts ascending), an expert's rows in slot order, which is
+ * what deepep_ll_dispatch_send_by_dest emits, and its message starts at row s * slot_rows.  With the
+ * gathered route counts every row's place then follows by arithmetic -- row j of source s belongs to
+ * the expert whose run of that source's column of the counts holds j -- so nothing is read from the
+ * rows to index them and no record list is needed: one index launch and the row copy, both sides of
+ * every (expert, source) pair contiguous.  Outputs as deepep_ll_dispatch_recv_by_source.
+ *   all_num_routed     [R, E] int32, as for deepep_ll_exchange_metadata (counts above M read as M)
+ *   record_packed_row  [row_capacity] int32 (out) or NULL, indexed like the records of
+ *                      deepep_ll_exchange_metadata: sources ascending, a source's rows in message order
+ *   expected_rows      as for deepep_ll_dispatch_recv_by_source
+ *   workspace          256 + 8 * min(R * slot_rows, E * M) bytes (deepep_ll_by_source_workspace_bytes(E,
+ *                      R * slot_rows) is enough)
+ * Rows of a message beyond the source's slot are lost (their records read -1).
+ * Replaces ll_recv_unpack_v2 (csrc/kernels/efa_kernels.cu:2121-2231; ranges :991-1010) for this
+ * build's own wire order; the reference cannot take this shortcut because its senders leave the
+ * order inside a message to an atomic (:2378-2380). */
+int deepep_ll_dispatch_recv_by_source_ordered(const void* recv_by_source, int64_t slot_rows,
+                                              const int32_t* all_num_routed,
+                                              int hidden, int num_experts, int num_ranks, int rank,
+                                              int num_max_dispatch_tokens_per_rank, int row_format,
+                                              void* packed_recv_x, void* packed_recv_scales,
+                                              int32_t* packed_recv_src_info,
+                                              int64_t* packed_recv_layout_range,
+                                              int32_t* packed_recv_count,
+                                              int32_t* cumulative_local_expert_recv_stats,
+                                              uint32_t* tokens_per_expert, int32_t* record_packed_row,
+                                              int64_t row_capacity, int64_t expected_rows,
+                                              void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ */
 /* Low-latency combine                                                */
@@ -444,6 +477,7 @@ int deepep_ll_combine_recv(const void* combine_staging, const int64_t* topk_idx,
  * being the record's place among the rows of source s = source_rank[i].
  *   recv_counts                 [R] int32     } outputs of deepep_ll_exchange_metadata
  *   combine_remote_recv_offset  [R] int64     }
+ *   expected_rows   rows the caller expects to return (0 = unknown: row_capacity); sizes the grid only
  *   peer_recv_flat  [R] device array of pointers to the ranks' receive buffers (the buffer
  *                   deepep_ll_combine_recv_flat reads, flat form), peer_recv_rows [R] int64 their rows
  * Replaces the gather + un-sort of deep_ep/buffer.py:2601-2608 and a2a_combine_send
@@ -457,7 +491,7 @@ int deepep_ll_combine_send_by_dest(const void* x, const int32_t* record_packed_r
                                    int num_max_dispatch_tokens_per_rank, void* send_flat,
                                    const int32_t* recv_counts, const int64_t* combine_remote_recv_offset,
                                    void* const* peer_recv_flat, const int64_t* peer_recv_rows,
-                                   void* stream);
+                                   int64_t expected_rows, void* stream);
 
 /* deepep_ll_combine_recv reading the answers from the buffer an all-to-all leaves them in: one row
  * per row this rank sent, in send order (deepep_ll_dispatch_send_by_dest), so that pair (t, k) is

@@ -280,7 +280,7 @@ def recv_by_source_on_gpu(rt, buf, routed, rank, e, m, h, fmt, slot_rows, capaci
         capi.ptr(dev), slot_rows, capi.ptr(meta["recv_counts"]), capi.ptr(meta["source_offset"]),
         capi.ptr(meta["num_recv_tokens"]), capacity, h, e, r, m, fmt, capi.ptr(st.packed_recv_x),
         capi.ptr(st.packed_recv_scales), capi.ptr(st.packed_recv_src_info), capi.ptr(st.packed_recv_layout_range),
-        capi.ptr(st.packed_recv_count), None, capi.ptr(tokens_per_expert), None, capi.ptr(ws), ws.numel(),
+        capi.ptr(st.packed_recv_count), None, capi.ptr(tokens_per_expert), None, 0, capi.ptr(ws), ws.numel(),
         torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     return st, tokens_per_expert, meta
@@ -959,7 +959,7 @@ def test_every_rank_on_one_gpu_through_an_all_to_all(rt, fmt):
             capi.ptr(buf), slot_rows, capi.ptr(meta["recv_counts"]), capi.ptr(meta["source_offset"]),
             capi.ptr(meta["num_recv_tokens"]), capacity, h, e, r, t, fmt, capi.ptr(st.packed_recv_x),
             capi.ptr(st.packed_recv_scales), capi.ptr(st.packed_recv_src_info), capi.ptr(st.packed_recv_layout_range),
-            capi.ptr(st.packed_recv_count), None, None, None, capi.ptr(ws), ws.numel(),
+            capi.ptr(st.packed_recv_count), None, None, None, 0, capi.ptr(ws), ws.numel(),
             torch.cuda.current_stream().cuda_stream))
         torch.cuda.synchronize()
         want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
@@ -1093,11 +1093,12 @@ def all_to_all_dispatch(states, fmt):
     return routed
 
 
+@pytest.mark.parametrize("receive", ["from_tails", "ordered"])
 @pytest.mark.parametrize("delivery", ["flat", "slotted", "direct"])
 @pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
 @pytest.mark.parametrize("r,t,h,k,e", [(4, 40, 512, 3, 16), (8, 700, 512, 8, 64), (3, 5, 256, 2, 3)],
                          ids=["small", "chunked_receive", "one_expert_per_rank"])
-def test_all_to_all_round_trip_on_one_gpu(rt, oracle_c, fmt, delivery, r, t, h, k, e):
+def test_all_to_all_round_trip_on_one_gpu(rt, oracle_c, fmt, delivery, receive, r, t, h, k, e):
     """Every rank on the one GPU, the transport replaced by slice copies of contiguous ranges: send by
     destination, exchange metadata from the gathered counts, receive by source, experts, return by
     destination (into a flat buffer that is copied range by range, or -- `direct` -- straight into the
@@ -1112,13 +1113,18 @@ def test_all_to_all_round_trip_on_one_gpu(rt, oracle_c, fmt, delivery, r, t, h, 
         st.dispatch_send(x_all[rank].cuda(), topk_all[rank].cuda())
         states.append(st)
     torch.cuda.synchronize()
-    all_to_all_dispatch(states, fmt)
+    routed = all_to_all_dispatch(states, fmt)
     ys = []
     for rank, st in enumerate(states):
         poison_outputs_keep_pair_slot(st)
         st.record_packed_row.fill_(-7)
-        st.dispatch_recv()
+        st.tokens_per_expert.fill_(-7)
+        if receive == "ordered":  # the messages are in this build's own order: placed from the counts alone
+            st.dispatch_recv_ordered(routed)
+        else:
+            st.dispatch_recv()
         torch.cuda.synchronize()
+        assert torch.equal(st.tokens_per_expert, st.packed_recv_count)
         want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
         check_dispatch(st, want, fmt)
         n = int(st.meta["num_recv_tokens"][1])
@@ -1245,8 +1251,9 @@ def test_all_to_all_hand_derived_world(rt):
     assert torch.equal(out.cpu().float(), expect)
 
 
-@pytest.mark.parametrize("t", [24, 1500], ids=["one_workgroup_per_source", "chunked"])
-def test_dispatch_recv_by_source_clamps_a_pair_to_max_tokens(rt, t):
+@pytest.mark.parametrize("t,hint", [(24, 0), (1500, 0), (1500, 1500)],
+                         ids=["one_workgroup_per_source", "chunked", "one_workgroup_per_source_past_its_hint"])
+def test_dispatch_recv_by_source_clamps_a_pair_to_max_tokens(rt, t, hint):
     """Slots wider than M and senders that put more than M rows into one (expert, source) pair: the pair keeps
     its first M rows in arrival order, the counts and ranges count only those, and an expert's ranges stay
     inside its R * M packed slots -- what the staged receive does with an over-full count."""
@@ -1268,7 +1275,7 @@ def test_dispatch_recv_by_source_clamps_a_pair_to_max_tokens(rt, t):
         capi.ptr(buf.cuda()), slot_rows, capi.ptr(meta["recv_counts"]), capi.ptr(meta["source_offset"]),
         capi.ptr(meta["num_recv_tokens"]), capacity, h, e, r, m, fmt, capi.ptr(st.packed_recv_x),
         capi.ptr(st.packed_recv_scales), capi.ptr(st.packed_recv_src_info), capi.ptr(st.packed_recv_layout_range),
-        capi.ptr(st.packed_recv_count), None, None, capi.ptr(rec), capi.ptr(ws), ws.numel(),
+        capi.ptr(st.packed_recv_count), None, None, capi.ptr(rec), hint, capi.ptr(ws), ws.numel(),
         torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     epr, n_slots = e // r, r * m
@@ -1302,3 +1309,65 @@ def test_dispatch_recv_by_source_clamps_a_pair_to_max_tokens(rt, t):
         assert count[le] == begin and begin <= n_slots
     assert max(count) == n_slots or t < 30  # source 1 alone fills its half of every expert
     assert rec[:i].cpu().tolist() == want_rec
+
+
+def test_ordered_receive_with_slots_too_small_and_counts_too_large(rt):
+    """The ordered receive on hostile inputs: a source whose message does not fit its slot loses the rows past
+    it (their records read -1, the ranges count only what was kept), and a count above M is read as M."""
+    r, rank, t, h, k, e, fmt = 2, 0, 30, 512, 4, 8, O.ROW_FP8
+    epr = e // r
+    x_all, topk_all, _ = make_world(r, t, h, k, e, seed=17, drop=0)
+    topk_all[1, :, :] = torch.tensor([0, 1, 2, 3])  # source 1 sends t rows to each of rank 0's four experts
+    slot_rows = 2 * t + 7  # ... but its slot holds two experts' worth and a bit
+    states = []
+    for s_ in range(r):
+        st = rt.ll.AllToAllState(rt.ll.LLShape(r, s_, e, t, h, k, fmt), slot_rows=slot_rows)
+        st.dispatch_send(x_all[s_].cuda(), topk_all[s_].cuda())
+        states.append(st)
+    torch.cuda.synchronize()
+    routed = torch.stack([st.send_count for st in states])
+    dst = states[rank]
+    dst.recv_by_source.fill_(0xEE)
+    for s_, src in enumerate(states):
+        lo, hi = [int(v) for v in src.send_cumsum[rank:rank + 2].cpu()]
+        n = min(hi - lo, slot_rows)
+        dst.recv_by_source[s_ * slot_rows:s_ * slot_rows + n] = src.send_rows[lo:lo + n]
+    routed_big = routed.clone()
+    routed_big[0, 1] += 1000  # nonsense from source 0 for expert 1: read as M rows
+    for mat in (routed, routed_big):
+        poison_outputs_keep_pair_slot(dst)
+        dst.record_packed_row.fill_(-7)
+        dst.dispatch_recv_ordered(mat)
+        torch.cuda.synchronize()
+        sent = mat[:, rank * epr:(rank + 1) * epr].cpu().clamp(max=t)  # [source, local expert]
+        want_rec, begin = [], [0] * epr
+        kept = torch.zeros((epr, r), dtype=torch.int64)
+        for s_ in range(r):
+            first = 0
+            for le in range(epr):
+                c = int(sent[s_, le])
+                kept[le, s_] = max(0, min(c, slot_rows - first))
+                first += c
+        layout = dst.packed_recv_layout_range.cpu()
+        for le in range(epr):
+            b = 0
+            for s_ in range(r):
+                n = int(kept[le, s_])
+                assert int(layout[le, s_]) == (((b << 32) | n) if n else 0)
+                b += n
+            assert int(dst.packed_recv_count[le]) == b
+        for s_ in range(r):
+            for le in range(epr):
+                b = int(kept[le, :s_].sum())
+                want_rec += [le * r * t + b + j if j < int(kept[le, s_]) else -1 for j in range(int(sent[s_, le]))]
+        n_rec = min(len(want_rec), dst.row_capacity)
+        assert dst.record_packed_row[:n_rec].cpu().tolist() == want_rec[:n_rec]
+        if mat is routed:  # the rows kept are the oracle's rows, in place
+            want = O.ll_dispatch(list(x_all), list(topk_all), rank, e, t, fmt)
+            px = dst.packed_recv_x.view(torch.uint8).cpu()
+            for le in range(epr):
+                n0 = int(kept[le, 0])
+                assert torch.equal(px[le, :n0], want["packed_recv_x"][le, :n0])  # source 0 fits whole
+                n1 = int(kept[le, 1])
+                full0 = int(want["packed_recv_layout_range"][le, 0] & 0xFFFFFFFF)
+                assert torch.equal(px[le, n0:n0 + n1], want["packed_recv_x"][le, full0:full0 + n1])
