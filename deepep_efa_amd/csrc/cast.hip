@@ -6,7 +6,10 @@
 
 namespace deepep {
 
-template <int kFmt>
+// kStream: the rows exceed what the caches are worth spending on (they are read once), so they are loaded
+// with the non-temporal hint: 16.5 against 17.5 us at 4096 x 7168 with the rows coming from HBM.  The
+// results are stored the ordinary way in either case: whoever packs or sends them next reads them.
+template <int kFmt, bool kStream>
 __global__ __launch_bounds__(256) void per_token_cast_kernel(const uint8_t* __restrict__ x, int64_t num_rows,
                                                              int num_cols, int pieces_per_row,
                                                              uint8_t* __restrict__ x_fp8,
@@ -22,8 +25,8 @@ __global__ __launch_bounds__(256) void per_token_cast_kernel(const uint8_t* __re
     u32x4 lo = {0u, 0u, 0u, 0u}, hi = {0u, 0u, 0u, 0u};
     if (live) {
         const uint8_t* src = x + (row * num_cols + int64_t(group) * kGroup + (lane & 7) * 16) * 2;
-        lo = *reinterpret_cast<const u32x4*>(src);
-        hi = *reinterpret_cast<const u32x4*>(src + 16);
+        lo = load_u32x4<kStream>(src);
+        hi = load_u32x4<kStream>(src + 16);
     }
     uint32_t scale_bits;
     const u32x4 q = quantise_16<kFmt>(lo, hi, scale_bits);
@@ -58,17 +61,20 @@ extern "C" int deepep_per_token_cast_to_fp8(const void* x, int num_rows, int num
     const uint8_t* xb = reinterpret_cast<const uint8_t*>(x);
     uint8_t* qb = reinterpret_cast<uint8_t*>(x_fp8);
     uint8_t* sb = reinterpret_cast<uint8_t*>(scales);
+    const bool streams = int64_t(num_rows) * num_cols * 3 > send_stream_bytes();
+#define DEEPEP_LAUNCH_CAST(FMT)                                                                                  \
+    do {                                                                                                         \
+        if (streams)                                                                                             \
+            per_token_cast_kernel<FMT, true><<<dim3(unsigned(blocks)), 256, 0, s>>>(xb, num_rows, num_cols, pieces, qb, sb);  \
+        else                                                                                                     \
+            per_token_cast_kernel<FMT, false><<<dim3(unsigned(blocks)), 256, 0, s>>>(xb, num_rows, num_cols, pieces, qb, sb); \
+    } while (0)
     switch (row_format) {
-        case kRowFP8:
-            per_token_cast_kernel<kRowFP8><<<dim3(unsigned(blocks)), 256, 0, s>>>(xb, num_rows, num_cols, pieces, qb, sb);
-            break;
-        case kRowFP8Pow2:
-            per_token_cast_kernel<kRowFP8Pow2><<<dim3(unsigned(blocks)), 256, 0, s>>>(xb, num_rows, num_cols, pieces, qb, sb);
-            break;
-        default:
-            per_token_cast_kernel<kRowFP8UE8M0><<<dim3(unsigned(blocks)), 256, 0, s>>>(xb, num_rows, num_cols, pieces, qb, sb);
-            break;
+        case kRowFP8: DEEPEP_LAUNCH_CAST(kRowFP8); break;
+        case kRowFP8Pow2: DEEPEP_LAUNCH_CAST(kRowFP8Pow2); break;
+        default: DEEPEP_LAUNCH_CAST(kRowFP8UE8M0); break;
     }
+#undef DEEPEP_LAUNCH_CAST
     EP_LAUNCH_CHECK();
     return 0;
 }

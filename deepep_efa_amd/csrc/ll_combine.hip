@@ -40,6 +40,7 @@ __device__ __forceinline__ void combine_send_rows_impl(const CombineSendArgs& a,
 
     WaveSegments<kPer> seg_table;
     int64_t ranges[kPer];
+    DEEPEP_PHASE(0);
     wave_load_int64<kPer>(a.layout_range, num_segments, lane, ranges);
 #pragma unroll
     for (int u = 0; u < kPer; ++u) {
@@ -51,6 +52,7 @@ __device__ __forceinline__ void combine_send_rows_impl(const CombineSendArgs& a,
         seg_table.aux[u] = int(ranges[u] >> 32);
     }
     wave_segments_finish(seg_table);
+    DEEPEP_PHASE(1);
 
     const int64_t row_bytes = int64_t(a.hidden) * 2;
     const int num_vec = int(row_bytes / 16);
@@ -79,6 +81,7 @@ __device__ __forceinline__ void combine_send_rows_impl(const CombineSendArgs& a,
         row_part_range(num_vec, parts, part, v_begin, v_end);
         wave_copy_vec16<4, kStream>(src, dst, v_begin, v_end, lane);
     }
+    DEEPEP_PHASE(2);
 }
 
 template <bool kStream>
@@ -239,6 +242,7 @@ __device__ __forceinline__ void combine_recv_piece(const CombineRecvArgs& a, int
         for (int i = 0; i < 4; ++i) o[i] = pack_bf16x2(acc[2 * i], acc[2 * i + 1]);
         store_u32x4<kStream>(a.out + int64_t(t) * row_bytes + off, o);
     }
+    DEEPEP_PHASE(3);
 }
 
 // kStream: the gathered rows exceed what the caches hold, so they are read (and the result written)

@@ -229,11 +229,28 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
         }
     }
 
+    // ---- every index load of the ranking, issued before anything waits -----
+    // The loads are unconditional (an index that is not wanted is clamped to one that exists and its
+    // value dropped): without branches around them the compiler can count them, so the first wait of
+    // wave 0 -- for the token's own selections -- does not also wait out a second round trip for the
+    // entries it sweeps.  The wave then has one memory round trip in front of its ballots, not two.
+    const int chunk = a.tokens_per_chunk > 0 ? t / a.tokens_per_chunk : 0;
+    const int sweep_begin = chunk * a.tokens_per_chunk * num_topk;
+    constexpr int kSweepAhead = 4;
+    const int64_t own_v = my_topk[entry0 + (tid < num_topk ? tid : num_topk - 1)];     // threads 0..K-1: selection tid
+    const int64_t sel_v = my_topk[entry0 + (lane < num_topk ? lane : num_topk - 1)];   // lane k of every wave: selection k
+    int64_t ahead_v[kSweepAhead];
+#pragma unroll
+    for (int r = 0; r < kSweepAhead; ++r) {
+        const int i = sweep_begin + tid + r * int(blockDim.x);
+        ahead_v[r] = my_topk[i < entry0 ? i : entry0];
+    }
+
     // ---- per-selection bookkeeping, once per token --------------------------
     int my_expert = -1, my_slot = -1, dst_rank = -1, local = 0;  // threads 0..K-1: selection k = tid
     int direct_begin = 0;
     if (tid < num_topk) {
-        const int64_t v = my_topk[entry0 + tid];
+        const int64_t v = own_v;
         if (v >= 0 && v < num_experts) {
             my_expert = int(v);
             // my_expert / E_l by multiply-high; magic 0 stands for E_l == 1
@@ -265,8 +282,6 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
     }
     // Medium and large batches: the token sweeps only the earlier entries of its own chunk; what the
     // chunks before it hold of each selection's expert comes from their histograms.
-    const int chunk = a.tokens_per_chunk > 0 ? t / a.tokens_per_chunk : 0;
-    const int sweep_begin = chunk * a.tokens_per_chunk * num_topk;
     int chunk_base = 0;
     if (chunk > 0 && tid < num_topk && my_expert >= 0) {
         const int32_t* hist = reinterpret_cast<const int32_t*>(a.scratch_base + int64_t(b) * a.scratch_stride);
@@ -286,20 +301,16 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
     // counts, per selection, how many of its entries name that selection's expert (a ballot and a
     // popcount, against the token's own entries read as wave-uniform values) and leaves the counts
     // in LDS.
-    constexpr int kSweepAhead = 4;
     int ahead[kSweepAhead];  // -1: no entry
 #pragma unroll
     for (int r = 0; r < kSweepAhead; ++r) {
         const int i = sweep_begin + tid + r * int(blockDim.x);
-        const int64_t v = i < entry0 ? my_topk[i] : -1;
-        ahead[r] = v >= 0 && v < num_experts ? int(v) : -1;
+        const int64_t v = ahead_v[r];
+        ahead[r] = i < entry0 && v >= 0 && v < num_experts ? int(v) : -1;
     }
     // lane k of every wave holds the token's selection k (-2: none, matches no entry)
     int sel = -2;
-    if (lane < num_topk) {
-        const int64_t v = my_topk[entry0 + lane];
-        if (v >= 0 && v < num_experts) sel = int(v);
-    }
+    if (lane < num_topk && sel_v >= 0 && sel_v < num_experts) sel = int(sel_v);
     const int w = wave_in_block();
     int my_count = 0;  // lane k: this wave's entries naming selection k's expert
     for (int k = 0; k < num_topk; ++k) {
@@ -618,11 +629,22 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
         row_part_range(num_vec, parts, part, it.v_begin, it.v_end);
         it.carries_tail = part == parts - 1;  // the last part is the shortest
     };
+    // What the tail-carrying part of a row moves besides payload: one scale word per lane (the first 64;
+    // a wider row's remainder is copied after the stores) and, in lane 0, the source index.  They are
+    // loaded with the payload, not behind its stores: one round trip per row instead of two.
+    const int scale_dwords = int(scale_bytes / 4);
+    const bool has_scales = a.packed_scales != nullptr && scale_dwords > 0;
+    uint32_t tail_scale = 0;
+    int32_t tail_info = 0;
     auto load_first = [&](const RecvItem& it, u32x4 (&r)[kRecvDepth]) {
 #pragma unroll
         for (int u = 0; u < kRecvDepth; ++u) {
             const int v = it.v_begin + u * kWave + lane;
             if (v < it.v_end) r[u] = load_u32x4<kStream>(it.src + int64_t(v) * 16);
+        }
+        if (it.carries_tail) {
+            if (has_scales && lane < scale_dwords) tail_scale = reinterpret_cast<const uint32_t*>(it.src + data_pad)[lane];
+            if (lane == 0) tail_info = *reinterpret_cast<const int32_t*>(it.src + data_pad + align16(scale_bytes));
         }
     };
     auto finish = [&](const RecvItem& it, const u32x4 (&r)[kRecvDepth]) {
@@ -637,13 +659,13 @@ __device__ __forceinline__ void recv_rows_impl(const RecvArgs& a, int block, int
         }
         wave_copy_vec16<kRecvDepth, kStream>(it.src, dst, it.v_begin + kRecvDepth * kWave, it.v_end, lane);
         if (!it.carries_tail) return;
-        if (a.packed_scales != nullptr && scale_bytes > 0) {
+        if (has_scales) {
             const uint32_t* s32 = reinterpret_cast<const uint32_t*>(it.src + data_pad);
             uint32_t* d32 = reinterpret_cast<uint32_t*>(a.packed_scales + out_row * scale_bytes);
-            for (int v = lane; v < int(scale_bytes / 4); v += kWave) d32[v] = s32[v];
+            if (lane < scale_dwords) d32[lane] = tail_scale;
+            for (int v = kWave + lane; v < scale_dwords; v += kWave) d32[v] = s32[v];
         }
-        if (lane == 0)
-            a.src_info[out_row] = *reinterpret_cast<const int32_t*>(it.src + data_pad + align16(scale_bytes));
+        if (lane == 0) a.src_info[out_row] = tail_info;
     };
 
     RecvItem it;
