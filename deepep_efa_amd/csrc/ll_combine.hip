@@ -335,11 +335,15 @@ __global__ __launch_bounds__(1024) void ll_combine_send_by_dest_kernel(CombineBy
     const int lane = lane_id();
     const int64_t row_bytes = int64_t(a.num_vec) * 16;
     for (int64_t i = blockIdx.x; i < records; i += gridDim.x) {
+        // padded_index[i] is i whenever the records come from deepep_ll_exchange_metadata, so the packed row
+        // is fetched for that guess together with the record itself, and again only if the guess was wrong:
+        // one round trip in front of the row loads instead of two
         const uint32_t p = a.padded_index[i];
-        if (int64_t(p) >= a.row_capacity) continue;
-        const int64_t src_row = a.record_packed_row[p];
-        if (src_row < 0 || src_row >= a.x_rows) continue;  // the record has no row
+        int64_t src_row = a.record_packed_row[i];
         const int64_t offset = a.combine_send_offset[i];
+        if (int64_t(p) >= a.row_capacity) continue;
+        if (int64_t(p) != i) src_row = a.record_packed_row[p];
+        if (src_row < 0 || src_row >= a.x_rows) continue;  // the record has no row
         uint8_t* dst;
         if (a.peer_recv == nullptr) {
             if (offset >= a.row_capacity) continue;
