@@ -141,6 +141,101 @@ def rotating(fns):
     return call
 
 
+def phase_marks(torch, args):
+    """Where the microseconds go inside the two step kernels: the timing build (bench_phase.hip: the library's
+    sources with the DEEPEP_PHASE hook writing the 100 MHz wall clock) runs the headline step, replayed and after
+    read flushes, and prints for each kind of workgroup the mean / latest time since the launch's first mark at
+    which its first and its last wave pass every mark."""
+    import ctypes
+
+    import numpy as np
+    from deepep_efa_amd import _capi
+    path = os.path.join(ROOT, "bench_phase.so")
+    if not os.path.exists(path):
+        raise ImportError(f"{path} is missing: build it with `python deepep_efa_amd/build.py`")
+    _capi._lib, _capi.LIB_PATH = None, path  # every C-ABI call below goes to the timing build
+    lib = _capi.load()
+    from deepep_efa_amd import ll_runtime, loopback
+    t, h, k, e, r, rank = args.tokens, args.hidden, args.topk, args.experts, args.ranks, args.rank
+    st = ll_runtime.LowLatencyState(ll_runtime.LLShape(r, rank, e, t, h, k, ll_runtime.ROW_FP8))
+    world = loopback.LoopbackWorld(r, rank, seed=args.seed)
+    world.synthesise(t, h, k, e)
+    x, topk = world.own_inputs()
+    w = torch.softmax(torch.randn((t, k), generator=torch.Generator().manual_seed(args.seed)), dim=-1).cuda()
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    y = torch.randn((e // r, r * t, h), device="cuda").to(torch.bfloat16)
+    st.dispatch_send(x, topk)
+    world.dispatch_from_peers(st)
+    st.dispatch_recv()
+    world.combine_from_peers(st, mode=1, seed=args.seed + 2)
+    torch.cuda.synchronize()
+    assert lib.deepep_ll_dispatch_is_single_launch(t, k, e, r, t * k) == 1, "the marks are read per workgroup of one launch"
+    log = torch.zeros((16384, 16), dtype=torch.int64, device="cuda")
+    lib.bench_phase_set_log.argtypes = [ctypes.c_void_p]
+    assert lib.bench_phase_set_log(ctypes.c_void_p(log.data_ptr())) == 0
+    flush = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
+
+    def collect(fn, cold, reps=40):
+        acc, n = None, 0
+        for i in range(reps + 5):
+            if cold:
+                flush.max()
+            else:
+                fn()
+            log.zero_()
+            torch.cuda.synchronize()
+            fn()
+            torch.cuda.synchronize()
+            if i < 5:
+                continue
+            ticks = log.cpu().numpy().astype("float64")
+            us = (ticks - ticks[ticks > 0].min()) * 0.01
+            us[ticks == 0] = float("nan")
+            acc = us if acc is None else acc + us
+            n += 1
+        return acc / n
+
+    def report(title, us, groups, names):
+        print(title)
+        for gname, rows in groups:
+            blk = us[rows]
+            if blk.size == 0 or np.isnan(blk).all():
+                continue
+            with np.errstate(all="ignore"):
+                mean, latest = np.nanmean(blk, axis=0), np.nanmax(blk, axis=0)
+            print(f"  {gname} ({blk.shape[0]} workgroups)")
+            for half, label in ((0, "first wave"), (8, "last wave ")):
+                cells = [f"{names[gname][i]} {mean[half + i]:.2f}/{latest[half + i]:.2f}" for i in range(8)
+                         if i in names[gname] and not np.isnan(mean[half + i])]
+                print(f"    {label}: " + "   ".join(cells))
+
+    send_marks = {0: "start", 1: "indices back", 3: "ranked+quantised", 4: "addresses known", 5: "stores begin",
+                  6: "stores issued"}
+    recv_marks = {0: "start", 1: "segment table", 2: "row loads begin", 3: "first row stored"}
+    names = {"send": send_marks, "receive": recv_marks, "metadata": {0: "start", 1: "segment table"},
+             "reduce": {0: "start", 1: "rows back", 2: "summed", 3: "stored"},
+             "row return": {0: "start", 1: "segment table", 2: "copies issued"}}
+    stamp = build_stamp(lib)
+    print(f"per-phase marks, {t} tokens x {h}, top-{k} of {e} experts, rank {rank} of {r}: mean/latest microseconds since "
+          "the launch's first mark, averaged over 40 launches")
+    print(f"build: abi={stamp['abi']} source={stamp['source_sha']}")
+    for cold in (False, True):
+        state = "every launch after 512 MiB of reads" if cold else "replayed"
+        us = collect(lambda: st.dispatch(x, topk), cold)
+        live = np.where(~np.isnan(us).all(axis=1))[0]
+        blocks = int(live.max()) + 1
+        report(f"ll_dispatch_fused_kernel, {state} ({blocks} workgroups)", us,
+               [("send", slice(0, t)), ("receive", slice(t + 1, blocks - 1)), ("metadata", slice(blocks - 1, blocks))],
+               names)
+        us = collect(lambda: st.combine(y, topk, w, out), cold)
+        live = np.where(~np.isnan(us).all(axis=1))[0]
+        blocks = int(live.max()) + 1
+        reduce_blocks = (t * ((2 * h + 1023) // 1024) + 3) // 4
+        report(f"ll_combine_fused_kernel, {state} ({blocks} workgroups)", us,
+               [("reduce", slice(0, reduce_blocks)), ("row return", slice(reduce_blocks, blocks))], names)
+    lib.bench_phase_set_log(None)
+
+
 def calibrate_copy(torch, _capi, lib):
     """A plain copy through the pack kernel with identity row ids: 32768 rows x 14336 B read and written once.
     Under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` the counters of pack_rows_kernel divided into the
@@ -566,6 +661,9 @@ def main():
     ap.add_argument("--no-skew-stress", action="store_true", help="skip the skewed 8192-token stress section")
     ap.add_argument("--only-ll-4096", action="store_true",
                     help="only time the LL entry points at 4096 tokens (8 ranks x 32 experts) and print that section")
+    ap.add_argument("--phase-marks", action="store_true",
+                    help="only print the in-kernel phase timestamps of the two step kernels (timing build "
+                         "bench_phase.so)")
     ap.add_argument("--skew-stress", action="store_true",
                     help="only time the LL entry points at the skewed 8192-token, 64-rank stress size and print that")
     args = ap.parse_args()
@@ -575,11 +673,14 @@ def main():
         sys.exit(2)
 
     import torch
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+    if args.phase_marks:
+        phase_marks(torch, args)
+        return
     from deepep_efa_amd import _capi, ll_runtime, loopback
 
     lib = _capi.load()
-    assert torch.cuda.is_available(), "bench.py needs the GPU"
-    torch.cuda.set_device(0)
     if args.calibrate_copy:
         calibrate_copy(torch, _capi, lib)
         return

@@ -46,6 +46,25 @@ def build_bench_probe(verbose: bool = True) -> str:
     return BENCH_PROBE
 
 
+BENCH_PHASE_SRC = os.path.join(os.path.dirname(HERE), "bench_phase.hip")
+BENCH_PHASE = os.path.join(os.path.dirname(HERE), "bench_phase.so")
+
+
+def build_bench_phase(verbose: bool = True) -> str:
+    """Builds the timing build for `bench.py --phase-marks` (bench_phase.hip beside bench.py -> bench_phase.so):
+    the whole C ABI again, with the two low-latency kernel files compiled with their phase marks switched on."""
+    rest = [s for s in SOURCES if s not in ("ll_dispatch.hip", "ll_combine.hip")]
+    cmd = (["hipcc"] + FLAGS + [f"-I{os.path.dirname(HERE)}", BENCH_PHASE_SRC] + [os.path.join(CSRC, s) for s in rest]
+           + ["-o", BENCH_PHASE])
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if verbose and out.strip():
+        print(out, file=sys.stderr)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    return BENCH_PHASE
+
+
 HOST_MODULE = os.path.join(HERE, "deep_ep_cpp.so")
 
 
@@ -75,3 +94,4 @@ if __name__ == "__main__":
     print(build_hip_library())
     print(build_host_module())
     print(build_bench_probe())
+    print(build_bench_phase())
