@@ -438,6 +438,14 @@ def bench_pack(torch, _capi, lib, loopback, args):
         us = time_calls(torch, fn, n)
         res[name] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
                      "frac_of_8TBps": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # The packs read every source row once per destination rank that wants it (s / t times on average).  The
+    # figure above counts each of those reads; if the caches served all but the first, HBM would see only the
+    # unique bytes: every source row once, every packed row once.  The counters say the L2 does not serve them
+    # (it fetches the full read bytes from the fabric); whether the memory-side cache does they cannot tell.
+    for name, row in (("pack_bf16", 2 * h), ("pack_fp8", h + h // 32)):
+        unique = t * row + s * row + s * 8
+        res[name]["unique_bytes"] = unique
+        res[name]["frac_of_8TBps_on_unique_bytes"] = round(unique / res[name]["us"] / 1e3 / HBM_PEAK_GBS, 4)
     return res
 
 
