@@ -58,6 +58,11 @@ def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0, packed=None):
         "dispatch_send_by_dest": t * 2 * h + t * k * 8 * 2 + p * stride + t * k * 4 + e * 8,
         "combine_send_by_dest": rv * 2 * h * 2 + rv * 16,
         "combine_recv_flat": p * 2 * h + t * k * 16 + e * 4 + t * 2 * h,
+        # the five launches (or launch pairs) of a step over that transport: send by destination, exchange
+        # metadata, ordered receive, return by destination, reduce from the flat buffer
+        "all_to_all_step": (t * 2 * h + t * k * 8 * 2 + p * stride + t * k * 4 + e * 8) + (r * e * 4 + rv * 16 + r * 24)
+                           + (rv * stride + rv * packed + small + r * e * 4 + rv * 8) + (rv * 2 * h * 2 + rv * 16)
+                           + (p * 2 * h + t * k * 16 + e * 4 + t * 2 * h),
     }
 
 
@@ -311,7 +316,20 @@ def all_to_all_entries(torch, _capi, lib, ll_runtime, st, world, x, topk, weight
     a2a.dispatch_recv()
     a2a.recv_flat.normal_()  # the peers' answers, one row per row sent
     torch.cuda.synchronize()
+    meta = a2a.meta
+    meta_args = [_capi.ptr(routed), e, r, sh.rank, a2a.slot_rows, a2a.row_capacity] + [_capi.ptr(meta[n]) for n in (
+        "send_counts", "recv_counts", "totals", "combine_remote_recv_offset", "source_rank", "source_offset",
+        "padded_index", "combine_send_offset", "num_recv_tokens", "tokens_per_expert")]
+
+    def whole_step():  # everything one rank launches for a step over such a transport, in stream order
+        a2a.dispatch_send(x, topk)
+        _capi.check(lib.deepep_ll_exchange_metadata(*meta_args, torch.cuda.current_stream().cuda_stream))
+        a2a.dispatch_recv_ordered(routed)
+        a2a.combine_send(y)
+        a2a.combine_recv(topk, weights, out)
+
     return {
+        "all_to_all_step": whole_step,
         "dispatch_send_by_dest": lambda: a2a.dispatch_send(x, topk),
         "dispatch_recv_by_source": lambda: a2a.dispatch_recv(),
         "dispatch_recv_by_source_ordered": lambda: a2a.dispatch_recv_ordered(routed),

@@ -33,6 +33,7 @@ namespace deepep {
 
 __host__ __device__ inline int64_t align256(int64_t v) { return (v + 255) & ~int64_t(255); }
 
+constexpr int kByDestInBlockEntries = 2048;  // by-destination batches up to here build their tables in the send launch
 constexpr int kSweepChunkEntries = 2048;  // a token sweeps at most this many earlier entries itself
 
 // Tokens per sweep chunk: whole tokens, about kSweepChunkEntries entries.
@@ -117,6 +118,12 @@ constexpr int kFusedMaxEntries = 8192;     // send + receive in one launch up to
 constexpr int kSelfRankMaxEntries = 8192;  // the send kernel ranks its own slots, unaided, up to here
 constexpr int kSendMaxWaves = 16;
 
+struct ByDestTables {
+    int32_t* expert_prefix;  // [E + 1]
+    int32_t* rank_counts;    // [R]
+    int64_t* rank_cumsum;    // [R + 1]
+};
+
 struct SendArgs {
     const uint8_t* x;
     const int64_t* topk_idx;
@@ -135,6 +142,11 @@ struct SendArgs {
     // By-destination form: send_slots is one buffer of rows, contiguous per destination rank, and every
     // row (the rank's own included) goes to row expert_prefix[expert] + slot of it.  Null: per-expert slots.
     const int32_t* expert_prefix;
+    // Small by-destination batches: no launch builds the tables first.  Every token's workgroup counts
+    // the batch's entries per expert itself and scans them in LDS (a few barriers beside its row loads,
+    // cheaper than a launch), and the counting row writes the tables out.
+    int prefix_in_block;
+    ByDestTables by_dest;
 };
 
 // Final destination of the rows a rank sends to its own experts, used by the
@@ -152,6 +164,49 @@ struct alignas(16) SendLds {
     uint64_t sel_row[kMaxTopk];                   // where selection k's payload goes (0: nowhere)
     uint64_t sel_scale[kMaxTopk];                 // where its scales go
 };
+
+// hist[e] (LDS, [E + 1]) = entries of topk_idx[0 .. n) naming expert e, clamped to max_tokens, then their
+// exclusive prefix over the experts with the total in hist[E]; the whole workgroup takes part.
+// counts_out (may be null): the clamped counts.
+__device__ __forceinline__ void expert_prefix_in_lds(const int64_t* __restrict__ topk_idx, int n, int num_experts,
+                                                     int max_tokens, int32_t* hist, int32_t* wave_totals,
+                                                     int32_t* counts_out) {
+    const int tid = threadIdx.x, threads = blockDim.x;
+    for (int e = tid; e < num_experts; e += threads) hist[e] = 0;
+    lds_barrier();
+    for (int base = 0; base < n; base += 4 * threads) {  // four loads in flight per thread
+        int64_t v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int i = base + u * threads + tid;
+            v[u] = i < n ? topk_idx[i] : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (v[u] >= 0 && v[u] < num_experts) atomicAdd(&hist[int(v[u])], 1);
+    }
+    lds_barrier();
+    for (int e = tid; e < num_experts; e += threads) {
+        const int c = hist[e] < max_tokens ? hist[e] : max_tokens;
+        hist[e] = c;
+        if (counts_out != nullptr) counts_out[e] = c;
+    }
+    lds_barrier();
+    block_exclusive_scan(hist, num_experts, wave_totals);
+}
+
+// The per-rank tables of the by-destination form from the prefix in LDS.
+__device__ __forceinline__ void by_dest_tables_out(const int32_t* hist, int num_experts, int num_ranks,
+                                                   const ByDestTables& out) {
+    const int tid = threadIdx.x, threads = blockDim.x;
+    for (int e = tid; e <= num_experts; e += threads) out.expert_prefix[e] = hist[e];
+    const int experts_per_rank = num_experts / num_ranks;
+    for (int r = tid; r < num_ranks; r += threads) {
+        out.rank_counts[r] = hist[(r + 1) * experts_per_rank] - hist[r * experts_per_rank];
+        out.rank_cumsum[r] = hist[r * experts_per_rank];
+    }
+    if (tid == 0) out.rank_cumsum[num_ranks] = hist[num_experts];
+}
 
 // The per-source counting workgroup.
 __device__ __forceinline__ void send_count_block(const SendArgs& a, int b, int32_t* lds_hist) {
@@ -189,7 +244,8 @@ __device__ __forceinline__ void send_count_block(const SendArgs& a, int b, int32
 // scales and tails stored, the ordinary way: the hint measured slower on those (63 and 56 us).
 template <int kFmt, bool kStream>
 __device__ __forceinline__ void send_token_block(const SendArgs& a, const DirectOut& direct, int b, int t,
-                                                 int block_in_token, SendLds& lds) {
+                                                 int block_in_token, SendLds& lds, int32_t* lds_hist,
+                                                 int32_t* lds_wave_totals) {
     const int lane = lane_id(), tid = threadIdx.x;
     const int num_topk = a.num_topk, num_experts = a.num_experts;
     const int n = a.num_tokens * num_topk;
@@ -260,7 +316,12 @@ __device__ __forceinline__ void send_token_block(const SendArgs& a, const Direct
         }
     }
     int dest_first = 0;  // by-destination form: where the expert's run of rows begins in the send buffer
-    if (a.expert_prefix != nullptr && my_expert >= 0) dest_first = a.expert_prefix[my_expert];
+    if (a.prefix_in_block) {
+        expert_prefix_in_lds(my_topk, n, num_experts, a.max_tokens, lds_hist, lds_wave_totals, nullptr);
+        if (my_expert >= 0) dest_first = lds_hist[my_expert];
+    } else if (a.expert_prefix != nullptr && my_expert >= 0) {
+        dest_first = a.expert_prefix[my_expert];
+    }
     if (direct.packed_x != nullptr && tid < kWave) {
         // Rows for this rank's own experts go straight to the packed tensors, at the place the
         // reference's range builder gives them: behind the rows of the lower source ranks
@@ -442,11 +503,17 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_send_kernel(SendArgs 
         return;
     }
     if (y == a.num_tokens) {  // the counting row of the grid
-        // (the by-destination form has its counts already: ll_by_dest_prefix_kernel ran first)
-        if (blockIdx.x == 0 && a.expert_prefix == nullptr) send_count_block(a, blockIdx.z, lds_hist);
+        if (blockIdx.x != 0) return;
+        if (a.prefix_in_block) {  // small by-destination batch: this workgroup writes the tables out
+            expert_prefix_in_lds(a.topk_idx, a.num_tokens * a.num_topk, a.num_experts, a.max_tokens, lds_hist,
+                                 index_wave_totals, a.send_count);
+            by_dest_tables_out(lds_hist, a.num_experts, a.num_ranks, a.by_dest);
+        } else if (a.expert_prefix == nullptr) {
+            send_count_block(a, blockIdx.z, lds_hist);
+        }  // else: ll_by_dest_prefix_kernel ran first
         return;
     }
-    send_token_block<kFmt, kStream>(a, direct, blockIdx.z, y, blockIdx.x, lds);
+    send_token_block<kFmt, kStream>(a, direct, blockIdx.z, y, blockIdx.x, lds, lds_hist, index_wave_totals);
 }
 
 // ---------------------------------------------------------------------
@@ -730,7 +797,8 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_dispatch_fused_kernel
     const int block = blockIdx.x;
     if (block < num_send_blocks) {
         const DirectOut direct = {ra.packed_x, ra.packed_scales, ra.src_info};
-        send_token_block<kFmt, kStream>(sa, direct, 0, block / blocks_per_token, block % blocks_per_token, lds);
+        send_token_block<kFmt, kStream>(sa, direct, 0, block / blocks_per_token, block % blocks_per_token, lds, dyn_lds,
+                                        wave_totals);
     } else if (block == num_send_blocks) {
         send_count_block(sa, 0, dyn_lds);
     } else {
@@ -741,7 +809,9 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_dispatch_fused_kernel
 
 // ---------------------------------------------------------------------
 // By-destination send (what an all-to-all ships: one contiguous message per
-// peer).  Before the send kernel runs, one workgroup turns the route counts into
+// peer).  Before the send kernel runs (batches of more than kByDestInBlockEntries entries;
+// smaller ones build the same tables inside the send launch, every token's workgroup
+// for itself), one workgroup turns the route counts into
 // the tables the rows are placed by: send_count[e] (clamped to the M slots of a
 // pair), its exclusive prefix over the experts -- the first row of every expert's
 // run, experts ascending, hence destination ranks ascending -- and the per-rank
@@ -749,12 +819,6 @@ __global__ __launch_bounds__(kSendMaxWaves* kWave) void ll_dispatch_fused_kernel
 // Reference: the count + prefix phases of ll_dispatch_route_and_pack_v3
 // (csrc/kernels/efa_kernels.cu:2358-2371: ll_dispatch_count_kernel, prefix_sum_kernel).
 // ---------------------------------------------------------------------
-struct ByDestTables {
-    int32_t* expert_prefix;  // [E + 1]
-    int32_t* rank_counts;    // [R]
-    int64_t* rank_cumsum;    // [R + 1]
-};
-
 __global__ __launch_bounds__(1024) void ll_by_dest_prefix_kernel(const int64_t* __restrict__ topk_idx, int n,
                                                                  int num_experts, int num_ranks, int max_tokens,
                                                                  const int32_t* __restrict__ chunk_hist, int num_chunks,
@@ -797,13 +861,7 @@ __global__ __launch_bounds__(1024) void ll_by_dest_prefix_kernel(const int64_t* 
     }
     lds_barrier();
     block_exclusive_scan(hist, num_experts, wave_totals);
-    for (int e = tid; e <= num_experts; e += threads) out.expert_prefix[e] = hist[e];
-    const int experts_per_rank = num_experts / num_ranks;
-    for (int r = tid; r < num_ranks; r += threads) {
-        out.rank_counts[r] = hist[(r + 1) * experts_per_rank] - hist[r * experts_per_rank];
-        out.rank_cumsum[r] = hist[r * experts_per_rank];
-    }
-    if (tid == 0) out.rank_cumsum[num_ranks] = hist[num_experts];
+    by_dest_tables_out(hist, num_experts, num_ranks, out);
 }
 
 // ---------------------------------------------------------------------
@@ -845,7 +903,10 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
             topk_idx, n, tpc * num_topk, num_experts, scratch_bytes, ws);
         EP_LAUNCH_CHECK();
     }
-    if (by_dest != nullptr) {  // the tables the by-destination rows are placed by
+    // A small by-destination batch needs no launch for its tables: every token's workgroup counts the
+    // batch itself (kByDestInBlockEntries entries are a few loads per thread).
+    const bool prefix_in_block = by_dest != nullptr && tpc == 0 && n <= kByDestInBlockEntries;
+    if (by_dest != nullptr && !prefix_in_block) {  // the tables the by-destination rows are placed by
         EP_HOST_ASSERT(num_src == 1 && src_ranks == nullptr && fused_recv == nullptr && own_rows_direct == nullptr);
         const int chunks = tpc > 0 ? (num_tokens + tpc - 1) / tpc : 0;
         ll_by_dest_prefix_kernel<<<1, 1024, size_t(num_experts + 1) * sizeof(int32_t), stream>>>(
@@ -886,6 +947,10 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     sa.send_slots = reinterpret_cast<uint8_t*>(send_slots);
     sa.pair_slot = pair_slot, sa.recv_count = recv_count, sa.send_count = send_count;
     sa.expert_prefix = by_dest != nullptr ? by_dest->expert_prefix : nullptr;
+    sa.prefix_in_block = prefix_in_block ? 1 : 0;
+    sa.by_dest = by_dest != nullptr ? *by_dest : ByDestTables{nullptr, nullptr, nullptr};
+    if (by_dest != nullptr)
+        EP_HOST_ASSERT(num_src == 1 && src_ranks == nullptr && fused_recv == nullptr && own_rows_direct == nullptr);
 
     if (fused_recv != nullptr) {  // single launch: send workgroups, the counting workgroup, receive workgroups
         EP_HOST_ASSERT(tpc == 0 && num_src == 1 && src_ranks == nullptr);
@@ -937,7 +1002,7 @@ static int launch_send_side(const void* x, const int64_t* topk_idx, const int32_
     }
     if (index_was_fused != nullptr) *index_was_fused = index_rows > 0;
     const dim3 grid(blocks_per_token, num_tokens + 1 + index_rows, num_src);  // + the counting row, + the index rows
-    const size_t lds = size_t(index_rows > 0 ? 2 * (num_experts + 1) : num_experts) * sizeof(int32_t);
+    const size_t lds = size_t(index_rows > 0 ? 2 * (num_experts + 1) : num_experts + 1) * sizeof(int32_t);
     // own_rows_direct (the two-launch form of the one-call dispatch): as in the single launch, the rows
     // for this rank's own experts go straight to their packed position behind the lower ranks' rows
     EP_HOST_ASSERT(own_rows_direct == nullptr || (num_src == 1 && src_ranks == nullptr));

@@ -359,6 +359,170 @@ __global__ __launch_bounds__(kIndexThreads) void ll_by_source_ordered_index_kern
     }
 }
 
+// ---------------------------------------------------------------------
+// The ordered receive for small batches (at most kLargeBatchRows rows expected): index and copy in one
+// launch, like the staged receive's ll_recv_kernel.  Every workgroup works out the (expert, source)
+// pairs' numbers for itself in LDS -- sent(e, s) from the gathered counts, first(e, s) (where the pair
+// starts in its source's message) and kept(e, s) -- one thread per pair; a copying wave then holds kept
+// and first in its registers (WaveSegments) and walks the flat index space of the rows kept, one wave
+// per row part; the first E_l * R waves of the grid then write the records' packed rows, a pair each.
+// The last workgroup copies nothing: it writes layout_range, packed_count, stats and tokens_per_expert.
+// lds: [4 * (E_l * R + 1)] ints.
+// ---------------------------------------------------------------------
+struct OrderedRecvArgs {
+    const uint8_t* rows;            // [R * slot_rows] staged rows
+    const int32_t* all_num_routed;  // [R, E]
+    int num_experts, num_local_experts, num_ranks, rank, max_tokens;
+    int hidden, fmt, parts_log2;
+    int64_t slot_rows, row_capacity;
+    uint8_t* packed_x;
+    uint8_t* packed_scales;
+    int32_t* src_info;
+    int64_t* layout_range;
+    int32_t* packed_count;
+    int32_t* stats;
+    uint32_t* tokens_per_expert;
+    int32_t* record_packed_row;
+};
+
+constexpr int kOrderedDepth = 4;  // 16-byte loads in flight per lane
+
+template <int kPer>
+__device__ __forceinline__ void ordered_recv_impl(const OrderedRecvArgs& a, int block, int num_copy_blocks,
+                                                  int32_t* lds, int32_t* wave_totals) {
+    const int tid = threadIdx.x, lane = lane_id(), w = wave_in_block();
+    const int threads = blockDim.x, waves = threads >> 6;
+    const int num_ranks = a.num_ranks, max_tokens = a.max_tokens, num_local = a.num_local_experts;
+    const int num_segments = num_local * num_ranks;
+    int32_t* sent = lds;                       // [S]
+    int32_t* first = sent + num_segments + 1;  // [S]
+    int32_t* kept = first + num_segments + 1;  // [S + 1] (scanned in place by the last workgroup)
+    int32_t* place = kept + num_segments + 1;  // [S + 1] (last workgroup only)
+
+    // sent / first / kept of every pair, pairs in (expert, source) order: one global load per pair,
+    // the sums over the lower experts from LDS
+    for (int seg = tid; seg < num_segments; seg += threads) {
+        const int le = seg / num_ranks, src = seg - le * num_ranks;
+        const int c = a.all_num_routed[int64_t(src) * a.num_experts + a.rank * num_local + le];
+        sent[seg] = c < 0 ? 0 : (c > max_tokens ? max_tokens : c);
+    }
+    lds_barrier();
+    for (int seg = tid; seg < num_segments; seg += threads) {
+        const int le = seg / num_ranks, src = seg - le * num_ranks;
+        int before = 0;
+        for (int e2 = 0; e2 < le; ++e2) before += sent[e2 * num_ranks + src];
+        const int64_t room = a.slot_rows - before;
+        const int mine = sent[seg];
+        first[seg] = before;
+        kept[seg] = room <= 0 ? 0 : (mine < room ? mine : int(room));
+    }
+    lds_barrier();
+
+    const int64_t slots_per_expert = int64_t(max_tokens) * num_ranks;
+    if (block == num_copy_blocks) {  // the metadata workgroup
+        for (int seg = tid; seg < num_segments; seg += threads) place[seg] = kept[seg];
+        lds_barrier();
+        block_exclusive_scan(place, num_segments, wave_totals);
+        for (int seg = tid; seg < num_segments; seg += threads) {
+            const int le = seg / num_ranks;
+            const int64_t begin = place[seg] - place[le * num_ranks];
+            a.layout_range[seg] = kept[seg] > 0 ? ((begin << 32) | int64_t(kept[seg])) : 0;
+        }
+        for (int le = tid; le < num_local; le += threads) {
+            const int n = place[(le + 1) * num_ranks] - place[le * num_ranks];
+            a.packed_count[le] = n;
+            if (a.stats != nullptr) a.stats[le] += n;
+            if (a.tokens_per_expert != nullptr) a.tokens_per_expert[le] = uint32_t(n);
+        }
+        return;
+    }
+
+    WaveSegments<kPer> seg_table;
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+        const int seg = lane * kPer + u;
+        seg_table.cnt[u] = seg < num_segments ? kept[seg] : 0;
+        seg_table.aux[u] = seg < num_segments ? first[seg] : 0;
+    }
+    wave_segments_finish(seg_table);
+
+    const int64_t data_bytes = row_data_bytes(a.hidden, a.fmt);
+    const int64_t data_pad = align16(data_bytes);
+    const int64_t scale_bytes = row_scale_bytes(a.hidden, a.fmt);
+    const int64_t stride = row_stride_bytes(a.hidden, a.fmt);
+    const int num_vec = int(data_bytes / 16);
+    const int parts = 1 << a.parts_log2;
+    const int num_items = seg_table.total << a.parts_log2;
+    const int waves_total = num_copy_blocks * waves;
+    const int scale_dwords = int(scale_bytes / 4);
+    const bool has_scales = a.packed_scales != nullptr && scale_dwords > 0;
+
+    for (int item = block * waves + w; item < num_items; item += waves_total) {
+        const int row = item >> a.parts_log2, part = item & (parts - 1);
+        int seg_first, in_message;
+        const int seg = wave_segments_find(seg_table, row, seg_first, in_message);
+        const int le = seg / num_ranks, src = seg - le * num_ranks;
+        const int j = row - seg_first;
+        const uint8_t* from = a.rows + (int64_t(src) * a.slot_rows + in_message + j) * stride;
+        const int64_t out_row = int64_t(le) * slots_per_expert + (row - wave_segments_prefix(seg_table, le * num_ranks));
+        uint8_t* to = a.packed_x + out_row * data_bytes;
+        int v_begin, v_end;
+        row_part_range(num_vec, parts, part, v_begin, v_end);
+        const bool carries_tail = part == parts - 1;  // the last part is the shortest
+        u32x4 r[kOrderedDepth];
+#pragma unroll
+        for (int u = 0; u < kOrderedDepth; ++u) {
+            const int v = v_begin + u * kWave + lane;
+            if (v < v_end) r[u] = load_u32x4<false>(from + int64_t(v) * 16);
+        }
+        uint32_t tail_scale = 0;
+        int32_t tail_info = 0;
+        if (carries_tail) {  // scales and source index travel with the payload: one round trip per row
+            if (has_scales && lane < scale_dwords) tail_scale = reinterpret_cast<const uint32_t*>(from + data_pad)[lane];
+            if (lane == 0) tail_info = *reinterpret_cast<const int32_t*>(from + data_pad + align16(scale_bytes));
+        }
+#pragma unroll
+        for (int u = 0; u < kOrderedDepth; ++u) {
+            const int v = v_begin + u * kWave + lane;
+            if (v < v_end) store_u32x4<false>(to + int64_t(v) * 16, r[u]);
+        }
+        wave_copy_vec16<kOrderedDepth, false>(from, to, v_begin + kOrderedDepth * kWave, v_end, lane);
+        if (!carries_tail) continue;
+        if (has_scales) {
+            const uint32_t* s32 = reinterpret_cast<const uint32_t*>(from + data_pad);
+            uint32_t* d32 = reinterpret_cast<uint32_t*>(a.packed_scales + out_row * scale_bytes);
+            if (lane < scale_dwords) d32[lane] = tail_scale;
+            for (int v = kWave + lane; v < scale_dwords; v += kWave) d32[v] = s32[v];
+        }
+        if (lane == 0) a.src_info[out_row] = tail_info;
+    }
+
+    // The records' packed rows, a pair per wave (the first E_l * R waves of the grid, after their copies).
+    // Record of row j of pair (e, s): the records of the lower sources (their whole messages, kept or
+    // not), then the source's rows for the lower experts, then j.
+    if (a.record_packed_row == nullptr) return;
+    for (int seg = block * waves + w; seg < num_segments; seg += waves_total) {
+        const int le = seg / num_ranks, src = seg - le * num_ranks;
+        int lower = 0;  // rows the lower sources sent, all experts
+        for (int q = lane; q < num_local * src; q += kWave) lower += sent[(q / src) * num_ranks + q % src];
+        const int64_t record0 = int64_t(wave_sum(lower)) + first[seg];
+        const int64_t packed0 = int64_t(le) * slots_per_expert +
+                                (wave_segments_prefix(seg_table, seg) - wave_segments_prefix(seg_table, le * num_ranks));
+        const int n_sent = sent[seg], n_kept = kept[seg];
+        for (int j = lane; j < n_sent; j += kWave)
+            if (record0 + j < a.row_capacity) a.record_packed_row[record0 + j] = j < n_kept ? int32_t(packed0 + j) : -1;
+    }
+}
+
+__global__ __launch_bounds__(256) void ll_recv_ordered_kernel(OrderedRecvArgs a) {
+    extern __shared__ int32_t ordered_lds[];
+    __shared__ int32_t wave_totals[kMaxBlockWaves];
+    if (a.num_local_experts * a.num_ranks <= 4 * kWave)
+        ordered_recv_impl<4>(a, blockIdx.x, int(gridDim.x) - 1, ordered_lds, wave_totals);
+    else
+        ordered_recv_impl<16>(a, blockIdx.x, int(gridDim.x) - 1, ordered_lds, wave_totals);
+}
+
 }  // namespace deepep
 
 using namespace deepep;
@@ -503,6 +667,30 @@ int deepep_ll_dispatch_recv_by_source_ordered(const void* recv_by_source, int64_
     EP_HOST_ASSERT(workspace_bytes >= size_t(by_source_head_bytes() + most_rows * int64_t(sizeof(RowDesc))));
     const int num_local_experts = num_experts / num_ranks;
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+    const int64_t expected = expected_rows > 0 ? expected_rows : most_rows;
+    if (expected <= kLargeBatchRows) {  // one launch: every workgroup indexes for itself
+        OrderedRecvArgs oa;
+        oa.rows = reinterpret_cast<const uint8_t*>(recv_by_source);
+        oa.all_num_routed = all_num_routed;
+        oa.num_experts = num_experts, oa.num_local_experts = num_local_experts, oa.num_ranks = num_ranks;
+        oa.rank = rank, oa.max_tokens = num_max_dispatch_tokens_per_rank;
+        oa.hidden = hidden, oa.fmt = row_format;
+        oa.parts_log2 = choose_row_parts_log2(expected, row_data_bytes(hidden, row_format));
+        oa.slot_rows = slot_rows, oa.row_capacity = row_capacity;
+        oa.packed_x = reinterpret_cast<uint8_t*>(packed_recv_x);
+        oa.packed_scales = row_format == kRowBF16 ? nullptr : reinterpret_cast<uint8_t*>(packed_recv_scales);
+        oa.src_info = packed_recv_src_info, oa.layout_range = packed_recv_layout_range;
+        oa.packed_count = packed_recv_count, oa.stats = cumulative_local_expert_recv_stats;
+        oa.tokens_per_expert = tokens_per_expert, oa.record_packed_row = record_packed_row;
+        int64_t rows = expected + expected / 8 + 16;
+        if (rows > most_rows) rows = most_rows;
+        int64_t blocks = ((rows << oa.parts_log2) + 3) / 4;
+        blocks = blocks < 1 ? 1 : (blocks > 1024 ? 1024 : blocks);
+        const size_t lds = size_t(4 * (num_experts + 1)) * sizeof(int32_t);
+        ll_recv_ordered_kernel<<<dim3(unsigned(blocks) + 1), 256, lds, hs>>>(oa);  // + the metadata workgroup
+        EP_LAUNCH_CHECK();
+        return 0;
+    }
     int32_t* flat_total = reinterpret_cast<int32_t*>(workspace);
     RowDesc* desc = reinterpret_cast<RowDesc*>(reinterpret_cast<uint8_t*>(workspace) + by_source_head_bytes());
     ll_by_source_ordered_index_kernel<<<num_experts, kIndexThreads, 0, hs>>>(

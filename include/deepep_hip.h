@@ -396,14 +396,15 @@ int deepep_ll_dispatch_recv_by_source(const void* recv_by_source, int64_t slot_r
  * what deepep_ll_dispatch_send_by_dest emits, and its message starts at row s * slot_rows.  With the
  * gathered route counts every row's place then follows by arithmetic -- row j of source s belongs to
  * the expert whose run of that source's column of the counts holds j -- so nothing is read from the
- * rows to index them and no record list is needed: one index launch and the row copy, both sides of
- * every (expert, source) pair contiguous.  Outputs as deepep_ll_dispatch_recv_by_source.
+ * rows to index them and no record list is needed: one launch for up to 8192 expected rows, one index
+ * launch and the row copy beyond, both sides of every (expert, source) pair contiguous.  Outputs as
+ * deepep_ll_dispatch_recv_by_source.
  *   all_num_routed     [R, E] int32, as for deepep_ll_exchange_metadata (counts above M read as M)
  *   record_packed_row  [row_capacity] int32 (out) or NULL, indexed like the records of
  *                      deepep_ll_exchange_metadata: sources ascending, a source's rows in message order
  *   expected_rows      as for deepep_ll_dispatch_recv_by_source
  *   workspace          256 + 8 * min(R * slot_rows, E * M) bytes (deepep_ll_by_source_workspace_bytes(E,
- *                      R * slot_rows) is enough)
+ *                      R * slot_rows) is enough); only read and written past 8192 expected rows
  * Rows of a message beyond the source's slot are lost (their records read -1).
  * Replaces ll_recv_unpack_v2 (csrc/kernels/efa_kernels.cu:2121-2231; ranges :991-1010) for this
  * build's own wire order; the reference cannot take this shortcut because its senders leave the

@@ -1055,6 +1055,8 @@ def check_send_by_dest(st, want, t):
     (1, 0, 16, 512, 2, 4),       # a world of one rank
     (4, 2, 24, 1536, 4, 16),     # hidden not a multiple of 1024
     (512, 500, 3, 512, 2, 1024),
+    (4, 3, 256, 512, 8, 32),     # 2048 entries: the last batch whose tables are built inside the send launch
+    (4, 3, 257, 512, 8, 32),     # 2056 entries: the first with a launch for them
 ])
 def test_send_by_dest(rt, fmt, r, rank, t, h, k, e):
     """One buffer, contiguous per destination rank, rows by expert and slot; counts, prefixes and every
@@ -1093,7 +1095,7 @@ def all_to_all_dispatch(states, fmt):
     return routed
 
 
-@pytest.mark.parametrize("receive", ["from_tails", "ordered"])
+@pytest.mark.parametrize("receive", ["from_tails", "ordered", "ordered_as_a_large_batch"])
 @pytest.mark.parametrize("delivery", ["flat", "slotted", "direct"])
 @pytest.mark.parametrize("fmt", [O.ROW_FP8, O.ROW_BF16])
 @pytest.mark.parametrize("r,t,h,k,e", [(4, 40, 512, 3, 16), (8, 700, 512, 8, 64), (3, 5, 256, 2, 3)],
@@ -1119,7 +1121,9 @@ def test_all_to_all_round_trip_on_one_gpu(rt, oracle_c, fmt, delivery, receive, 
         poison_outputs_keep_pair_slot(st)
         st.record_packed_row.fill_(-7)
         st.tokens_per_expert.fill_(-7)
-        if receive == "ordered":  # the messages are in this build's own order: placed from the counts alone
+        if receive.startswith("ordered"):  # the messages are in this build's own order: placed from the counts alone
+            if receive == "ordered_as_a_large_batch":  # the index launch + flat row copy instead of the single launch
+                st.expected_rows = 9000
             st.dispatch_recv_ordered(routed)
         else:
             st.dispatch_recv()
@@ -1334,9 +1338,10 @@ def test_ordered_receive_with_slots_too_small_and_counts_too_large(rt):
         dst.recv_by_source[s_ * slot_rows:s_ * slot_rows + n] = src.send_rows[lo:lo + n]
     routed_big = routed.clone()
     routed_big[0, 1] += 1000  # nonsense from source 0 for expert 1: read as M rows
-    for mat in (routed, routed_big):
+    for mat, hint in ((routed, t * k), (routed_big, t * k), (routed, 9000), (routed_big, 9000)):
         poison_outputs_keep_pair_slot(dst)
         dst.record_packed_row.fill_(-7)
+        dst.expected_rows = hint  # the single launch, then the index launch + flat row copy
         dst.dispatch_recv_ordered(mat)
         torch.cuda.synchronize()
         sent = mat[:, rank * epr:(rank + 1) * epr].cpu().clamp(max=t)  # [source, local expert]
