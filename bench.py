@@ -102,13 +102,14 @@ def time_calls(torch, fn, n):
 
 def time_graph_samples(torch, fn, warmup, steps, samples=10):
     """`fn` enqueued by HIP-graph replays so that the GPU never waits for the host: the time is the stream's,
-    kernels plus the gaps between them.  The graph holds a whole multiple of `steps` calls, at least 20 (a
-    graph of one 16 us step would mostly measure the events around it); a sample is as many back-to-back
-    replays as make about 100 calls, between its own pair of events; `samples` of them are taken whatever
+    kernels plus the gaps between them.  The graph holds a whole multiple of `steps` calls, at least 100 (what
+    a replay costs by itself, a few microseconds, is then under a tenth of a microsecond per call whatever
+    `steps` is: with graphs of 20 steps the 128-token step read 16.2 us, with graphs of 200 steps 15.8) and at
+    most 1000; a sample is one replay between its own pair of events, and `samples` of them are taken whatever
     `steps` is.  Returns the median per call with the fastest and slowest sample beside it, so the figure does
     not depend on how many steps were asked for."""
-    per_graph = steps * max(1, -(-20 // steps))
-    replays = max(1, 100 // per_graph)
+    per_graph = min(1000, steps * max(1, -(-100 // steps)))
+    replays = 1
     g = torch.cuda.CUDAGraph()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
