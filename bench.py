@@ -100,6 +100,14 @@ def time_calls(torch, fn, n):
     return e0.elapsed_time(e1) * 1e3 / n
 
 
+def time_calls_median(torch, fn, n=10, samples=5):
+    """The large entries (tens to hundreds of microseconds a call): `samples` runs of `n` eager calls, each run
+    between its own pair of events; the median run with the fastest and slowest beside it.  Independent of
+    --steps."""
+    runs = sorted(time_calls(torch, fn, n) for _ in range(samples))
+    return runs[len(runs) // 2], [round(runs[0], 2), round(runs[-1], 2)]
+
+
 def time_graph_samples(torch, fn, warmup, steps, samples=10):
     """`fn` enqueued by HIP-graph replays so that the GPU never waits for the host: the time is the stream's,
     kernels plus the gaps between them.  The graph holds a whole multiple of `steps` calls, at least 100 (what
@@ -439,7 +447,6 @@ def bench_pack(torch, _capi, lib, loopback, args):
     reduce = rotating([reduce_on(i) for i in range(2)])
     reduce_from_list = rotating([reduce_from_list_on(i) for i in range(2)])
 
-    n = max(10, args.steps // 4)
     res = {"workload": "4096 tokens x 7168 bf16, top-8 of 256 experts, 8 ranks x 32 experts", "rows_packed": s,
            "buffers": "cast, packs and reduce rotate over 7 / 2 / 2 sets of buffers, so no call finds its bytes in "
                       "the memory-side cache"}
@@ -454,9 +461,9 @@ def bench_pack(torch, _capi, lib, loopback, args):
                              ("combine_reduce", reduce, s * 2 * h + s * k * 4 + t * r * 5 + t * 2 * h + t * k * 4),
                              ("combine_reduce_from_the_list", reduce_from_list,
                               s * 2 * h + s * k * 4 + s * 12 + t * r + t * 2 * h + t * k * 4)):
-        us = time_calls(torch, fn, n)
+        us, spread = time_calls_median(torch, fn)
         res[name] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
-                     "frac_of_8TBps": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+                     "frac_of_8TBps": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "us_min_max": spread}
     # The packs read every source row once per destination rank that wants it (s / t times on average).  The
     # figure above counts each of those reads; if the caches served all but the first, HBM would see only the
     # unique bytes: every source row once, every packed row once.  The counters say the L2 does not serve them
@@ -549,14 +556,13 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
         if skewed:  # millisecond kernels: every call between its own events, so the spread shows
             samples = sorted(time_calls(torch, fn, 1) for _ in range(6))
             us = samples[len(samples) // 2]
+            spread = [round(samples[0], 2), round(samples[-1], 2)]
         else:
-            us = time_calls(torch, fn, max(10, args.steps // 10))
+            us, spread = time_calls_median(torch, fn)
         res[name] = {"us": round(us, 2), "bytes": nbytes[name], "GBps": round(nbytes[name] / us / 1e3, 1),
-                     "frac_of_8TBps": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBS, 4)}
-        if skewed:
-            res[name]["us_min_max"] = [round(samples[0], 2), round(samples[-1], 2)]
+                     "frac_of_8TBps": round(nbytes[name] / us / 1e3 / HBM_PEAK_GBS, 4), "us_min_max": spread}
     if not skewed:  # what the same send measures when every call goes to the same buffers
-        us = time_calls(torch, lambda: st.dispatch_send(x, topk), max(10, args.steps // 10))
+        us, _ = time_calls_median(torch, lambda: st.dispatch_send(x, topk))
         res["dispatch_send"]["us_on_one_set_of_buffers"] = round(us, 2)
     # The send's memory traffic without the send: a bare kernel that reads every token row and stores one
     # byte per element to the rows the send writes (remote experts' slots; the rows for this rank's own
@@ -579,7 +585,7 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
         samples = sorted(time_calls(torch, probe, 1) for _ in range(6))
         us = samples[len(samples) // 2]
     else:
-        us = time_calls(torch, probe, max(10, args.steps // 10))
+        us, _ = time_calls_median(torch, probe)
     probe_bytes = t * 2 * h + p * h
     res["bare_row_scatter"] = {"us": round(us, 2), "bytes": probe_bytes, "GBps": round(probe_bytes / us / 1e3, 1),
                                "frac_of_8TBps": round(probe_bytes / us / 1e3 / HBM_PEAK_GBS, 4),
@@ -603,7 +609,7 @@ def bench_ll_large(torch, _capi, lib, ll_runtime, loopback, args, skewed=False):
         samples = sorted(time_calls(torch, plain, 1) for _ in range(6))
         us = samples[len(samples) // 2]
     else:
-        us = time_calls(torch, plain, max(10, args.steps // 10))
+        us, _ = time_calls_median(torch, plain)
     res["plain_stream_copy"] = {"us": round(us, 2), "bytes": 2 * half, "GBps": round(2 * half / us / 1e3, 1),
                                 "frac_of_8TBps": round(2 * half / us / 1e3 / HBM_PEAK_GBS, 4),
                                 "what": "one contiguous copy of the bytes the receive copy moves"}
