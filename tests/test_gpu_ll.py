@@ -1117,6 +1117,26 @@ def test_all_to_all_round_trip_at_the_headline_shape(rt, oracle_c, delivery, rec
     run_all_to_all_round_trip(rt, oracle_c, O.ROW_FP8, delivery, receive, 32, 128, 7168, 8, 256, check_ranks=(0, 5, 31))
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_all_to_all_round_trip_random_worlds(rt, oracle_c, seed):
+    """Seeded random small worlds through the same flow: odd rank counts, one to five experts a rank, one token
+    to a few hundred (both sides of the 2048 entries up to which the send builds its own tables), every format,
+    receive and delivery."""
+    rng = np.random.default_rng(1000 + seed)
+    r = int(rng.choice([1, 2, 3, 4, 6, 8, 16]))
+    epr = int(rng.choice([1, 2, 3, 5]))
+    e = r * epr
+    k = int(rng.integers(1, min(8, e) + 1))
+    t = int(rng.choice([1, 2, 7, 33, 64, 129, 260, 300]))
+    h = int(rng.choice([128, 256, 512, 1024, 1536, 2048]))
+    fmt = [O.ROW_FP8, O.ROW_BF16, O.ROW_FP8_POW2, O.ROW_FP8_UE8M0][int(rng.integers(4))]
+    if fmt == O.ROW_FP8_UE8M0 and (h // 128) % 4:
+        h = 512  # packed UE8M0 scales come four to a word
+    delivery = ["flat", "slotted", "direct"][int(rng.integers(3))]
+    receive = ["from_tails", "ordered", "ordered_as_a_large_batch"][int(rng.integers(3))]
+    run_all_to_all_round_trip(rt, oracle_c, fmt, delivery, receive, r, t, h, k, e)
+
+
 def test_all_to_all_round_trip_with_large_batches(rt, oracle_c):
     """4096 tokens a rank, 8 ranks x 32 experts, hidden 2048 (every rank on the one GPU needs ~9 GB then): the
     send runs on chunk histograms with the prefix launch, the receive on the ordered index and the flat row copy,
