@@ -63,6 +63,9 @@ def algorithmic_bytes(t, h, k, p, rv, stride, e, r, own=0, packed=None):
         "all_to_all_step": (t * 2 * h + t * k * 8 * 2 + p * stride + t * k * 4 + e * 8) + (r * e * 4 + rv * 16 + r * 24)
                            + (rv * stride + rv * packed + small + r * e * 4 + rv * 8) + (rv * 2 * h * 2 + rv * 16)
                            + (p * 2 * h + t * k * 16 + e * 4 + t * 2 * h),
+        "all_to_all_step_without_metadata_launch": (t * 2 * h + t * k * 8 * 2 + p * stride + t * k * 4 + e * 8)
+                           + (rv * stride + rv * packed + small + r * e * 4 + rv * 8) + (rv * 2 * h * 2 + rv * 16)
+                           + (p * 2 * h + t * k * 16 + e * 4 + t * 2 * h),
     }
 
 
@@ -337,8 +340,18 @@ def all_to_all_entries(torch, _capi, lib, ll_runtime, st, world, x, topk, weight
         a2a.combine_send(y)
         a2a.combine_recv(topk, weights, out)
 
+    def critical_path():
+        # The ordered receive does not read the exchange metadata (the return by destination does): on a
+        # real transport that launch goes to a side stream while the rows are on the wire, and what is
+        # left in stream order between the inputs and the combined rows are these four.
+        a2a.dispatch_send(x, topk)
+        a2a.dispatch_recv_ordered(routed)
+        a2a.combine_send(y)
+        a2a.combine_recv(topk, weights, out)
+
     return {
         "all_to_all_step": whole_step,
+        "all_to_all_step_without_metadata_launch": critical_path,
         "dispatch_send_by_dest": lambda: a2a.dispatch_send(x, topk),
         "dispatch_recv_by_source": lambda: a2a.dispatch_recv(),
         "dispatch_recv_by_source_ordered": lambda: a2a.dispatch_recv_ordered(routed),

@@ -1066,6 +1066,37 @@ def test_send_by_dest(rt, fmt, r, rank, t, h, k, e):
     check_send_by_dest(st, O.ll_send_by_dest(x_all[rank], topk_all[rank], rank, e, t, fmt, r), t)
 
 
+@pytest.mark.parametrize("receive", ["from_tails", "ordered"])
+def test_all_to_all_with_an_empty_batch(rt, receive):
+    """No token anywhere: the tables are zeros, nothing is received, the records stay untouched, and the reduce of
+    no tokens is a no-op."""
+    r, rank, m, h, k, e = 4, 2, 8, 512, 2, 8
+    x = torch.empty((0, h), dtype=torch.bfloat16)
+    topk = torch.empty((0, k), dtype=torch.int64)
+    st = send_by_dest_on_gpu(rt, x, topk, rank, r, e, m, O.ROW_FP8)
+    assert (st.send_count == 0).all() and (st.send_expert_prefix == 0).all()
+    assert (st.send_counts == 0).all() and (st.send_cumsum == 0).all()
+    assert (st.send_rows == 0xEE).all()
+    routed = torch.zeros((r, e), dtype=torch.int32, device="cuda")
+    st.exchange_metadata(routed)
+    poison_outputs_keep_pair_slot(st)
+    st.record_packed_row.fill_(-7)
+    if receive == "ordered":
+        st.dispatch_recv_ordered(routed)
+    else:
+        st.dispatch_recv()
+    torch.cuda.synchronize()
+    assert (st.packed_recv_count == 0).all() and (st.packed_recv_layout_range == 0).all()
+    assert (st.tokens_per_expert == 0).all() and (st.record_packed_row == -7).all()
+    y = torch.zeros((e // r, r * m, h), dtype=torch.bfloat16, device="cuda")
+    st.send_flat.view(torch.int16).fill_(0x7FC0)
+    st.combine_send(y)
+    out = torch.empty((0, h), dtype=torch.bfloat16, device="cuda")
+    st.combine_recv(topk.cuda(), torch.empty((0, k), dtype=torch.float32, device="cuda"), out)
+    torch.cuda.synchronize()
+    assert (st.send_flat.view(torch.int16) == 0x7FC0).all()
+
+
 def test_send_by_dest_with_repeated_experts_and_full_pairs(rt):
     """Tokens naming an expert more than once: pairs beyond a pair's M slots are dropped from the counts,
     the prefixes and the buffer alike."""
