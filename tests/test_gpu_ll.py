@@ -1168,6 +1168,74 @@ def test_all_to_all_round_trip_random_worlds(rt, oracle_c, seed):
     run_all_to_all_round_trip(rt, oracle_c, fmt, delivery, receive, r, t, h, k, e)
 
 
+@pytest.mark.parametrize("t", [48, 1100], ids=["decode_size", "large_batch"])
+def test_all_to_all_step_replays_in_a_hip_graph(rt, t):
+    """A rank's five calls over the all-to-all surface captured once and replayed: they must allocate nothing
+    and record no memset, and every replay, with eager work and synchronisations in between, must leave what the
+    eager calls left (the peers' messages and answers stay where the eager exchange put them)."""
+    r, rank, h, k, e, fmt = 4, 1, 1024, 8, 32, O.ROW_FP8
+    epr = e // r
+    x_all, topk_all, w_all = make_world(r, t, h, k, e, seed=77, drop=5)
+    states = []
+    for s_ in range(r):
+        st = rt.ll.AllToAllState(rt.ll.LLShape(r, s_, e, t, h, k, fmt))
+        st.dispatch_send(x_all[s_].cuda(), topk_all[s_].cuda())
+        states.append(st)
+    torch.cuda.synchronize()
+    routed = all_to_all_dispatch(states, fmt)  # also runs every rank's exchange_metadata
+    me = states[rank]
+    x, topk, w = x_all[rank].cuda(), topk_all[rank].cuda(), w_all[rank].cuda()
+    y = torch.empty((epr, r * t, h), dtype=torch.bfloat16, device="cuda")
+    rt.capi.check(rt.capi.load().deepep_synth_bf16_rows(rt.capi.ptr(y), epr * r * t, h, h * 2, None, 0, 31, 0,
+                                                        torch.cuda.current_stream().cuda_stream))
+    me.recv_flat.normal_()  # the peers' answers
+    out = torch.empty((t, h), dtype=torch.bfloat16, device="cuda")
+    meta = me.meta
+    lib, capi = rt.capi.load(), rt.capi
+    meta_args = [capi.ptr(routed), e, r, rank, me.slot_rows, me.row_capacity] + [capi.ptr(meta[n]) for n in (
+        "send_counts", "recv_counts", "totals", "combine_remote_recv_offset", "source_rank", "source_offset",
+        "padded_index", "combine_send_offset", "num_recv_tokens", "tokens_per_expert")]
+
+    def step():
+        me.dispatch_send(x, topk)
+        capi.check(lib.deepep_ll_exchange_metadata(*meta_args, torch.cuda.current_stream().cuda_stream))
+        me.dispatch_recv_ordered(routed)
+        me.combine_send(y)
+        me.combine_recv(topk, w, out)
+
+    n_records = int(meta["num_recv_tokens"][1])  # the records past them are nobody's to write
+    outputs = lambda: (me.send_rows, me.send_expert_prefix, me.send_cumsum, me.pair_slot, me.packed_recv_count,
+                       me.packed_recv_layout_range, me.record_packed_row[:n_records], me.send_flat.view(torch.int16),
+                       out.view(torch.int16))
+    me.send_rows.fill_(0xEE)
+    me.send_flat.view(torch.int16).fill_(0x7FC0)
+    step()
+    torch.cuda.synchronize()
+    want = [v.clone() for v in outputs()]
+    n_rows = int(me.packed_recv_count.sum())
+    assert n_rows > (8192 if t > 1024 else 0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    for replay in range(4):
+        me.send_rows.fill_(0xEE)  # eager work between the replays: scribble over what the step writes
+        me.send_flat.view(torch.int16).fill_(0x7FC0)
+        out.zero_()
+        me.packed_recv_count.fill_(-1)
+        me.record_packed_row.fill_(-7)
+        me.pair_slot.fill_(-9)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for i, (got, exp) in enumerate(zip(outputs(), want)):
+            assert torch.equal(got, exp), f"replay {replay}: output {i}"
+
+
 def test_all_to_all_round_trip_with_large_batches(rt, oracle_c):
     """4096 tokens a rank, 8 ranks x 32 experts, hidden 2048 (every rank on the one GPU needs ~9 GB then): the
     send runs on chunk histograms with the prefix launch, the receive on the ordered index and the flat row copy,
